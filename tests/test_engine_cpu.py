@@ -1,0 +1,52 @@
+"""Host side of the engine (batching, cache manager, step function) on a CPU, with the kernels'
+plain PyTorch references standing in for the kernels, against the plain whole-sequence model."""
+import pytest
+import torch
+
+from helpers import CONFIGS, PAGE_SIZE, Harness, make_folder, random_tokens
+from plain_qwen2 import qwen2_logits, read_model_folder
+from torch_ops import TorchOps
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole_then_decode_matches_plain(tmp_path, name):
+    folder = make_folder(tmp_path, name)
+    config, weights = read_model_folder(folder)
+    tokens = random_tokens(config["vocab_size"], 45, seed=7)
+    expected = qwen2_logits(config, weights, tokens)
+    h = Harness(folder, TorchOps(), torch.float32, "cpu", PAGE_SIZE[name], num_pages=32)
+    split = 30
+    got = [h.feed([("a", tokens[:split], list(range(split)))])]
+    for i in range(split, len(tokens)):
+        got.append(h.feed([("a", [tokens[i]], [0])]))
+    got = torch.cat(got)
+    torch.testing.assert_close(got, expected, rtol=1e-4, atol=1e-5)
+    h.feed([], end=["a"]) if False else h.cache.free_sequence(h.live.pop("a")[0])
+    h.cache.assert_consistent([])
+
+
+def test_mixed_batch_with_page_reuse(tmp_path):
+    name = "B"
+    folder = make_folder(tmp_path, name)
+    config, weights = read_model_folder(folder)
+    prompts = {rid: random_tokens(config["vocab_size"], n, seed=i) for i, (rid, n) in enumerate([("a", 23), ("b", 17), ("c", 9), ("d", 31)])}
+    expected = {rid: qwen2_logits(config, weights, toks) for rid, toks in prompts.items()}
+    h = Harness(folder, TorchOps(), torch.float32, "cpu", PAGE_SIZE[name], num_pages=9)  # 8 usable pages of 8
+    got = {rid: [] for rid in prompts}
+    # a and b start; a finishes, its pages go to c; then d takes what b and c give back
+    def run(batch, end=()):
+        out = h.feed([(rid, prompts[rid][lo:hi], list(range(hi - lo))) for rid, lo, hi in batch], end=end)
+        row = 0
+        for rid, lo, hi in batch:
+            got[rid].append(out[row:row + hi - lo])
+            row += hi - lo
+    run([("a", 0, 7), ("b", 0, 2)])
+    run([("a", 7, 8), ("b", 2, 11)])
+    run([("a", 8, 23), ("b", 11, 12)], end=["a"])
+    run([("b", 12, 13), ("c", 0, 9)], end=["c"])
+    run([("b", 13, 17), ("d", 0, 5)], end=["b"])
+    run([("d", 5, 31)], end=["d"])
+    for rid in prompts:
+        torch.testing.assert_close(torch.cat(got[rid]), expected[rid], rtol=1e-4, atol=1e-5)
+    h.cache.assert_consistent([])
+    assert h.cache.num_used_pages() == 0

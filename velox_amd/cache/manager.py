@@ -1,0 +1,305 @@
+"""The cache manager: page pools per group of layers, block tables per request, state slots.
+
+Every schedule entry of a model states what its mixer needs (``PagedNeed``, ``StateNeed``
+or nothing).  Entries with equal paged needs form a *group*: one pool of pages, one
+allocator, one block table per request; page ``p`` of a group addresses page ``p`` of
+every entry in it (the reference has exactly one such group for all layers,
+``src/paged_kv_cache.py:51-55``).  A group whose need has a window gives pages back as soon
+as every key in them lies behind the window of all queries still to come.  Entries with
+a ``StateNeed`` get one row per request in fixed-size tensors, indexed by the request's
+*slot* (the reference's ``seq_index``, ``engine/scheduler.py:58,113-129``); slot rows are zeroed
+when a request takes the slot.
+
+Page layout, per entry of a group: keys ``[pages, kv_heads, page_size, head_dim]``, values
+``[pages, kv_heads, head_dim, page_size]`` (values are stored transposed inside a page so
+that the attention kernels read a run of consecutive keys for one channel in one
+contiguous access).
+
+Growth rule per group (reference ``src/block_manager.py:74-99``): a request that has
+``num_computed`` tokens in the cache and is given ``n`` more needs
+``ceil((num_computed + n) / page_size)`` table entries.  All groups grow together or
+not at all.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..parts.base import PagedNeed, StateNeed
+from .allocator import NULL_PAGE, OutOfPagesError, PageAllocator
+
+
+@dataclass
+class SequenceCache:
+    """What one live request holds: a block table per group and (always) a slot."""
+
+    slot: int
+    tables: List[List[int]]
+    released: List[int]  # per group: number of leading table entries already given back
+
+
+class PageGroup:
+    def __init__(self, need: PagedNeed, entries: List[int], num_pages: int, page_size: int, dtype: torch.dtype, device, allocate_tensors: bool) -> None:
+        self.need = need
+        self.entries = list(entries)
+        self.page_size = int(page_size)
+        self.allocator = PageAllocator(num_pages)
+        self.dtype = dtype
+        self.keys: Optional[torch.Tensor] = None
+        self.values: Optional[torch.Tensor] = None
+        if allocate_tensors:
+            n, h, d = len(entries), need.num_kv_heads, need.head_dim
+            self.keys = torch.zeros((n, num_pages, h, page_size, d), dtype=dtype, device=device)
+            self.values = torch.zeros((n, num_pages, h, d, page_size), dtype=dtype, device=device)
+
+    def bytes_per_page(self) -> int:
+        element = torch.empty((), dtype=self.dtype).element_size()
+        return 2 * self.page_size * self.need.num_kv_heads * self.need.head_dim * element * len(self.entries)
+
+    def table_entries_for(self, num_tokens: int) -> int:
+        return (num_tokens + self.page_size - 1) // self.page_size
+
+    def first_needed_page(self, num_computed: int) -> int:
+        """Index of the first table entry a query at position >= num_computed may still read."""
+        if self.need.window is None:
+            return 0
+        first_key = max(0, num_computed - self.need.window + 1)
+        return first_key // self.page_size
+
+
+class StateSlots:
+    """Rows of fixed-size state, one per live request, plus one spare row for padded batch rows."""
+
+    def __init__(self, needs: Dict[int, StateNeed], max_num_seqs: int, dtype: torch.dtype, device, allocate_tensors: bool) -> None:
+        self.max_num_seqs = int(max_num_seqs)
+        self.pad_slot = self.max_num_seqs
+        self._free: List[int] = list(range(self.max_num_seqs - 1, -1, -1))
+        self._held = [False] * self.max_num_seqs
+        self.tensors: Dict[int, Dict[str, torch.Tensor]] = {}
+        if allocate_tensors:
+            for entry, need in needs.items():
+                self.tensors[entry] = {
+                    name: torch.zeros((self.max_num_seqs + 1, *shape), dtype=dt or dtype, device=device)
+                    for name, shape, dt in need.tensors
+                }
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def acquire(self) -> Optional[int]:
+        if not self._free:
+            return None
+        slot = self._free.pop()
+        self._held[slot] = True
+        for tensors in self.tensors.values():
+            for tensor in tensors.values():
+                tensor[slot].zero_()
+        return slot
+
+    def release(self, slot: int) -> None:
+        if not 0 <= slot < self.max_num_seqs or not self._held[slot]:
+            raise RuntimeError(f"slot {slot} is not held")
+        self._held[slot] = False
+        self._free.append(slot)
+
+    def assert_consistent(self) -> None:
+        if len(set(self._free)) != len(self._free):
+            raise AssertionError("slot free list contains duplicates")
+        for slot in range(self.max_num_seqs):
+            if self._held[slot] == (slot in self._free):
+                raise AssertionError(f"slot {slot}: held={self._held[slot]} but free={slot in self._free}")
+
+
+@dataclass
+class PagedView:
+    """What a mixer with a ``PagedNeed`` is handed for one schedule entry and one step."""
+
+    k: torch.Tensor
+    v: torch.Tensor
+    block_size: int
+    batch: object  # engine.batch.GroupBatch of this step
+
+
+@dataclass
+class StateView:
+    tensors: Dict[str, torch.Tensor]
+
+
+class CacheManager:
+    def __init__(
+        self,
+        needs: Sequence[object],
+        page_size: int,
+        num_pages: int,
+        max_num_seqs: int,
+        dtype: torch.dtype,
+        device="cpu",
+        max_model_len: Optional[int] = None,
+        allocate_tensors: bool = True,
+    ) -> None:
+        if page_size <= 0 or (page_size & (page_size - 1)) != 0:
+            raise ValueError(f"page_size must be a power of two, got {page_size}")
+        self.page_size = int(page_size)
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.groups: List[PageGroup] = []
+        self.entry_group: Dict[int, Tuple[int, int]] = {}
+        by_need: Dict[PagedNeed, List[int]] = {}
+        state_needs: Dict[int, StateNeed] = {}
+        for entry, need in enumerate(needs):
+            if isinstance(need, PagedNeed):
+                by_need.setdefault(need, []).append(entry)
+            elif isinstance(need, StateNeed):
+                state_needs[entry] = need
+            elif need is not None:
+                raise TypeError(f"schedule entry {entry}: unknown cache need {need!r}")
+        for need, entries in by_need.items():
+            index = len(self.groups)
+            self.groups.append(PageGroup(need, entries, num_pages, page_size, dtype, self.device, allocate_tensors))
+            for position, entry in enumerate(entries):
+                self.entry_group[entry] = (index, position)
+        self.state = StateSlots(state_needs, max_num_seqs, dtype, self.device, allocate_tensors)
+        self.state_entries = set(state_needs)
+        capacity = (num_pages - 1) * page_size
+        self.max_model_len = min(max_model_len, capacity) if max_model_len else capacity
+        self.max_pages_per_seq = (self.max_model_len + page_size - 1) // page_size
+
+    # -- sizes --------------------------------------------------------------------------
+    def bytes_per_page(self) -> int:
+        return sum(group.bytes_per_page() for group in self.groups)
+
+    @property
+    def num_total_pages(self) -> int:
+        return min((g.allocator.num_total for g in self.groups), default=0)
+
+    def num_free_pages(self) -> int:
+        """Free pages of the tightest group (what bounds growth)."""
+        return min((g.allocator.num_free for g in self.groups), default=1 << 30)
+
+    def num_used_pages(self) -> int:
+        return max((g.allocator.num_used for g in self.groups), default=0)
+
+    # -- sequences ----------------------------------------------------------------------
+    def new_sequence(self) -> Optional[SequenceCache]:
+        slot = self.state.acquire()
+        if slot is None:
+            return None
+        return SequenceCache(slot=slot, tables=[[] for _ in self.groups], released=[0 for _ in self.groups])
+
+    def pages_to_append(self, seq: SequenceCache, num_computed: int, num_new: int) -> List[int]:
+        return [
+            max(0, group.table_entries_for(num_computed + num_new) - len(table))
+            for group, table in zip(self.groups, seq.tables)
+        ]
+
+    def can_append(self, seq: SequenceCache, num_computed: int, num_new: int) -> bool:
+        if num_computed + num_new > self.max_model_len:
+            return False
+        extra = self.pages_to_append(seq, num_computed, num_new)
+        return all(n <= g.allocator.num_free for n, g in zip(extra, self.groups))
+
+    def max_new_tokens(self, seq: Optional[SequenceCache], num_computed: int, headroom_pages: Optional[int] = None) -> int:
+        """How many tokens past ``num_computed`` fit in the pages the request has plus the free ones
+        (less ``headroom_pages`` held back), capped by ``max_model_len`` (reference ``engine/scheduler.py:210-219``)."""
+        limit = self.max_model_len - num_computed
+        for index, group in enumerate(self.groups):
+            have = len(seq.tables[index]) if seq is not None else 0
+            free = group.allocator.num_free if headroom_pages is None else min(group.allocator.num_free, headroom_pages)
+            pages = min(have + max(0, free), self.max_pages_per_seq)
+            limit = min(limit, pages * group.page_size - num_computed)
+        return max(0, limit)
+
+    def append(self, seq: SequenceCache, num_computed: int, num_new: int) -> bool:
+        """Grows every group's table to cover ``num_computed + num_new`` tokens; all or nothing."""
+        if num_computed + num_new > self.max_model_len:
+            return False
+        extra = self.pages_to_append(seq, num_computed, num_new)
+        for n, group, table in zip(extra, self.groups, seq.tables):
+            if n > group.allocator.num_free or len(table) + n > self.max_pages_per_seq:
+                return False
+        for n, group, table in zip(extra, self.groups, seq.tables):
+            table.extend(group.allocator.allocate_many(n))
+        return True
+
+    def release_behind_window(self, seq: SequenceCache, num_computed: int) -> int:
+        """Gives back pages no later query can read; their table entries become the null page."""
+        given_back = 0
+        for index, group in enumerate(self.groups):
+            first = min(group.first_needed_page(num_computed), len(seq.tables[index]))
+            table = seq.tables[index]
+            for position in range(seq.released[index], first):
+                if table[position] != NULL_PAGE:
+                    group.allocator.free(table[position])
+                    table[position] = NULL_PAGE
+                    given_back += 1
+            seq.released[index] = max(seq.released[index], first)
+        return given_back
+
+    def free_pages(self, seq: SequenceCache) -> None:
+        for index, group in enumerate(self.groups):
+            for page in seq.tables[index]:
+                if page != NULL_PAGE:
+                    group.allocator.free(page)
+            seq.tables[index] = []
+            seq.released[index] = 0
+
+    def free_sequence(self, seq: SequenceCache) -> None:
+        self.free_pages(seq)
+        if seq.slot is not None and seq.slot >= 0:
+            self.state.release(seq.slot)
+            seq.slot = -1
+
+    def slot_for(self, seq: SequenceCache, group_index: int, token_index: int) -> int:
+        page = seq.tables[group_index][token_index // self.page_size]
+        return page * self.page_size + token_index % self.page_size
+
+    # -- views handed to the mixers ----------------------------------------------------------
+    def view(self, entry: int, group_batches: Sequence[object]):
+        if entry in self.entry_group:
+            g, position = self.entry_group[entry]
+            group = self.groups[g]
+            return PagedView(group.keys[position], group.values[position], group.page_size, group_batches[g])
+        if entry in self.state_entries:
+            return StateView(self.state.tensors[entry])
+        return None
+
+    def gather_sequence(self, entry: int, seq: SequenceCache, length: int):
+        """Contiguous keys and values ``[length, kv_heads, head_dim]`` of one request (a debugging aid,
+        reference ``src/paged_kv_cache.py:125-150``)."""
+        g, position = self.entry_group[entry]
+        group = self.groups[g]
+        index = torch.arange(length)
+        pages = torch.tensor(seq.tables[g], dtype=torch.long)[index // group.page_size].to(self.device)
+        offsets = (index % group.page_size).to(self.device)
+        keys = group.keys[position][pages, :, offsets, :]
+        values = group.values[position][pages, :, :, offsets]
+        return keys, values
+
+    # -- invariants ---------------------------------------------------------------------
+    def assert_consistent(self, live: Sequence[SequenceCache] = ()) -> None:
+        """Allocator invariants, and: the pages the live requests hold are exactly the used ones, each held once."""
+        self.state.assert_consistent()
+        for index, group in enumerate(self.groups):
+            group.allocator.assert_consistent()
+            held: List[int] = [p for seq in live for p in seq.tables[index] if p != NULL_PAGE]
+            if len(set(held)) != len(held):
+                raise AssertionError(f"group {index}: a page is held twice")
+            for page in held:
+                if group.allocator.ref_count(page) != 1:
+                    raise AssertionError(f"group {index}: held page {page} has refcount {group.allocator.ref_count(page)}")
+            if live is not None and len(held) != group.allocator.num_used:
+                raise AssertionError(f"group {index}: {group.allocator.num_used} pages used but {len(held)} held (a page was lost)")
+
+
+def pages_that_fit(bytes_per_page: int, free_bytes: int, utilization: float, reserve_bytes: int) -> int:
+    """Pool size from free memory (reference ``src/paged_kv_cache.py:183-194``)."""
+    budget = int(free_bytes * utilization) - reserve_bytes
+    if budget <= 0:
+        raise RuntimeError("not enough free GPU memory for a cache pool")
+    pages = budget // max(1, bytes_per_page)
+    if pages < 2:
+        raise RuntimeError("free GPU memory is too small to hold even one cache page")
+    return int(pages)

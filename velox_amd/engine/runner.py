@@ -1,0 +1,150 @@
+"""The step function: one batch of (request, its next tokens) through the model, from the cache.
+
+The reference runs a step as up to two forwards, a varlen prefill batch and a decode
+batch (``engine/engine.py:303-316``, ``engine/model_runner.py:298-313``).  Here a step is ONE
+forward over one flat batch: every entry brings ``q_len >= 1`` tokens that start at its own
+position; portions of prompts sit beside single decoded tokens.  Only the tokens given
+are run; everything earlier is read from the cache.  Logits come back for the wanted rows
+only, in float32 (the reference likewise runs its head on chosen rows,
+``engine/engine.py:307-309,339-341``).
+
+A batch in which every entry has one token may be replayed from a captured HIP graph:
+graphs are captured per batch-size bucket 1, 2, 4, ... (reference
+``engine/model_runner.py:19-26,331-368``), rows beyond the batch are padded with one-token
+rows that read and write the reserved null page, and the step's tensors live at fixed
+addresses that the host refreshes before each replay.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..cache.manager import CacheManager
+from ..parts.model import DecoderModel
+from .batch import BatchBuilder, StepContext, StepEntry, Workspace
+
+
+def decode_buckets(max_num_seqs: int) -> List[int]:
+    buckets: List[int] = []
+    size = 1
+    while size < max_num_seqs:
+        buckets.append(size)
+        size *= 2
+    buckets.append(max_num_seqs)
+    return buckets
+
+
+class ModelRunner:
+    def __init__(
+        self,
+        model: DecoderModel,
+        cache: CacheManager,
+        ops,
+        dtype: torch.dtype,
+        device,
+        max_num_tokens: int,
+        max_num_seqs: int,
+        enable_graphs: bool = False,
+    ) -> None:
+        self.model = model
+        self.cache = cache
+        self.ops = ops
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.max_num_tokens = max(int(max_num_tokens), int(max_num_seqs))
+        self.max_num_seqs = int(max_num_seqs)
+        self.builder = BatchBuilder(cache, self.device, self.max_num_tokens, self.max_num_seqs)
+        self.workspace = Workspace(self.device)
+        self.enable_graphs = bool(enable_graphs) and self.device.type == "cuda"
+        self._graphs: Dict[int, Tuple[object, torch.Tensor, torch.Tensor]] = {}
+        self._graph_buffers: Dict[int, torch.Tensor] = {}
+        self._graph_pool = None
+        self.num_graph_replays = 0
+
+    # -- the step -----------------------------------------------------------------------
+    @torch.no_grad()
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Runs the entries' tokens as one batch; returns float32 logits ``[wanted, vocab]``
+        in the order of the entries and of their ``want`` (None when nothing is wanted)."""
+        if self.enable_graphs and all(len(e.token_ids) == 1 for e in entries):
+            if all(list(e.want) == [0] for e in entries):
+                bucket = self._bucket_for(len(entries))
+                if bucket is not None:
+                    return self._replay(bucket, entries)
+        ctx = self.builder.build(entries, self.ops, self.dtype, self.workspace)
+        return self._forward(ctx)
+
+    def _forward(self, ctx: StepContext) -> Optional[torch.Tensor]:
+        residual, pending = self.model.forward(ctx.token_ids, ctx)
+        if ctx.rows is None:
+            return None
+        return self.model.logits(residual, pending, ctx.rows, ctx)
+
+    # -- captured decode ----------------------------------------------------------------
+    def _bucket_for(self, batch: int) -> Optional[int]:
+        for bucket in sorted(self._graphs):
+            if bucket >= batch:
+                return bucket
+        return None
+
+    def _padded_entries_context(self, bucket: int, entries: Sequence[StepEntry]) -> StepContext:
+        buffer = self._graph_buffers[bucket]
+        padded = [StepEntry(e.seq, e.token_ids, e.start, [0]) for e in entries]
+        ctx = self.builder.build(
+            padded, self.ops, self.dtype, self.workspace,
+            device_buffer=buffer, pad_to=bucket, width=self.builder.width,
+        )
+        return ctx
+
+    @torch.no_grad()
+    def capture_decode_graphs(self, buckets: Optional[Sequence[int]] = None, warmup_iters: int = 2) -> None:
+        """Captures one graph per bucket over padded one-token rows (reference ``engine/model_runner.py:331-368``)."""
+        if not self.enable_graphs:
+            return
+        buckets = list(buckets) if buckets is not None else decode_buckets(self.max_num_seqs)
+        self._graph_pool = torch.cuda.graph_pool_handle()
+        for bucket in buckets:
+            capacity = self.builder.section_total(bucket, bucket, bucket, self.builder.width)
+            self._graph_buffers[bucket] = torch.zeros(capacity, dtype=torch.int32, device=self.device)
+            ctx = self._graph_context(bucket)
+            stream = torch.cuda.Stream(device=self.device)
+            stream.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(stream):
+                for _ in range(warmup_iters):
+                    self._forward(ctx)
+            torch.cuda.current_stream().wait_stream(stream)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                logits = self._forward(ctx)
+            self._graphs[bucket] = (graph, logits, ctx)
+        torch.cuda.synchronize()
+
+    def _graph_context(self, bucket: int) -> StepContext:
+        """A context of ``bucket`` padded rows only (all on the null page), laid out in the bucket's buffer."""
+        from ..cache.manager import SequenceCache
+
+        null_seq = SequenceCache(slot=self.cache.state.pad_slot, tables=[[0] for _ in self.cache.groups], released=[0 for _ in self.cache.groups])
+        entries = [StepEntry(null_seq, [0], 0, [0]) for _ in range(bucket)]
+        ctx = self.builder.build(
+            entries, self.ops, self.dtype, self.workspace,
+            device_buffer=self._graph_buffers[bucket], pad_to=bucket, width=self.builder.width,
+        )
+        ctx.all_decode = True
+        # lengths are read from device memory at replay; the capture must not specialise on them
+        for group in ctx.groups:
+            group.max_kv_len = self.cache.max_model_len
+        ctx.rows = ctx.rows[:bucket]
+        return ctx
+
+    def _replay(self, bucket: int, entries: Sequence[StepEntry]) -> torch.Tensor:
+        graph, logits, _ = self._graphs[bucket]
+        self._padded_entries_context(bucket, entries)  # refreshes the bucket's buffer in place
+        graph.replay()
+        self.num_graph_replays += 1
+        return logits[: len(entries)]
+
+    @property
+    def uses_graphs(self) -> bool:
+        return bool(self._graphs)

@@ -1,0 +1,2 @@
+"""Architectures built in; importing the package registers them."""
+from . import qwen2  # noqa: F401

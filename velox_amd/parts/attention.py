@@ -1,0 +1,96 @@
+"""Grouped-query attention over the paged cache.
+
+Order of operations follows the reference's ``SelfAttention.forward``
+(``src/self_attention.py:46-90``): one fused QKV product (rows ``[Wq; Wk; Wv]``, bias
+``[bq; bk; bv]``), split into heads, rotate Q and K, write K and V into the cache,
+attend over the cache (so a portion reads its own keys from the cache), output
+product.  ``scale = head_dim ** -0.5`` is applied to the float32 scores after the dot
+(``src/self_attention.py:35``, ``src/attention_prefill.py:101``).  Query head ``h`` reads
+KV head ``h // (heads / kv_heads)`` (``src/attention_prefill.py:36``).
+
+Every size is a constructor argument; ``window`` (None = all keys) and ``bias`` are
+options of the part, chosen by the architecture per layer.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .base import Mixer, PagedNeed, Param, PositionEncoding, fused_rows, register_part, single
+
+
+class AttentionMixer(Mixer):
+    def __init__(
+        self,
+        prefix: str,
+        hidden_size: int,
+        num_heads: int,
+        num_kv_heads: int,
+        head_dim: int,
+        position: Optional[PositionEncoding] = None,
+        qkv_bias: bool = True,
+        window: Optional[int] = None,
+        scale: Optional[float] = None,
+    ) -> None:
+        super().__init__(prefix)
+        if num_heads % num_kv_heads != 0:
+            raise ValueError(f"num_heads={num_heads} must be a multiple of num_kv_heads={num_kv_heads}")
+        if head_dim % 16 != 0 or not 16 <= head_dim <= 256:
+            raise ValueError(f"head_dim={head_dim}: the attention kernels take multiples of 16 from 16 to 256")
+        if window is not None and window < 1:
+            raise ValueError(f"window={window} must be at least 1")
+        self.hidden_size = int(hidden_size)
+        self.num_heads = int(num_heads)
+        self.num_kv_heads = int(num_kv_heads)
+        self.head_dim = int(head_dim)
+        self.position = position
+        self.qkv_bias = bool(qkv_bias)
+        self.window = window
+        self.scale = float(scale) if scale is not None else 1.0 / (self.head_dim ** 0.5)
+        self.q_size = self.num_heads * self.head_dim
+        self.kv_size = self.num_kv_heads * self.head_dim
+        self.qkv_weight: Optional[torch.Tensor] = None
+        self.qkv_bias_vec: Optional[torch.Tensor] = None
+        self.o_weight: Optional[torch.Tensor] = None
+
+    def params(self) -> Dict[str, Param]:
+        h, q, kv = self.hidden_size, self.q_size, self.kv_size
+        out = {
+            "qkv_weight": fused_rows(
+                ("q_proj.weight", "k_proj.weight", "v_proj.weight"), ((q, h), (kv, h), (kv, h))
+            ),
+            "o_weight": single("o_proj.weight", (h, q)),
+        }
+        if self.qkv_bias:
+            out["qkv_bias_vec"] = fused_rows(
+                ("q_proj.bias", "k_proj.bias", "v_proj.bias"), ((q,), (kv,), (kv,)), role="vector"
+            )
+        return out
+
+    def cache_need(self):
+        return PagedNeed(self.num_kv_heads, self.head_dim, self.window)
+
+    def forward(self, x, ctx, cache, owns_cache: bool = True):
+        ops = ctx.ops
+        qkv = ops.linear(x, self.qkv_weight, self.qkv_bias_vec if self.qkv_bias else None, ctx.dtype)
+        tables = self.position.rotary_tables() if self.position is not None else None
+        cos, sin = tables if tables is not None else (None, None)
+        meta = cache.batch
+        ops.rope_kv_write(
+            qkv, self.num_heads, self.num_kv_heads, self.head_dim,
+            ctx.positions, cos, sin,
+            meta.slot_mapping, cache.k, cache.v, cache.block_size,
+            write_kv=owns_cache,
+        )
+        attn = ops.paged_attention(
+            qkv, self.num_heads, self.num_kv_heads, self.head_dim,
+            cache.k, cache.v, cache.block_size,
+            meta.block_tables, ctx.cu_q, meta.kv_lens,
+            ctx.max_q_len, meta.max_kv_len, self.scale, self.window,
+            ctx.all_decode, ctx.workspace,
+        )
+        return ops.linear(attn, self.o_weight, None, ctx.dtype)
+
+
+register_part("mixer", "attention", AttentionMixer)

@@ -1,0 +1,177 @@
+"""Interfaces of the parts a decoder is put together from.
+
+A *part* owns tensors (declared as :class:`Param`) and one piece of arithmetic.
+It is given its sizes and constants at construction and never learns which
+model it sits in.  Four kinds exist, each with a registry from a kind name to a
+class so that an architecture (or a test) can add its own:
+
+``Mixer``
+    mixes information between the tokens of a sequence (attention here).  It
+    declares what it needs of the cache manager through :meth:`cache_need`.
+``FeedForward``
+    ``[T, H] -> [T, H]`` per token (dense gated MLP here; routed experts would
+    be another kind behind the same call).
+``Norm``
+    owns the residual update: ``residual += delta; return normalise(residual)``.
+``PositionEncoding``
+    either changes the embeddings (absolute encodings) or hands rotary tables to
+    the mixer, which fuses the rotation into its cache write.
+
+``Block`` arranges one mixer, one feed-forward and their norms.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, Dict, Optional, Tuple
+
+import torch
+
+
+# ----------------------------------------------------------------------------------------
+# parameters
+# ----------------------------------------------------------------------------------------
+@dataclass(frozen=True)
+class Param:
+    """One tensor a part owns and where it comes from in a checkpoint.
+
+    ``sources`` are checkpoint tensor names relative to the part's prefix; more
+    than one means "concatenate along dim 0" (the reference fuses q/k/v and
+    gate/up the same way, ``src/weight_loader.py:91-98``).  ``role`` decides the
+    dtype it is held in: a ``matrix`` follows the run's dtype (a checkpoint tensor
+    stored in 32-bit stays 32-bit), a ``vector`` (norm weights, biases) is always
+    held in float32.  ``init`` names the random-weights law: ``normal`` is
+    N(0, 0.02), ``one_plus_normal`` is 1 + N(0, 0.02).
+    """
+
+    shape: Tuple[int, ...]
+    sources: Tuple[str, ...]
+    source_shapes: Tuple[Tuple[int, ...], ...]
+    role: str = "matrix"
+    init: str = "normal"
+    alias_of: Optional[str] = None  # absolute checkpoint name this falls back to (tied head)
+
+
+def single(name: str, shape: Tuple[int, ...], role: str = "matrix", init: str = "normal") -> Param:
+    return Param(shape=tuple(shape), sources=(name,), source_shapes=(tuple(shape),), role=role, init=init)
+
+
+def fused_rows(names: Tuple[str, ...], shapes: Tuple[Tuple[int, ...], ...], role: str = "matrix") -> Param:
+    rows = sum(s[0] for s in shapes)
+    return Param(shape=(rows,) + tuple(shapes[0][1:]), sources=tuple(names), source_shapes=tuple(tuple(s) for s in shapes), role=role)
+
+
+class Part:
+    """Base of every part: a prefix in the checkpoint's name space plus declared tensors."""
+
+    def __init__(self, prefix: str = "") -> None:
+        self.prefix = prefix
+
+    def params(self) -> Dict[str, Param]:
+        """attribute name -> Param; the loader sets ``self.<attribute>`` to the bound tensor."""
+        return {}
+
+    def children(self) -> Tuple["Part", ...]:
+        return ()
+
+    def finalize(self, device: torch.device, dtype: torch.dtype) -> None:
+        """Called once after the weights are bound (build tables, derived tensors)."""
+
+
+# ----------------------------------------------------------------------------------------
+# what a mixer needs of the cache manager
+# ----------------------------------------------------------------------------------------
+@dataclass(frozen=True)
+class PagedNeed:
+    """Keys and values that grow by one entry per token, kept in pages.
+
+    ``window`` = None keeps every key; an integer keeps the last ``window`` keys
+    (a query at position p reads keys p-window+1 .. p), so pages wholly behind
+    the window can be given back while the request is still running.
+    """
+
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Per-request state of fixed size: ``(name, shape, dtype)`` per tensor, dtype None = run dtype."""
+
+    tensors: Tuple[Tuple[str, Tuple[int, ...], Optional[torch.dtype]], ...]
+
+
+class Mixer(Part):
+    def cache_need(self):
+        """``PagedNeed``, ``StateNeed`` or None."""
+        return None
+
+    def forward(self, x: torch.Tensor, ctx, cache, owns_cache: bool = True) -> torch.Tensor:
+        """``x`` [T, H] in the run dtype -> [T, H].
+
+        ``cache`` is this schedule entry's view of the cache (or the entry's it reads
+        from when ``owns_cache`` is false: then nothing may be written to it).
+        """
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Norm(Part):
+    def forward(self, residual: torch.Tensor, delta: Optional[torch.Tensor], ctx, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``residual`` [T, H] float32.
+
+        With ``rows`` None: ``residual += delta`` in place (delta may be None) and the
+        normalised residual comes back in the run dtype, [T, H].  With ``rows`` (int32
+        [R]): nothing is changed and ``normalise(residual[rows] + delta[rows])`` comes back.
+        """
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def on_embeddings(self, hidden: torch.Tensor, ctx) -> torch.Tensor:
+        return hidden
+
+    def rotary_tables(self) -> Optional[Tuple[torch.Tensor, torch.Tensor]]:
+        """(cos, sin), float32 [max_position, rotary_dim/2], or None when nothing rotates."""
+        return None
+
+
+# ----------------------------------------------------------------------------------------
+# registries of kinds
+# ----------------------------------------------------------------------------------------
+_MIXERS: Dict[str, Callable[..., Mixer]] = {}
+_FEED_FORWARDS: Dict[str, Callable[..., FeedForward]] = {}
+_NORMS: Dict[str, Callable[..., Norm]] = {}
+_POSITIONS: Dict[str, Callable[..., PositionEncoding]] = {}
+_TABLES = {"mixer": _MIXERS, "feed_forward": _FEED_FORWARDS, "norm": _NORMS, "position": _POSITIONS}
+
+
+def register_part(family: str, kind: str, factory: Callable[..., Part]) -> None:
+    table = _TABLES[family]
+    table[kind] = factory
+
+
+def make_part(family: str, kind: str, **kwargs) -> Part:
+    table = _TABLES[family]
+    if kind not in table:
+        raise KeyError(f"unknown {family} kind {kind!r}; registered: {sorted(table)}")
+    return table[kind](**kwargs)
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    """A kind name plus the constants handed to its constructor."""
+
+    kind: str
+    args: Tuple[Tuple[str, object], ...] = ()
+
+    @staticmethod
+    def of(kind: str, **kwargs) -> "PartSpec":
+        return PartSpec(kind, tuple(sorted(kwargs.items())))
+
+    def kwargs(self) -> Dict[str, object]:
+        return dict(self.args)

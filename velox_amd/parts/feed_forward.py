@@ -1,0 +1,41 @@
+"""Dense gated feed-forward.
+
+Reference ``src/mlp.py:9-15``: one fused product with rows ``[Wgate; Wup]`` (no bias),
+``act(gate) * up``, down product (no bias); ``silu(x) = x * sigmoid(x)``.  The
+activation and the product are one kernel here and are computed in float32
+from the stored gate/up values, with one rounding at the store.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .base import FeedForward, Param, fused_rows, register_part, single
+
+
+class GatedMLP(FeedForward):
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, activation: str = "silu") -> None:
+        super().__init__(prefix)
+        if activation != "silu":
+            raise ValueError(f"activation {activation!r} is not implemented (only 'silu')")
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        self.gate_up_weight: Optional[torch.Tensor] = None
+        self.down_weight: Optional[torch.Tensor] = None
+
+    def params(self) -> Dict[str, Param]:
+        h, i = self.hidden_size, self.intermediate_size
+        return {
+            "gate_up_weight": fused_rows(("gate_proj.weight", "up_proj.weight"), ((i, h), (i, h))),
+            "down_weight": single("down_proj.weight", (h, i)),
+        }
+
+    def forward(self, x, ctx):
+        ops = ctx.ops
+        gate_up = ops.linear(x, self.gate_up_weight, None, ctx.dtype)
+        act = ops.silu_mul(gate_up)
+        return ops.linear(act, self.down_weight, None, ctx.dtype)
+
+
+register_part("feed_forward", "gated_mlp", GatedMLP)

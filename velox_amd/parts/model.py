@@ -1,0 +1,174 @@
+"""A decoder described as data, and the object built from that description.
+
+``ModelSpec`` is what an architecture produces from its configuration: one
+``LayerSpec`` per weight-owning layer (each naming its own mixer, feed-forward and
+norm kinds with their constants), shared position encodings, and ``schedule``, the
+order in which layers run.  The schedule is a list of ``ScheduleEntry``: an entry may
+name a layer that an earlier entry already named (the layer's weights run twice, each
+run with a cache of its own), or set ``cache_from`` to an earlier entry to read that
+entry's cache instead of owning one.
+
+``DecoderModel`` runs the whole thing the way the reference's ``QwenDecoderModel``
+does (``src/transformer.py:43-52``): embed, blocks in schedule order, final norm; the
+output head is a separate call on chosen rows (``src/transformer.py:67-68``).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from .base import Param, Part, PartSpec, make_part, single
+from .block import BLOCK_ARRANGEMENTS
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    prefix: str
+    mixer: PartSpec
+    feed_forward: PartSpec
+    mixer_norm: PartSpec
+    ff_norm: PartSpec
+    position: Optional[str] = None  # key into ModelSpec.positions handed to the mixer
+    arrangement: str = "pre_norm"
+    mixer_prefix: str = "self_attn."
+    feed_forward_prefix: str = "mlp."
+    mixer_norm_prefix: str = "input_layernorm."
+    ff_norm_prefix: str = "post_attention_layernorm."
+
+
+@dataclass(frozen=True)
+class ScheduleEntry:
+    layer: int
+    cache_from: Optional[int] = None
+
+
+@dataclass
+class ModelSpec:
+    vocab_size: int
+    hidden_size: int
+    max_position: int
+    layers: List[LayerSpec]
+    schedule: List[ScheduleEntry]
+    final_norm: PartSpec
+    positions: Dict[str, PartSpec] = field(default_factory=dict)
+    embedding_position: Optional[str] = None  # a position encoding applied to the embeddings
+    tie_head: bool = False
+    embed_name: str = "model.embed_tokens.weight"
+    head_name: str = "lm_head.weight"
+    final_norm_prefix: str = "model.norm."
+    eos_token_ids: Tuple[int, ...] = ()
+
+    def validate(self) -> None:
+        if not self.layers:
+            raise ValueError("a model needs at least one layer")
+        for index, entry in enumerate(self.schedule):
+            if not 0 <= entry.layer < len(self.layers):
+                raise ValueError(f"schedule[{index}] names layer {entry.layer}, but there are {len(self.layers)}")
+            if entry.cache_from is not None:
+                if not 0 <= entry.cache_from < index:
+                    raise ValueError(f"schedule[{index}].cache_from must name an earlier entry")
+                if self.schedule[entry.cache_from].cache_from is not None:
+                    raise ValueError(f"schedule[{index}].cache_from must name an entry that owns its cache")
+
+
+class Embedding(Part):
+    def __init__(self, name: str, vocab_size: int, hidden_size: int) -> None:
+        super().__init__("")
+        self.name = name
+        self.vocab_size = vocab_size
+        self.hidden_size = hidden_size
+        self.table: Optional[torch.Tensor] = None
+
+    def params(self) -> Dict[str, Param]:
+        return {"table": single(self.name, (self.vocab_size, self.hidden_size))}
+
+    def forward(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
+        return ctx.ops.embed(token_ids, self.table)
+
+
+class OutputHead(Part):
+    """``logits = hidden @ W^T`` without bias; ``W`` is the embedding table when tied
+    (reference ``src/transformer.py:60-62``).  Logits are returned in float32."""
+
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str]) -> None:
+        super().__init__("")
+        self.name = name
+        self.vocab_size = vocab_size
+        self.hidden_size = hidden_size
+        self.tied_to = tied_to
+        self.weight: Optional[torch.Tensor] = None
+
+    def params(self) -> Dict[str, Param]:
+        base = single(self.name, (self.vocab_size, self.hidden_size))
+        if self.tied_to is None:
+            return {"weight": base}
+        return {"weight": Param(base.shape, base.sources, base.source_shapes, base.role, base.init, alias_of=self.tied_to)}
+
+    def forward(self, hidden_rows: torch.Tensor, ctx) -> torch.Tensor:
+        return ctx.ops.linear(hidden_rows, self.weight, None, torch.float32)
+
+
+class DecoderModel(Part):
+    def __init__(self, spec: ModelSpec) -> None:
+        super().__init__("")
+        spec.validate()
+        self.spec = spec
+        self.positions = {key: make_part("position", ps.kind, **ps.kwargs()) for key, ps in spec.positions.items()}
+        self.embedding = Embedding(spec.embed_name, spec.vocab_size, spec.hidden_size)
+        self.blocks = []
+        for layer in spec.layers:
+            mixer_kwargs = layer.mixer.kwargs()
+            if layer.position is not None:
+                mixer_kwargs["position"] = self.positions[layer.position]
+            mixer = make_part("mixer", layer.mixer.kind, prefix=layer.prefix + layer.mixer_prefix, **mixer_kwargs)
+            ff = make_part("feed_forward", layer.feed_forward.kind, prefix=layer.prefix + layer.feed_forward_prefix, **layer.feed_forward.kwargs())
+            norm1 = make_part("norm", layer.mixer_norm.kind, prefix=layer.prefix + layer.mixer_norm_prefix, **layer.mixer_norm.kwargs())
+            norm2 = make_part("norm", layer.ff_norm.kind, prefix=layer.prefix + layer.ff_norm_prefix, **layer.ff_norm.kwargs())
+            self.blocks.append(BLOCK_ARRANGEMENTS[layer.arrangement](layer.prefix, mixer, ff, norm1, norm2))
+        self.final_norm = make_part("norm", spec.final_norm.kind, prefix=spec.final_norm_prefix, **spec.final_norm.kwargs())
+        self.head = OutputHead(spec.head_name, spec.vocab_size, spec.hidden_size, spec.embed_name if spec.tie_head else None)
+        self.schedule = list(spec.schedule)
+
+    # -- structure ----------------------------------------------------------------------
+    def children(self) -> Tuple[Part, ...]:
+        return (self.embedding, *self.positions.values(), *self.blocks, self.final_norm, self.head)
+
+    def all_parts(self) -> List[Part]:
+        out: List[Part] = []
+
+        def walk(part: Part) -> None:
+            out.append(part)
+            for child in part.children():
+                walk(child)
+
+        for child in self.children():
+            walk(child)
+        return out
+
+    def cache_needs(self) -> List[object]:
+        """One entry per schedule entry: the mixer's need, or None when it reads another entry's cache."""
+        needs = []
+        for entry in self.schedule:
+            need = self.blocks[entry.layer].mixer.cache_need()
+            needs.append(need if entry.cache_from is None else None)
+        return needs
+
+    # -- arithmetic ---------------------------------------------------------------------
+    def forward(self, token_ids: torch.Tensor, ctx):
+        """Runs every block; returns ``(residual float32 [T, H], pending [T, H])``."""
+        residual = self.embedding.forward(token_ids, ctx)
+        if self.spec.embedding_position is not None:
+            residual = self.positions[self.spec.embedding_position].on_embeddings(residual, ctx)
+        pending = None
+        for index, entry in enumerate(self.schedule):
+            owner = index if entry.cache_from is None else entry.cache_from
+            cache = ctx.cache_view(owner)
+            pending = self.blocks[entry.layer].forward(residual, pending, ctx, cache, entry.cache_from is None)
+        return residual, pending
+
+    def logits(self, residual: torch.Tensor, pending, rows: torch.Tensor, ctx) -> torch.Tensor:
+        """Final norm and output head on ``rows`` (int32 [R]) only: float32 [R, vocab]."""
+        hidden = self.final_norm.forward(residual, pending, ctx, rows=rows)
+        return self.head.forward(hidden, ctx)
