@@ -1,0 +1,311 @@
+"""Each HIP kernel alone against its plain PyTorch reference (tests/torch_ops.py), in float32 and
+bfloat16, at sizes other than the engine's tiny models: widths and vocabularies that are no power
+of two, head sizes 16 .. 256, groups of 1, 3, 7, page sizes 4 .. 64."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from torch_ops import TorchOps, exponential_noise
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from velox_amd.kernels import load_ops
+
+    return load_ops("cuda")
+
+
+@pytest.fixture(scope="module")
+def ref():
+    return TorchOps()
+
+
+def tol(dtype):
+    return dict(rtol=2e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-3)
+
+
+def rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).cuda()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden,vocab", [(96, 320), (3584, 1000), (50, 77)])
+def test_embed(ops, ref, dtype, hidden, vocab):
+    table = rand((vocab, hidden), dtype, 0)
+    ids = torch.randint(0, vocab, (37,), generator=torch.Generator().manual_seed(1)).to(torch.int32).cuda()
+    torch.testing.assert_close(ops.embed(ids, table), ref.embed(ids, table), rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [64, 96, 3584, 1000])
+def test_add_rmsnorm(ops, ref, dtype, hidden):
+    tokens = 19
+    residual = rand((tokens, hidden), torch.float32, 2)
+    delta = rand((tokens, hidden), dtype, 3)
+    weight = 1 + rand((hidden,), torch.float32, 4, 0.02)
+    r_hip, r_ref = residual.clone(), residual.clone()
+    got = ops.add_rmsnorm(r_hip, delta, weight, 1e-5, dtype)
+    want = ref.add_rmsnorm(r_ref, delta, weight, 1e-5, dtype)
+    torch.testing.assert_close(r_hip, r_ref, rtol=0, atol=0)
+    torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+    # no delta: the residual is untouched
+    before = r_hip.clone()
+    got = ops.add_rmsnorm(r_hip, None, weight, 1e-6, dtype)
+    torch.testing.assert_close(r_hip, before, rtol=0, atol=0)
+    torch.testing.assert_close(got.float(), ref.add_rmsnorm(r_ref, None, weight, 1e-6, dtype).float(), **tol(dtype))
+    # chosen rows: nothing is written
+    rows = torch.tensor([18, 0, 7, 7], dtype=torch.int32).cuda()
+    got = ops.add_rmsnorm_rows(r_hip, delta, rows, weight, 1e-6, dtype)
+    torch.testing.assert_close(r_hip, before, rtol=0, atol=0)
+    torch.testing.assert_close(got.float(), ref.add_rmsnorm_rows(r_ref, delta, rows, weight, 1e-6, dtype).float(), **tol(dtype))
+
+
+def test_rmsnorm_eps_is_inside_the_root(ops):
+    # tiny inputs: rsqrt(ms + eps) and 1 / (sqrt(ms) + eps) differ by orders of magnitude
+    hidden = 128
+    x = torch.full((1, hidden), 1e-4, device="cuda")
+    w = torch.ones(hidden, device="cuda")
+    got = ops.add_rmsnorm(x.clone(), None, w, 1e-6, torch.float32)
+    want = 1e-4 / math.sqrt(1e-8 + 1e-6)
+    torch.testing.assert_close(got, torch.full_like(got, want), rtol=1e-5, atol=0)
+
+
+@pytest.mark.parametrize("a_dtype,w_dtype,out_dtype", [
+    (torch.float32, torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16, torch.bfloat16),
+    (torch.bfloat16, torch.float32, torch.bfloat16), (torch.bfloat16, torch.bfloat16, torch.float32),
+])
+@pytest.mark.parametrize("m,n,k", [(1, 320, 96), (7, 263, 80), (65, 130, 150), (130, 64, 224), (3, 70, 37)])
+def test_gemm_fma(ops, ref, a_dtype, w_dtype, out_dtype, m, n, k):
+    x = rand((m, k), a_dtype, 5)
+    w = rand((n, k), w_dtype, 6, 0.05)
+    bias = rand((n,), torch.float32, 7)
+    for b in (None, bias):
+        got = ops.gemm_fma(x, w, b, out_dtype)
+        want = ref.linear(x, w, b, out_dtype)
+        torch.testing.assert_close(got.float(), want.float(), **tol(out_dtype))
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 320, 96), (8, 152064 // 8, 512), (64, 1000, 3584), (300, 4608, 3584)])
+def test_linear_bf16_library_path(ops, ref, m, n, k):
+    x = rand((m, k), torch.bfloat16, 8)
+    w = rand((n, k), torch.bfloat16, 9, 0.02)
+    got = ops.linear(x, w, None, torch.bfloat16)
+    want = ref.linear(x, w, None, torch.bfloat16)
+    torch.testing.assert_close(got.float(), want.float(), rtol=2e-2, atol=2e-2)
+    got32 = ops.linear(x, w, None, torch.float32)
+    torch.testing.assert_close(got32, ref.linear(x, w, None, torch.float32), rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("inter", [128, 224, 150, 18944])
+def test_silu_mul(ops, ref, dtype, inter):
+    gate_up = rand((11, 2 * inter), dtype, 10, 2.0)
+    torch.testing.assert_close(ops.silu_mul(gate_up).float(), ref.silu_mul(gate_up).float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,half,page", [(4, 2, 16, 8, 4), (3, 1, 32, 16, 8), (6, 2, 48, 24, 16), (28, 4, 128, 64, 16), (2, 2, 64, 16, 32), (5, 5, 16, 0, 4)])
+def test_rope_kv_write(ops, ref, dtype, nh, nkv, d, half, page):
+    tokens, pages = 23, 12
+    width = (nh + 2 * nkv) * d
+    qkv = rand((tokens, width), dtype, 11)
+    bias = rand((width,), torch.float32, 12, 0.1)
+    positions = torch.randint(0, 500, (tokens,), generator=torch.Generator().manual_seed(13)).to(torch.int32).cuda()
+    slots = (torch.randperm((pages - 1) * page, generator=torch.Generator().manual_seed(14))[:tokens] + page).to(torch.int32).cuda()
+    if half:
+        angles = torch.outer(torch.arange(512, dtype=torch.float32), 1.0 / (10000.0 ** (torch.arange(half, dtype=torch.float32) / half)))
+        cos, sin = angles.cos().cuda(), angles.sin().cuda()
+    else:
+        cos = sin = None
+    for use_bias in (bias, None):
+        caches = []
+        for impl in (ops, ref):
+            k_cache = torch.zeros((pages, nkv, page, d), dtype=dtype, device="cuda")
+            v_cache = torch.zeros((pages, nkv, d, page), dtype=dtype, device="cuda")
+            buf = qkv.clone()
+            impl.rope_kv_write(buf, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, write_kv=True, bias=use_bias)
+            caches.append((buf[:, : nh * d].float(), k_cache.float(), v_cache.float()))
+        for got, want in zip(*caches):
+            torch.testing.assert_close(got, want, **tol(dtype))
+    # write_kv=False leaves the cache alone
+    k_cache = torch.zeros((pages, nkv, page, d), dtype=dtype, device="cuda")
+    v_cache = torch.zeros((pages, nkv, d, page), dtype=dtype, device="cuda")
+    ops.rope_kv_write(qkv.clone(), nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, write_kv=False, bias=bias)
+    assert not k_cache.any() and not v_cache.any()
+
+
+def _attention_case(dtype, nh, nkv, d, page, seqs, seed, garbage=False):
+    """seqs: list of (q_len, kv_len).  Builds a paged cache with shuffled pages and a flat qkv."""
+    g = torch.Generator().manual_seed(seed)
+    total_pages = sum((kv + page - 1) // page for _, kv in seqs) + 3
+    perm = (torch.randperm(total_pages - 1, generator=g) + 1).tolist()
+    k_cache = torch.zeros((total_pages, nkv, page, d), dtype=dtype)
+    v_cache = torch.zeros((total_pages, nkv, d, page), dtype=dtype)
+    if garbage:
+        k_cache.normal_(0, 50.0, generator=g)
+        v_cache.normal_(0, 50.0, generator=g)
+    width = max((kv + page - 1) // page for _, kv in seqs)
+    tables = torch.zeros((len(seqs), width), dtype=torch.int32)
+    tokens = sum(q for q, _ in seqs)
+    qkv = (torch.randn((tokens, (nh + 2 * nkv) * d), generator=g)).to(dtype)
+    cu = [0]
+    for b, (q_len, kv_len) in enumerate(seqs):
+        n_pages = (kv_len + page - 1) // page
+        mine = [perm.pop() for _ in range(n_pages)]
+        tables[b, :n_pages] = torch.tensor(mine, dtype=torch.int32)
+        keys = torch.randn((kv_len, nkv, d), generator=g).to(dtype)
+        values = torch.randn((kv_len, nkv, d), generator=g).to(dtype)
+        for n in range(kv_len):
+            k_cache[mine[n // page], :, n % page, :] = keys[n]
+            v_cache[mine[n // page], :, :, n % page] = values[n]
+        cu.append(cu[-1] + q_len)
+    return dict(
+        qkv=qkv.cuda(), k_cache=k_cache.cuda(), v_cache=v_cache.cuda(), tables=tables.cuda(),
+        cu=torch.tensor(cu, dtype=torch.int32).cuda(), kv=torch.tensor([kv for _, kv in seqs], dtype=torch.int32).cuda(),
+        max_q=max(q for q, _ in seqs), max_kv=max(kv for _, kv in seqs),
+    )
+
+
+def _run_attention(impl, case, nh, nkv, d, page, window=None, splits=None, all_decode=False, workspace=None):
+    return impl.paged_attention(
+        case["qkv"], nh, nkv, d, case["k_cache"], case["v_cache"], page, case["tables"], case["cu"], case["kv"],
+        case["max_q"], case["max_kv"], 1.0 / math.sqrt(d), window, all_decode, workspace, splits=splits,
+    ).float()
+
+
+ATTN_SHAPES = [(4, 2, 16, 4), (3, 1, 32, 8), (6, 2, 48, 16), (28, 4, 128, 16), (8, 8, 64, 64), (7, 1, 96, 32), (2, 1, 256, 16), (40, 8, 128, 2)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,page", ATTN_SHAPES)
+def test_paged_attention_mixed_batch(ops, ref, dtype, nh, nkv, d, page):
+    # whole prompts, a portion with earlier context, single decoded tokens, a two-token portion
+    seqs = [(70, 70), (33, 141), (1, 97), (2, 66), (1, 1), (130, 130)]
+    case = _attention_case(dtype, nh, nkv, d, page, seqs, seed=d + nh)
+    got = _run_attention(ops, case, nh, nkv, d, page)
+    want = _run_attention(ref, case, nh, nkv, d, page)
+    torch.testing.assert_close(got, want, **(dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 4), (28, 4, 128, 16), (3, 1, 32, 8)])
+def test_paged_attention_garbage_in_unused_slots_and_null_page(ops, ref, dtype, nh, nkv, d, page):
+    seqs = [(5, 37), (1, 64), (9, 9)]
+    clean = _attention_case(dtype, nh, nkv, d, page, seqs, seed=3)
+    dirty = _attention_case(dtype, nh, nkv, d, page, seqs, seed=3, garbage=True)
+    # same seed: same real keys, values and queries? the garbage draw shifts the stream, so copy them over
+    dirty["qkv"] = clean["qkv"]
+    tables = clean["tables"].cpu()
+    for b, (_, kv_len) in enumerate(seqs):
+        for n in range(kv_len):
+            p, o = int(tables[b, n // page]), n % page
+            dirty["k_cache"][p, :, o, :] = clean["k_cache"][p, :, o, :]
+            dirty["v_cache"][p, :, :, o] = clean["v_cache"][p, :, :, o]
+    dirty["tables"] = clean["tables"]
+    got_clean = _run_attention(ops, clean, nh, nkv, d, page)
+    got_dirty = _run_attention(ops, dirty, nh, nkv, d, page)
+    torch.testing.assert_close(got_dirty, got_clean, rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 4), (28, 4, 128, 16), (7, 1, 96, 32)])
+@pytest.mark.parametrize("window", [1, 5, 64, 100])
+def test_paged_attention_window(ops, ref, dtype, nh, nkv, d, page, window):
+    seqs = [(70, 70), (33, 141), (1, 197), (2, 66)]
+    case = _attention_case(dtype, nh, nkv, d, page, seqs, seed=11)
+    got = _run_attention(ops, case, nh, nkv, d, page, window=window)
+    want = _run_attention(ref, case, nh, nkv, d, page, window=window)
+    torch.testing.assert_close(got, want, **(dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 4), (28, 4, 128, 16), (3, 1, 32, 8), (2, 1, 256, 16)])
+def test_decode_split_keys_equals_one_pass(ops, ref, dtype, nh, nkv, d, page):
+    from velox_amd.engine.batch import Workspace
+
+    seqs = [(1, 700), (1, 3), (1, 129), (1, 64), (1, 1)]
+    case = _attention_case(dtype, nh, nkv, d, page, seqs, seed=21)
+    workspace = Workspace(torch.device("cuda"))
+    one = _run_attention(ops, case, nh, nkv, d, page, splits=1, all_decode=True, workspace=workspace)
+    want = _run_attention(ref, case, nh, nkv, d, page)
+    t = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(one, want, **t)
+    for splits in (2, 3, 8, 32):  # 32 splits leave most of them empty for the short sequences
+        got = _run_attention(ops, case, nh, nkv, d, page, splits=splits, all_decode=True, workspace=workspace)
+        torch.testing.assert_close(got, want, **t)
+
+
+def test_far_key_among_hundreds_is_found(ops):
+    # one key far back matches the query strongly: the output must be (nearly) that key's value
+    nh, nkv, d, page = 4, 2, 64, 16
+    seqs = [(1, 900)]
+    case = _attention_case(torch.float32, nh, nkv, d, page, seqs, seed=5)
+    target = 37
+    tables = case["tables"].cpu()
+    q = case["qkv"][0, : nh * d].view(nh, d)
+    p, o = int(tables[0, target // page]), target % page
+    for h in range(nh):
+        case["k_cache"][p, h // 2, o, :] = 0
+    case["k_cache"][p, 0, o, :] = 4.0 * (q[0] + q[1]) / 2
+    case["k_cache"][p, 1, o, :] = 4.0 * (q[2] + q[3]) / 2
+    out = _run_attention(ops, case, nh, nkv, d, page).view(nh, d)
+    want = _run_attention(TorchOps(), case, nh, nkv, d, page).view(nh, d)
+    torch.testing.assert_close(out, want, rtol=1e-4, atol=1e-5)
+
+
+def test_argmax_and_sampling(ops, ref):
+    vocab = 1003
+    logits = rand((6, vocab), torch.float32, 30, 3.0)
+    logits[2, 77] = logits[2, 900] = 50.0  # a tie: the first index wins
+    torch.testing.assert_close(ops.argmax(logits), ref.argmax(logits))
+    assert int(ops.argmax(logits)[2]) == 77
+
+    options = np.zeros((6, 6), dtype=np.int32)
+    f = options.view(np.float32)
+    rows = [(0.0, 1.0, 0), (0.8, 1.0, 0), (1.0, 0.9, 0), (1.3, 1.0, 5), (0.7, 0.5, 50), (1.0, 1.0, 1)]
+    for r, (temp, top_p, top_k) in enumerate(rows):
+        f[r, 0], f[r, 1] = temp, top_p
+        options[r, 2:] = (top_k, 1234 + r, 99, r)
+    got = ops.sample(logits, torch.from_numpy(options).cuda()).cpu().numpy()
+    for r in range(6):
+        token, scores = TorchOps.sample_row(logits[r].cpu().numpy(), options[r])
+        assert np.isfinite(scores[got[r]]), f"row {r}: token {got[r]} was filtered out"
+        assert scores[got[r]] >= scores.max() - 1e-3, f"row {r}: token {got[r]} score {scores[got[r]]} vs best {scores.max()} ({token})"
+    assert got[0] == int(logits[0].argmax())
+    assert got[5] == int(logits[5].argmax())  # top_k = 1 is greedy
+
+
+def test_sampling_follows_the_distribution(ops):
+    vocab = 50
+    logits = rand((1, vocab), torch.float32, 31, 1.5).repeat(4000, 1).contiguous()
+    options = np.zeros((4000, 6), dtype=np.int32)
+    options.view(np.float32)[:, 0] = 0.9
+    options.view(np.float32)[:, 1] = 1.0
+    options[:, 3] = 7
+    options[:, 5] = np.arange(4000)
+    got = ops.sample(logits, torch.from_numpy(options).cuda()).cpu().numpy()
+    probs = torch.softmax(logits[0].cpu() / 0.9, -1).numpy()
+    counts = np.bincount(got, minlength=vocab)
+    expected = probs * 4000
+    keep = expected > 5
+    chi2 = (((counts - expected) ** 2) / expected)[keep].sum()
+    assert chi2 < 2.0 * keep.sum() + 30, f"chi-square {chi2} over {keep.sum()} bins"
+
+
+def test_penalties(ops, ref):
+    vocab, rows, width = 333, 3, 40
+    logits = rand((rows, vocab), torch.float32, 32, 2.0)
+    tokens = torch.randint(0, 60, (rows, width), generator=torch.Generator().manual_seed(33)).to(torch.int32).cuda()
+    lengths = torch.tensor([40, 0, 17], dtype=torch.int32).cuda()
+    coeffs = torch.tensor([[1.3, 0.5, 0.2], [2.0, 1.0, 1.0], [0.8, 0.0, 0.7]], dtype=torch.float32).cuda()
+    got, want = logits.clone(), logits.clone()
+    ops.apply_penalties(got, tokens, lengths, coeffs)
+    ref.apply_penalties(want, tokens, lengths, coeffs)
+    torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-6)

@@ -92,23 +92,26 @@ class TorchOps:
         return (gate * torch.sigmoid(gate) * up).to(gate_up.dtype)
 
     # -- rotary + cache write -----------------------------------------------------------
-    def rope_kv_write(self, qkv, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size, write_kv=True):
+    def rope_kv_write(self, qkv, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size, write_kv=True, bias=None):
         t = qkv.shape[0]
         q_size, kv_size = num_heads * head_dim, num_kv_heads * head_dim
-        q = qkv[:, :q_size].view(t, num_heads, head_dim)
-        k = qkv[:, q_size:q_size + kv_size].view(t, num_kv_heads, head_dim)
-        v = qkv[:, q_size + kv_size:].view(t, num_kv_heads, head_dim)
+        wide = qkv.float()
+        if bias is not None:
+            wide = wide + bias
+        q = wide[:, :q_size].reshape(t, num_heads, head_dim).clone()
+        k = wide[:, q_size:q_size + kv_size].reshape(t, num_kv_heads, head_dim).clone()
+        v = wide[:, q_size + kv_size:].reshape(t, num_kv_heads, head_dim)
         if cos is not None:
             half = cos.shape[1]
             c = cos[positions.long()].unsqueeze(1)
             s = sin[positions.long()].unsqueeze(1)
             for x in (q, k):
-                lo = x[..., :half].float()
-                hi = x[..., half:2 * half].float()
-                new_lo = (lo * c - hi * s).to(x.dtype)
-                new_hi = (lo * s + hi * c).to(x.dtype)
-                x[..., :half] = new_lo
-                x[..., half:2 * half] = new_hi
+                lo = x[..., :half].clone()
+                hi = x[..., half:2 * half].clone()
+                x[..., :half] = lo * c - hi * s
+                x[..., half:2 * half] = lo * s + hi * c
+        # one rounding, at the store; only the rotated queries go back into qkv
+        qkv[:, :q_size] = q.reshape(t, q_size).to(qkv.dtype)
         if write_kv:
             pages = (slot_mapping.long() // block_size)
             offsets = (slot_mapping.long() % block_size)
@@ -116,7 +119,7 @@ class TorchOps:
             v_cache[pages, :, :, offsets] = v.to(v_cache.dtype)
 
     # -- attention over the paged cache -------------------------------------------------
-    def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens, max_q_len, max_kv_len, scale, window, all_decode, workspace):
+    def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens, max_q_len, max_kv_len, scale, window, all_decode, workspace, splits=None):
         t = qkv.shape[0]
         group = num_heads // num_kv_heads
         q_all = qkv[:, : num_heads * head_dim].view(t, num_heads, head_dim)

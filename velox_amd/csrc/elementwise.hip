@@ -1,0 +1,187 @@
+// Memory-bound kernels of the decoder step for gfx950: embedding gather, residual-add + RMSNorm,
+// SiLU(gate) * up, and the fused bias + rotary + cache write.  All arithmetic is float32; values
+// are rounded once, at the store.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------------
+// embedding: out[t, :] = float(table[ids[t], :]); an id outside the table yields NaN rows.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out, int hidden, int vocab) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  float* dst = out + (size_t)t * hidden;
+  if (id < 0 || id >= vocab) {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = __builtin_nanf("");
+    return;
+  }
+  const T* src = table + (size_t)id * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32(src[i]);
+}
+
+extern "C" int velox_embed(const int* ids, const void* table, float* out, int tokens, int hidden, int vocab, int table_dtype, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (table_dtype == VELOX_BF16)
+    embed_kernel<bf16_t><<<tokens, 256, 0, stream>>>(ids, (const bf16_t*)table, out, hidden, vocab);
+  else
+    embed_kernel<float><<<tokens, 256, 0, stream>>>(ids, (const float*)table, out, hidden, vocab);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// residual add + RMSNorm.  One block per output row.
+//   rows == nullptr: r = residual[row] (+ delta[row]); residual[row] = r; out[row] = norm(r)
+//   rows != nullptr: r = residual[rows[row]] (+ delta[rows[row]]); out[row] = norm(r); nothing else is written
+//   norm(r) = r * rsqrt(sum(r^2) / H + eps) * w
+// ---------------------------------------------------------------------------------------------
+template <typename TD, typename TO>
+__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta, const int* __restrict__ rows,
+                                   const float* __restrict__ weight, TO* __restrict__ out, int hidden, float eps) {
+  __shared__ float scratch[16];
+  const int row = blockIdx.x;
+  const size_t src_row = rows ? (size_t)rows[row] : (size_t)row;
+  float* res = residual + src_row * hidden;
+  const TD* del = delta ? delta + src_row * hidden : nullptr;
+  const bool write_back = (rows == nullptr) && (delta != nullptr);
+  float sumsq = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float r = res[i];
+    if (del) r += to_f32(del[i]);
+    if (write_back) res[i] = r;
+    sumsq += r * r;
+  }
+  const float total = block_sum(sumsq, scratch);
+  const float inv = rsqrtf(total / (float)hidden + eps);
+  TO* dst = out + (size_t)row * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float r = res[i];
+    if (del && !write_back) r += to_f32(del[i]);
+    dst[i] = from_f32<TO>(r * inv * weight[i]);
+  }
+}
+
+extern "C" int velox_add_rmsnorm(float* residual, const void* delta, const int* rows, const float* weight, void* out,
+                                 int num_rows, int hidden, float eps, int delta_dtype, int out_dtype, hipStream_t stream) {
+  if (num_rows <= 0) return 0;
+  const int threads = hidden >= 2048 ? 512 : 256;
+#define LAUNCH(TD, TO) add_rmsnorm_kernel<TD, TO><<<num_rows, threads, 0, stream>>>(residual, (const TD*)delta, rows, weight, (TO*)out, hidden, eps)
+  if (delta_dtype == VELOX_BF16 && out_dtype == VELOX_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (delta_dtype == VELOX_F32 && out_dtype == VELOX_F32) LAUNCH(float, float);
+  else if (delta_dtype == VELOX_BF16 && out_dtype == VELOX_F32) LAUNCH(bf16_t, float);
+  else LAUNCH(float, bf16_t);
+#undef LAUNCH
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[t, i] = silu(gate_up[t, i]) * gate_up[t, inter + i], silu(x) = x / (1 + exp(-x))
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter) {
+  const int t = blockIdx.y;
+  const T* row = gate_up + (size_t)t * 2 * inter;
+  T* dst = out + (size_t)t * inter;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < inter; i += gridDim.x * blockDim.x) {
+    const float g = to_f32(row[i]);
+    const float u = to_f32(row[inter + i]);
+    dst[i] = from_f32<T>(g / (1.f + expf(-g)) * u);
+  }
+}
+
+extern "C" int velox_silu_mul(const void* gate_up, void* out, int tokens, int inter, int dtype, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  int bx = (inter + 255) / 256;
+  if (bx > 64) bx = 64;
+  dim3 grid(bx, tokens);
+  if (dtype == VELOX_BF16) silu_mul_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, inter);
+  else silu_mul_kernel<float><<<grid, 256, 0, stream>>>((const float*)gate_up, (float*)out, inter);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// bias + rotary + cache write, one block per token.
+//   qkv[t] = [q (nh*d) | k (nkv*d) | v (nkv*d)], optional float32 bias of the same width.
+//   q: q += bias; rotate; stored back in place.
+//   k: k += bias; rotate; stored to k_cache[page, kv_head, offset, :]
+//   v: v += bias;          stored to v_cache[page, kv_head, :, offset]
+//   rotation of the first 2*half channels of a head, halves paired (i, i + half):
+//     lo' = lo*cos - hi*sin, hi' = lo*sin + hi*cos, cos/sin = table[position[t], i]
+//   slot = page * page_size + offset.  With write_kv == 0 only q is touched.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restrict__ bias, const int* __restrict__ positions,
+                                     const float* __restrict__ cos_table, const float* __restrict__ sin_table, int half,
+                                     const int* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                     int nh, int nkv, int d, int page_size, int write_kv) {
+  const int t = blockIdx.x;
+  const int width = (nh + 2 * nkv) * d;
+  T* row = qkv + (size_t)t * width;
+  const int pos = positions[t];
+  const float* cs = cos_table ? cos_table + (size_t)pos * half : nullptr;
+  const float* sn = sin_table ? sin_table + (size_t)pos * half : nullptr;
+  const int slot = slots[t];
+  const size_t page = (size_t)(slot / page_size);
+  const int offset = slot % page_size;
+  const int half_d = d / 2;  // work items per head: pairs (i, i + d/2) so every channel is visited once
+
+  const int q_items = nh * half_d;
+  const int k_items = write_kv ? nkv * half_d : 0;
+  for (int item = threadIdx.x; item < q_items + k_items; item += blockDim.x) {
+    const bool is_k = item >= q_items;
+    const int local = is_k ? item - q_items : item;
+    const int head = local / half_d;
+    const int i = local % half_d;
+    const int base = (is_k ? nh * d : 0) + head * d;
+    // the two channels this item owns
+    int c0, c1;
+    bool rotate;
+    if (cs != nullptr && i < half) { c0 = i; c1 = i + half; rotate = true; }
+    else {
+      // channels outside the rotated span are handled in pairs of their own so that all d are covered
+      // rotated span is [0, 2*half); the remaining d - 2*half channels are split over items i >= half
+      const int rest = (cs != nullptr) ? 2 * half : 0;
+      const int j = (cs != nullptr) ? i - half : i;
+      c0 = rest + 2 * j; c1 = c0 + 1; rotate = false;
+    }
+    float x0 = to_f32(row[base + c0]);
+    float x1 = to_f32(row[base + c1]);
+    if (bias) { x0 += bias[base + c0]; x1 += bias[base + c1]; }
+    float y0 = x0, y1 = x1;
+    if (rotate) {
+      const float c = cs[i], s = sn[i];
+      y0 = x0 * c - x1 * s;
+      y1 = x0 * s + x1 * c;
+    }
+    if (!is_k) {
+      row[base + c0] = from_f32<T>(y0);
+      row[base + c1] = from_f32<T>(y1);
+    } else {
+      T* dst = k_cache + ((page * nkv + head) * page_size + offset) * d;
+      dst[c0] = from_f32<T>(y0);
+      dst[c1] = from_f32<T>(y1);
+    }
+  }
+  if (write_kv) {
+    const int v_base = (nh + nkv) * d;
+    for (int item = threadIdx.x; item < nkv * d; item += blockDim.x) {
+      const int head = item / d;
+      const int c = item % d;
+      float x = to_f32(row[v_base + item]);
+      if (bias) x += bias[v_base + item];
+      v_cache[((page * nkv + head) * d + c) * page_size + offset] = from_f32<T>(x);
+    }
+  }
+}
+
+extern "C" int velox_rope_kv_write(void* qkv, const float* bias, const int* positions, const float* cos_table, const float* sin_table,
+                                   int half, const int* slots, void* k_cache, void* v_cache, int tokens, int nh, int nkv, int d,
+                                   int page_size, int write_kv, int dtype, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (dtype == VELOX_BF16)
+    rope_kv_write_kernel<bf16_t><<<tokens, 256, 0, stream>>>((bf16_t*)qkv, bias, positions, cos_table, sin_table, half, slots,
+                                                            (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, page_size, write_kv);
+  else
+    rope_kv_write_kernel<float><<<tokens, 256, 0, stream>>>((float*)qkv, bias, positions, cos_table, sin_table, half, slots,
+                                                           (float*)k_cache, (float*)v_cache, nh, nkv, d, page_size, write_kv);
+  VELOX_RETURN_LAUNCH_STATUS();
+}

@@ -1,0 +1,299 @@
+"""Python face of the HIP kernels: shape and dtype checks on the host, then a C call on the current stream.
+
+Every kernel the model calls goes through one method of :class:`HipOps`.  The methods check
+what the kernels and their launch grids assume (devices, dtypes, contiguity, alignment, sizes)
+before launching, because a kernel that reads out of bounds takes the whole GPU down.  There
+is no fallback: without a GPU, without hipcc or without the libraries, loading fails.
+
+Matrix products: a float32 run uses the exact FMA kernel (``gemm.hip``); so does any operand mix
+a library has no call for.  bfloat16 x bfloat16 products go to the library behind
+``torch.nn.functional.linear`` (hipBLASLt), as the reference uses cuBLAS through ``nn.Linear``
+(reference ``src/self_attention.py:48,90``, ``src/mlp.py:13,15``).
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Dict, Optional
+
+import torch
+
+from . import build
+
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+_F = ctypes.c_float
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype not in _DTYPE_CODE:
+        raise KernelError(f"kernels take float32 or bfloat16, got {dtype}")
+    return _DTYPE_CODE[dtype]
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return _P(0) if t is None else _P(t.data_ptr())
+
+
+class HipOps:
+    name = "hip-gfx950"
+
+    def __init__(self, device) -> None:
+        self.device = torch.device(device)
+        if self.device.type != "cuda" or not torch.cuda.is_available():
+            raise KernelError("the HIP kernels need a GPU (device 'cuda'); there is no CPU path")
+        if self.device.index is None:
+            self.device = torch.device("cuda", torch.cuda.current_device())
+        arch = torch.cuda.get_device_properties(self.device).gcnArchName.split(":")[0]
+        if arch != build.ARCH:
+            raise KernelError(f"the kernels are built for {build.ARCH}; this GPU is {arch}")
+        self._core = ctypes.CDLL(build.ensure_core())
+        self._attention: Dict[int, ctypes.CDLL] = {}
+        self._declare_core()
+        self.num_cus = torch.cuda.get_device_properties(self.device).multi_processor_count
+        self.use_library_gemm = True
+        self._mm_out_dtype_ok: Optional[bool] = None
+
+    # -- loading --------------------------------------------------------------------------------
+    def _declare_core(self) -> None:
+        c = self._core
+        c.velox_embed.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
+        c.velox_add_rmsnorm.argtypes = [_P, _P, _P, _P, _P, _I, _I, _F, _I, _I, _P]
+        c.velox_silu_mul.argtypes = [_P, _P, _I, _I, _I, _P]
+        c.velox_rope_kv_write.argtypes = [_P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_gemm_fma.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_argmax.argtypes = [_P, _P, _I, _I, _P]
+        c.velox_sample.argtypes = [_P, _P, _P, _I, _I, _P]
+        c.velox_apply_penalties.argtypes = [_P, _P, _P, _P, _I, _I, _I, _P]
+        for fn in (c.velox_embed, c.velox_add_rmsnorm, c.velox_silu_mul, c.velox_rope_kv_write, c.velox_gemm_fma,
+                   c.velox_argmax, c.velox_sample, c.velox_apply_penalties):
+            fn.restype = _I
+
+    def attention_library(self, head_dim: int) -> ctypes.CDLL:
+        lib = self._attention.get(head_dim)
+        if lib is None:
+            lib = ctypes.CDLL(build.ensure_attention(head_dim))
+            lib.velox_paged_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P]
+            lib.velox_paged_attention.restype = _I
+            lib.velox_attention_head_dim.restype = _I
+            if lib.velox_attention_head_dim() != head_dim:
+                raise KernelError(f"attention library for head_dim={head_dim} reports {lib.velox_attention_head_dim()}")
+            self._attention[head_dim] = lib
+        return lib
+
+    def prepare(self, model, dtype) -> None:
+        """Builds (at first use) and loads what this model's mixers need."""
+        for need in model.cache_needs():
+            if need is not None and hasattr(need, "head_dim"):
+                self.attention_library(need.head_dim)
+
+    # -- helpers --------------------------------------------------------------------------------
+    def _stream(self):
+        return _P(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def _check(self, name: str, t: torch.Tensor, dtype=None, shape=None, align: int = 4) -> None:
+        if not isinstance(t, torch.Tensor) or t.device != self.device:
+            raise KernelError(f"{name}: expected a tensor on {self.device}, got {getattr(t, 'device', type(t))}")
+        if not t.is_contiguous():
+            raise KernelError(f"{name}: must be contiguous (shape {tuple(t.shape)}, strides {t.stride()})")
+        if dtype is not None and t.dtype != dtype:
+            raise KernelError(f"{name}: expected {dtype}, got {t.dtype}")
+        if shape is not None and tuple(t.shape) != tuple(shape):
+            raise KernelError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
+        if t.data_ptr() % align != 0:
+            raise KernelError(f"{name}: address must be a multiple of {align}")
+
+    @staticmethod
+    def _launched(status: int, what: str) -> None:
+        if status != 0:
+            raise KernelError(f"{what}: launch failed with HIP error {status}")
+
+    # -- embedding and norms ----------------------------------------------------------------------
+    def embed(self, token_ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+        self._check("token_ids", token_ids, torch.int32)
+        self._check("table", table)
+        if token_ids.dim() != 1 or table.dim() != 2:
+            raise KernelError("embed: token_ids must be [T] and the table [V, H]")
+        vocab, hidden = table.shape
+        out = torch.empty((token_ids.shape[0], hidden), dtype=torch.float32, device=self.device)
+        status = self._core.velox_embed(_ptr(token_ids), _ptr(table), _ptr(out), token_ids.shape[0], hidden, vocab, _code(table.dtype), self._stream())
+        self._launched(status, "embed")
+        return out
+
+    def _norm(self, residual, delta, rows, weight, eps, out_dtype):
+        self._check("residual", residual, torch.float32)
+        if residual.dim() != 2:
+            raise KernelError("add_rmsnorm: residual must be [T, H]")
+        tokens, hidden = residual.shape
+        self._check("weight", weight, torch.float32, (hidden,))
+        if delta is not None:
+            self._check("delta", delta, None, (tokens, hidden))
+        if rows is not None:
+            self._check("rows", rows, torch.int32)
+            count = rows.shape[0]
+        else:
+            count = tokens
+        out = torch.empty((count, hidden), dtype=out_dtype, device=self.device)
+        delta_code = _code(delta.dtype) if delta is not None else _code(out_dtype)
+        status = self._core.velox_add_rmsnorm(_ptr(residual), _ptr(delta), _ptr(rows), _ptr(weight), _ptr(out), count, hidden, float(eps), delta_code, _code(out_dtype), self._stream())
+        self._launched(status, "add_rmsnorm")
+        return out
+
+    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype):
+        return self._norm(residual, delta, None, weight, eps, out_dtype)
+
+    def add_rmsnorm_rows(self, residual, delta, rows, weight, eps, out_dtype):
+        return self._norm(residual, delta, rows, weight, eps, out_dtype)
+
+    # -- matrix products --------------------------------------------------------------------------
+    def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype) -> torch.Tensor:
+        self._check("x", x, align=16)
+        self._check("weight", weight, align=16)
+        if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
+            raise KernelError(f"linear: x {tuple(x.shape)} and weight {tuple(weight.shape)} do not match")
+        m, k = x.shape
+        n = weight.shape[0]
+        if bias is not None:
+            self._check("bias", bias, torch.float32, (n,))
+        if self.use_library_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and bias is None:
+            if out_dtype == torch.bfloat16:
+                return torch.nn.functional.linear(x, weight)
+            if out_dtype == torch.float32 and self._mm_out_dtype_ok is not False:
+                try:
+                    out = torch.mm(x, weight.t(), out_dtype=torch.float32)
+                    self._mm_out_dtype_ok = True
+                    return out
+                except (RuntimeError, TypeError):
+                    self._mm_out_dtype_ok = False
+        return self.gemm_fma(x, weight, bias, out_dtype)
+
+    def gemm_fma(self, x, weight, bias, out_dtype):
+        m, k = x.shape
+        n = weight.shape[0]
+        out = torch.empty((m, n), dtype=out_dtype, device=self.device)
+        status = self._core.velox_gemm_fma(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), m, n, k, _code(x.dtype), _code(weight.dtype), _code(out_dtype), self._stream())
+        self._launched(status, "gemm_fma")
+        return out
+
+    def silu_mul(self, gate_up: torch.Tensor) -> torch.Tensor:
+        self._check("gate_up", gate_up)
+        if gate_up.dim() != 2 or gate_up.shape[1] % 2 != 0:
+            raise KernelError("silu_mul: expected [T, 2 * intermediate]")
+        tokens, inter = gate_up.shape[0], gate_up.shape[1] // 2
+        out = torch.empty((tokens, inter), dtype=gate_up.dtype, device=self.device)
+        status = self._core.velox_silu_mul(_ptr(gate_up), _ptr(out), tokens, inter, _code(gate_up.dtype), self._stream())
+        self._launched(status, "silu_mul")
+        return out
+
+    # -- rotary + cache write ---------------------------------------------------------------------
+    def rope_kv_write(self, qkv, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size, write_kv=True, bias=None):
+        tokens = qkv.shape[0]
+        width = (num_heads + 2 * num_kv_heads) * head_dim
+        self._check("qkv", qkv, None, (tokens, width), align=16)
+        self._check("positions", positions, torch.int32, (tokens,))
+        self._check("slot_mapping", slot_mapping, torch.int32, (tokens,))
+        if bias is not None:
+            self._check("bias", bias, torch.float32, (width,))
+        half = 0
+        if cos is not None:
+            self._check("cos", cos, torch.float32)
+            self._check("sin", sin, torch.float32, tuple(cos.shape))
+            half = cos.shape[1]
+            if 2 * half > head_dim:
+                raise KernelError(f"rotary span {2 * half} exceeds head_dim {head_dim}")
+        pages = k_cache.shape[0]
+        self._check("k_cache", k_cache, qkv.dtype, (pages, num_kv_heads, block_size, head_dim), align=16)
+        self._check("v_cache", v_cache, qkv.dtype, (pages, num_kv_heads, head_dim, block_size), align=16)
+        # positions index the tables and slots index the cache: both are built by the batch builder from
+        # block tables the cache manager handed out, bounded by max_model_len and the pool size
+        status = self._core.velox_rope_kv_write(
+            _ptr(qkv), _ptr(bias), _ptr(positions), _ptr(cos), _ptr(sin), half, _ptr(slot_mapping), _ptr(k_cache), _ptr(v_cache),
+            tokens, num_heads, num_kv_heads, head_dim, block_size, 1 if write_kv else 0, _code(qkv.dtype), self._stream())
+        self._launched(status, "rope_kv_write")
+
+    # -- attention ------------------------------------------------------------------------------
+    def choose_splits(self, num_seqs: int, num_kv_heads: int, row_tiles: int, max_kv_len: int, all_decode: bool) -> int:
+        """Splits of the key range for an all-decode step (reference ``src/decode_attention.py:237-252``:
+        enough workgroups to fill the GPU, at least 128 keys each)."""
+        if not all_decode:
+            return 1
+        base = num_seqs * num_kv_heads * row_tiles
+        target = 2 * self.num_cus
+        if base >= target or max_kv_len < 256:
+            return 1
+        wanted = (target + base - 1) // base
+        return max(1, min(wanted, 32, max_kv_len // 128))
+
+    def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens,
+                        max_q_len, max_kv_len, scale, window, all_decode, workspace, splits: Optional[int] = None):
+        tokens = qkv.shape[0]
+        width = (num_heads + 2 * num_kv_heads) * head_dim
+        self._check("qkv", qkv, None, (tokens, width), align=16)
+        num_seqs = kv_lens.shape[0]
+        self._check("kv_lens", kv_lens, torch.int32, (num_seqs,))
+        self._check("cu_q", cu_q, torch.int32, (num_seqs + 1,))
+        self._check("block_tables", block_tables, torch.int32)
+        if block_tables.dim() != 2 or block_tables.shape[0] != num_seqs:
+            raise KernelError(f"block_tables must be [{num_seqs}, W], got {tuple(block_tables.shape)}")
+        if block_size <= 0 or block_size & (block_size - 1):
+            raise KernelError(f"block_size must be a power of two, got {block_size}")
+        if block_tables.shape[1] * block_size < max_kv_len:
+            raise KernelError(f"block tables of width {block_tables.shape[1]} cannot cover {max_kv_len} keys")
+        pages = k_cache.shape[0]
+        self._check("k_cache", k_cache, qkv.dtype, (pages, num_kv_heads, block_size, head_dim), align=16)
+        self._check("v_cache", v_cache, qkv.dtype, (pages, num_kv_heads, head_dim, block_size), align=16)
+        if num_heads % num_kv_heads != 0:
+            raise KernelError("num_heads must be a multiple of num_kv_heads")
+        if max_q_len < 1 or max_q_len > tokens:
+            raise KernelError(f"max_q_len={max_q_len} outside [1, {tokens}]")
+        lib = self.attention_library(head_dim)
+        group = num_heads // num_kv_heads
+        row_tiles = (max_q_len * group + 63) // 64
+        if splits is None:
+            splits = self.choose_splits(num_seqs, num_kv_heads, row_tiles, max_kv_len, all_decode)
+        if num_seqs * splits > 65535:
+            raise KernelError(f"{num_seqs} sequences x {splits} splits exceed the launch grid")
+        out = torch.empty((tokens, num_heads * head_dim), dtype=qkv.dtype, device=self.device)
+        part_o = part_lse = None
+        if splits > 1:
+            if workspace is None:
+                raise KernelError("split attention needs a workspace")
+            part_o = workspace.get("attention_partial_out", splits * tokens * num_heads * head_dim)
+            part_lse = workspace.get("attention_partial_lse", splits * tokens * num_heads)
+        status = lib.velox_paged_attention(
+            _ptr(qkv), width, _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), block_tables.shape[1], _ptr(cu_q), _ptr(kv_lens),
+            _ptr(out), _ptr(part_o), _ptr(part_lse), num_seqs, tokens, max_q_len, num_heads, num_kv_heads,
+            block_size.bit_length() - 1, float(scale), int(window or 0), splits, _code(qkv.dtype), self._stream())
+        self._launched(status, "paged_attention")
+        return out
+
+    # -- sampling -------------------------------------------------------------------------------
+    def argmax(self, logits: torch.Tensor) -> torch.Tensor:
+        self._check("logits", logits, torch.float32)
+        rows, vocab = logits.shape
+        out = torch.empty(rows, dtype=torch.int32, device=self.device)
+        self._launched(self._core.velox_argmax(_ptr(logits), _ptr(out), rows, vocab, self._stream()), "argmax")
+        return out
+
+    def sample(self, logits: torch.Tensor, options: torch.Tensor) -> torch.Tensor:
+        self._check("logits", logits, torch.float32)
+        rows, vocab = logits.shape
+        self._check("options", options, torch.int32, (rows, 6))
+        out = torch.empty(rows, dtype=torch.int32, device=self.device)
+        self._launched(self._core.velox_sample(_ptr(logits), _ptr(options), _ptr(out), rows, vocab, self._stream()), "sample")
+        return out
+
+    def apply_penalties(self, logits, tokens, lengths, coeffs) -> None:
+        self._check("logits", logits, torch.float32)
+        rows, vocab = logits.shape
+        self._check("tokens", tokens, torch.int32)
+        if tokens.dim() != 2 or tokens.shape[0] != rows:
+            raise KernelError("apply_penalties: tokens must be [rows, width]")
+        self._check("lengths", lengths, torch.int32, (rows,))
+        self._check("coeffs", coeffs, torch.float32, (rows, 3))
+        status = self._core.velox_apply_penalties(_ptr(logits), _ptr(tokens), _ptr(lengths), _ptr(coeffs), rows, vocab, tokens.shape[1], self._stream())
+        self._launched(status, "apply_penalties")

@@ -73,7 +73,8 @@ class AttentionMixer(Mixer):
 
     def forward(self, x, ctx, cache, owns_cache: bool = True):
         ops = ctx.ops
-        qkv = ops.linear(x, self.qkv_weight, self.qkv_bias_vec if self.qkv_bias else None, ctx.dtype)
+        # the bias is added (in float32) by the kernel that rotates and stores, which reads qkv anyway
+        qkv = ops.linear(x, self.qkv_weight, None, ctx.dtype)
         tables = self.position.rotary_tables() if self.position is not None else None
         cos, sin = tables if tables is not None else (None, None)
         meta = cache.batch
@@ -82,6 +83,7 @@ class AttentionMixer(Mixer):
             ctx.positions, cos, sin,
             meta.slot_mapping, cache.k, cache.v, cache.block_size,
             write_kv=owns_cache,
+            bias=self.qkv_bias_vec if self.qkv_bias else None,
         )
         attn = ops.paged_attention(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim,
