@@ -1,0 +1,210 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on one MI355X, as one JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
+
+A "step" is one decode step of the whole engine loop (scheduler, one forward over the batch,
+sampling, the host's read of the sampled tokens).  The default run has the layer sizes of
+Qwen2.5-7B with random weights N(0, 0.02), a batch of 8 and a context of 4096 tokens: the
+requests are prefilled through the engine so that they reach the context length at the last
+timed step.  ``value`` is decoded tokens per second.  The same line carries the prefill of one
+2,048-token prompt, the decode step's share of the HBM roofline, and decode at batch 1 and 64.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+PEAK_HBM_GBS = 8000.0
+SLACK = 512  # requests whose prompt is done first decode on while the others' prompts are still being read
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+QWEN25_7B = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "num_hidden_layers": 28, "hidden_size": 3584, "num_attention_heads": 28, "num_key_value_heads": 4,
+    "intermediate_size": 18944, "vocab_size": 152064, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": False, "use_sliding_window": False, "max_position_embeddings": 32768,
+}
+
+
+def linear_params_per_layer(c):
+    h, nh, nkv, inter = c["hidden_size"], c["num_attention_heads"], c["num_key_value_heads"], c["intermediate_size"]
+    d = c.get("head_dim") or h // nh
+    return h * (nh + 2 * nkv) * d + nh * d * h + 3 * h * inter
+
+
+def decode_bytes(c, layers, batch, context, elem):
+    """Bytes a decode step has to read: every weight it uses once, and the cache of the live requests."""
+    h, nh, nkv = c["hidden_size"], c["num_attention_heads"], c["num_key_value_heads"]
+    d = c.get("head_dim") or h // nh
+    per_layer = linear_params_per_layer(c) * elem + (nh + 2 * nkv) * d * 4 + 2 * h * 4
+    weights = layers * per_layer + c["vocab_size"] * h * elem + h * 4 + batch * h * elem
+    cache = batch * context * layers * 2 * nkv * d * elem
+    return weights + cache
+
+
+def prefill_flops(c, layers, tokens):
+    h, nh = c["hidden_size"], c["num_attention_heads"]
+    d = c.get("head_dim") or h // nh
+    linear = 2 * tokens * layers * linear_params_per_layer(c)
+    attention = layers * 2 * tokens * tokens * nh * d  # QK^T and PV over the causal half
+    head = 2 * h * c["vocab_size"]
+    return linear + attention + head
+
+
+def make_engine(model_config, dtype, batch, context, chunk, graphs, seed=0):
+    from velox_amd import Engine, EngineConfig
+
+    max_len = context + SLACK
+    pages = batch * ((max_len + 15) // 16 + 1) + (chunk + 15) // 16 + 64
+    return Engine.from_random(
+        model_config, seed,
+        EngineConfig(dtype=dtype, device="cuda:0", max_model_len=max_len, max_num_seqs=batch,
+                     max_num_batched_tokens=max(chunk, batch), max_prefill_chunk_size=chunk, block_size=16,
+                     num_gpu_blocks=pages, enable_cuda_graphs=graphs, seed=seed),
+        generator_device="cuda",
+    )
+
+
+def time_decode(engine, vocab, batch, context, steps, warmup, seed=0):
+    """Reads ``batch`` prompts in through the engine, then times ``steps`` steps in which every request decodes.
+    Every request holds at least ``context`` tokens at the last timed step (those admitted first a few more).
+    Returns (seconds per step, mean tokens in the cache per request over the timed steps)."""
+    import random
+
+    import torch
+
+    from velox_amd import Request, SamplingParams
+    from velox_amd.engine.request import RequestStatus
+
+    rng = random.Random(seed)
+    prompt_len = max(1, context - steps - warmup)
+    requests = [
+        Request(f"decode-{batch}-{i}", [rng.randrange(vocab) for _ in range(prompt_len)],
+                SamplingParams(temperature=0.0, max_tokens=steps + warmup + SLACK - 1, ignore_eos=True))
+        for i in range(batch)
+    ]
+    for request in requests:
+        engine.add_request(request)
+    while any(r.status is not RequestStatus.RUNNING_DECODE for r in requests):
+        engine.step()
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    before = [len(r.output_token_ids) for r in requests]
+    held = sum(r.num_computed_tokens for r in requests)
+    start = time.perf_counter()
+    for _ in range(steps):
+        engine.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - start
+    assert all(len(r.output_token_ids) == n + steps for r, n in zip(requests, before)), "a timed step did not decode one token per request"
+    mean_context = (held / batch) + (steps + 1) / 2
+    for request in requests:
+        engine.abort_request(request.request_id)
+    return elapsed / steps, mean_context
+
+
+def time_prefill(engine, vocab, tokens, repeats=3, seed=1):
+    import random
+
+    import torch
+
+    from velox_amd import Request, SamplingParams
+
+    rng = random.Random(seed)
+    best = None
+    for attempt in range(repeats + 1):
+        request = Request(f"prefill-{attempt}", [rng.randrange(vocab) for _ in range(tokens)],
+                          SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True))
+        engine.add_request(request)
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        engine.step()  # the whole prompt in one step, logits of the last row, one sampled token
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - start
+        assert len(request.output_token_ids) == 1, "the prompt did not prefill in one step"
+        engine.step()  # reaps the finished request
+        if attempt > 0:
+            best = elapsed if best is None else min(best, elapsed)
+    return best
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=64)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (both numbers are reported)")
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--context", type=int, default=4096)
+    parser.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    parser.add_argument("--prefill-tokens", type=int, default=2048)
+    parser.add_argument("--no-graphs", action="store_true")
+    parser.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine (single-GPU tier)")
+        return 2
+
+    import torch
+
+    model_config = dict(QWEN25_7B)
+    full_layers = model_config["num_hidden_layers"]
+    layers = args.layers or full_layers
+    model_config["num_hidden_layers"] = layers
+    elem = 2 if args.dtype == "bf16" else 4
+    vocab = model_config["vocab_size"]
+    graphs = not args.no_graphs
+    batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
+
+    engine = make_engine(model_config, args.dtype, max(batches), args.context, args.prefill_tokens, graphs)
+    step_s, contexts = {}, {}
+    for batch in batches:
+        steps = args.steps if batch == args.batch else max(8, args.steps // 2)
+        step_s[batch], contexts[batch] = time_decode(engine, vocab, batch, args.context, steps, args.warmup)
+    prefill_s = time_prefill(engine, vocab, args.prefill_tokens)
+
+    main_step = step_s[args.batch]
+    bytes_read = decode_bytes(model_config, layers, args.batch, contexts[args.batch], elem)
+    achieved = bytes_read / main_step / 1e9
+    flops = prefill_flops(model_config, layers, args.prefill_tokens)
+    result = {
+        "metric": "decode_tokens_per_second",
+        "value": round(args.batch / main_step, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(main_step * 1000, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": args.dtype,
+        "data": "synthetic: random weights N(0,0.02), uniform random token ids",
+        "config": {
+            "model": "Qwen2.5-7B shape", "layers": layers, "layers_full": full_layers,
+            "hidden": model_config["hidden_size"], "heads": model_config["num_attention_heads"],
+            "kv_heads": model_config["num_key_value_heads"], "head_dim": model_config["hidden_size"] // model_config["num_attention_heads"],
+            "intermediate": model_config["intermediate_size"], "vocab": vocab,
+            "global_batch": args.batch, "seq_len": args.context, "mean_context": round(contexts[args.batch], 1), "page_size": 16,
+            "prefill_tokens": args.prefill_tokens, "hip_graphs": graphs, "parallelism": "single-gpu",
+        },
+        "prefill": {
+            "value": round(args.prefill_tokens / prefill_s, 1), "tokens": args.prefill_tokens,
+            "ms": round(prefill_s * 1000, 3), "frac": round(flops / prefill_s / PEAK_FLOPS[args.dtype], 4),
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": round(achieved / PEAK_HBM_GBS, 4),
+        },
+        "points": {f"decode_b{b}": round(b / s, 2) for b, s in step_s.items() if b != args.batch},
+    }
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
