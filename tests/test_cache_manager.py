@@ -1,0 +1,140 @@
+"""Page allocator, page groups, windows and state slots: no page lost, held twice or freed twice."""
+import random
+
+import pytest
+import torch
+
+from velox_amd.cache import NULL_PAGE, CacheManager, OutOfPagesError, PageAllocator
+from velox_amd.parts.base import PagedNeed, StateNeed
+
+
+def test_allocator_order_and_errors():
+    a = PageAllocator(6)
+    assert [a.allocate() for _ in range(3)] == [1, 2, 3]  # page 0 is never handed out
+    a.free(2)
+    assert a.allocate() == 2  # the page freed last is used again first
+    assert a.allocate_many(2) == [4, 5]
+    with pytest.raises(OutOfPagesError):
+        a.allocate()
+    with pytest.raises(OutOfPagesError):
+        a.allocate_many(1)
+    a.free(4)
+    with pytest.raises(RuntimeError):
+        a.free(4)  # freed twice
+    with pytest.raises(RuntimeError):
+        a.incref(4)  # free page
+    a.incref(1)
+    assert a.free(1) == 1 and a.num_free == 1
+    assert a.free(NULL_PAGE) == 1  # the reserved page stays
+    with pytest.raises(IndexError):
+        a.free(6)
+    with pytest.raises(ValueError):
+        PageAllocator(1)
+    a.assert_consistent()
+
+
+def _manager(needs, pages=9, page=4, seqs=4, max_len=None):
+    return CacheManager(needs, page, pages, seqs, torch.float32, "cpu", max_model_len=max_len)
+
+
+def test_growth_and_release():
+    need = PagedNeed(2, 16)
+    m = _manager([need, need, need])
+    assert len(m.groups) == 1 and m.groups[0].keys.shape == (3, 9, 2, 4, 16) and m.groups[0].values.shape == (3, 9, 2, 16, 4)
+    assert m.max_model_len == 32
+    s = m.new_sequence()
+    assert m.append(s, 0, 5) and s.tables[0] == [1, 2]
+    assert m.append(s, 5, 3) and s.tables[0] == [1, 2]  # 8 tokens still fit two pages
+    assert m.append(s, 8, 1) and s.tables[0] == [1, 2, 3]
+    assert m.slot_for(s, 0, 6) == 2 * 4 + 2
+    t = m.new_sequence()
+    assert not m.append(t, 0, 21) and t.tables[0] == []  # all or nothing
+    assert m.append(t, 0, 20) and m.num_free_pages() == 0
+    assert not m.can_append(s, 9, 4) and m.can_append(s, 9, 3)
+    assert not m.append(s, 9, 100)  # beyond max_model_len
+    m.assert_consistent([s, t])
+    m.free_sequence(t)
+    assert m.num_free_pages() == 5
+    u = m.new_sequence()
+    assert m.append(u, 0, 1) and u.tables[0] == [8]  # the page freed last is handed out first
+    m.free_sequence(s)
+    m.free_sequence(u)
+    m.assert_consistent([])
+    assert m.num_used_pages() == 0 and m.state.num_free == 4
+
+
+def test_groups_by_need_and_window_release():
+    full = PagedNeed(2, 16)
+    windowed = PagedNeed(2, 16, window=6)
+    m = _manager([full, windowed, full, windowed, None], pages=12)
+    assert len(m.groups) == 2 and m.entry_group[0] == (0, 0) and m.entry_group[2] == (0, 1) and m.entry_group[3] == (1, 1)
+    s = m.new_sequence()
+    assert m.append(s, 0, 10)
+    assert s.tables == [[1, 2, 3], [1, 2, 3]]  # each group has pages of its own
+    assert m.release_behind_window(s, 10) == 1  # a query at 10 reads keys 5..: page 0 (keys 0..3) goes back
+    assert s.tables[1] == [NULL_PAGE, 2, 3] and s.tables[0] == [1, 2, 3]
+    assert m.groups[1].allocator.num_free == 9 and m.groups[0].allocator.num_free == 8
+    assert m.append(s, 10, 7)  # 17 tokens: 5 entries
+    assert s.tables[1][3] == 1  # the page given back is used again, by the same request
+    assert m.release_behind_window(s, 17) == 2  # keys 12.. are needed: pages 1 and 2 go back
+    assert m.release_behind_window(s, 17) == 0
+    m.assert_consistent([s])
+    m.free_sequence(s)
+    m.assert_consistent([])
+    assert all(g.allocator.num_used == 0 for g in m.groups)
+
+
+def test_state_slots_are_zeroed_on_take():
+    need = StateNeed((("sum", (3,), torch.float32), ("count", (), None)))
+    m = _manager([PagedNeed(1, 16), need], seqs=2)
+    a, b = m.new_sequence(), m.new_sequence()
+    assert m.new_sequence() is None and {a.slot, b.slot} == {0, 1}
+    view = m.view(1, [None])
+    assert view.tensors["sum"].shape == (3, 3) and view.tensors["count"].shape == (3,)  # one spare row for padding
+    view.tensors["sum"][a.slot] = 7.0
+    m.free_sequence(a)
+    with pytest.raises(RuntimeError):
+        m.state.release(a.slot if a.slot >= 0 else 0 if b.slot != 0 else 1)
+    c = m.new_sequence()
+    assert float(view.tensors["sum"][c.slot].abs().sum()) == 0.0
+    m.free_sequence(b)
+    m.free_sequence(c)
+    m.assert_consistent([])
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_of_requests(seed):
+    rng = random.Random(seed)
+    windowed = seed % 2 == 1
+    needs = [PagedNeed(1, 16), PagedNeed(1, 16, window=9) if windowed else PagedNeed(1, 16)]
+    m = _manager(needs, pages=14, page=4, seqs=5)
+    live = {}
+    for step in range(600):
+        action = rng.random()
+        if action < 0.25 and len(live) < 5:
+            seq = m.new_sequence()
+            assert seq is not None
+            live[step] = [seq, 0]
+        elif action < 0.85 and live:
+            key = rng.choice(list(live))
+            seq, computed = live[key]
+            n = rng.choice([1, 1, 1, 2, 5, 7, 13])
+            before = [list(t) for t in seq.tables]
+            if m.append(seq, computed, n):
+                live[key][1] = computed + n
+                m.release_behind_window(seq, computed + n)
+            else:
+                assert [list(t) for t in seq.tables] == before  # a refused growth changes nothing
+        elif live:
+            key = rng.choice(list(live))
+            m.free_sequence(live.pop(key)[0])
+        m.assert_consistent([s for s, _ in live.values()])
+        for seq, computed in live.values():
+            for g, group in enumerate(m.groups):
+                first = group.first_needed_page(computed)
+                for index in range(first, group.table_entries_for(computed)):
+                    assert seq.tables[g][index] != NULL_PAGE  # every page a query may read is held
+    for seq, _ in live.values():
+        m.free_sequence(seq)
+    m.assert_consistent([])
+    assert m.num_used_pages() == 0 and m.state.num_free == 5

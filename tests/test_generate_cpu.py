@@ -1,0 +1,98 @@
+"""Generation through the Python entry point on a CPU (plain references as kernels): scheduler, step
+function, sampler and request bookkeeping together."""
+import pytest
+import torch
+
+from helpers import CONFIGS, PAGE_SIZE, make_folder, random_tokens
+from plain_qwen2 import qwen2_logits, read_model_folder
+from torch_ops import TorchOps
+from velox_amd import Engine, EngineConfig, Request, SamplingParams
+from velox_amd.engine.request import FinishReason
+
+
+def engine_for(folder, name, **overrides):
+    options = dict(model=folder, dtype="float32", device="cpu", max_model_len=128, max_num_seqs=4, max_num_batched_tokens=32,
+                   max_prefill_chunk_size=7, block_size=PAGE_SIZE[name], num_gpu_blocks=64, enable_cuda_graphs=False, seed=0)
+    options.update(overrides)
+    return Engine.from_pretrained(EngineConfig(**options), ops=TorchOps())
+
+
+def plain_greedy(config, weights, prompt, n):
+    tokens = list(prompt)
+    for _ in range(n):
+        tokens.append(int(qwen2_logits(config, weights, tokens)[-1].argmax()))
+    return tokens[len(prompt):]
+
+
+def greedy(prompts, n, prefix="r"):
+    return [Request(f"{prefix}{i}", p, SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True)) for i, p in enumerate(prompts)]
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_matches_plain_and_batched_equals_alone(tmp_path, name):
+    folder = make_folder(tmp_path, name)
+    config, weights = read_model_folder(folder)
+    prompts = [random_tokens(config["vocab_size"], n, seed=n) for n in (5, 9, 13, 22)]
+    engine = engine_for(folder, name)
+    together = engine.generate(greedy(prompts, 8))
+    for request, prompt in zip(together, prompts):
+        assert request.output_token_ids == plain_greedy(config, weights, prompt, 8)
+        assert request.finish_reason is FinishReason.LENGTH and len(request.output_token_ids) == 8
+    for i, prompt in enumerate(prompts):
+        alone = engine.generate(greedy([prompt], 8, prefix=f"alone{i}-"))[0]
+        assert alone.output_token_ids == together[i].output_token_ids
+    assert engine.cache.num_used_pages() == 0
+    engine.cache.assert_consistent([])
+    assert engine.snapshot()["num_finished"] == 8.0
+
+
+def test_preemption_does_not_change_the_tokens(tmp_path):
+    folder = make_folder(tmp_path, "B")
+    config, _ = read_model_folder(folder)
+    prompts = [random_tokens(config["vocab_size"], n, seed=40 + n) for n in (20, 31, 12, 25)]
+    roomy = engine_for(folder, "B", num_gpu_blocks=64).generate(greedy(prompts, 24))
+    tight_engine = engine_for(folder, "B", num_gpu_blocks=13, watermark=0.01)  # 12 pages of 8 for 4 x (up to 55) tokens
+    tight = tight_engine.generate(greedy(prompts, 24))
+    assert tight_engine.scheduler.num_preemptions > 0
+    for a, b in zip(roomy, tight):
+        assert a.output_token_ids == b.output_token_ids and len(b.output_token_ids) == 24
+    assert tight_engine.cache.num_used_pages() == 0
+    tight_engine.cache.assert_consistent([])
+
+
+def test_stop_tokens_and_limits(tmp_path):
+    folder = make_folder(tmp_path, "A")
+    config, weights = read_model_folder(folder)
+    prompt = random_tokens(256, 6, 2)
+    expected = plain_greedy(config, weights, prompt, 6)
+    engine = engine_for(folder, "A")
+    stop_at = expected[2]
+    request = Request("stop", prompt, SamplingParams(temperature=0.0, max_tokens=6, stop_token_ids=[stop_at]))
+    engine.generate([request])
+    cut = expected.index(stop_at) + 1
+    assert request.output_token_ids == expected[:cut] and request.finish_reason is FinishReason.STOP  # the stop token stays
+    with pytest.raises(ValueError):
+        engine.add_request(Request("big", [1] * 200, SamplingParams(max_tokens=1)))
+    with pytest.raises(ValueError):
+        engine.add_request(Request("oov", [1, 256], SamplingParams(max_tokens=1)))
+
+
+def test_seeded_sampling_is_independent_of_the_batch(tmp_path):
+    folder = make_folder(tmp_path, "B")
+    config, _ = read_model_folder(folder)
+    prompts = [random_tokens(config["vocab_size"], n, seed=70 + n) for n in (1, 17, 40, 8)]
+
+    def sampled(i, prompt):
+        return Request(f"s{i}", prompt, SamplingParams(temperature=0.8, max_tokens=6, seed=100 + i, ignore_eos=True))
+
+    engine = engine_for(folder, "B")
+    together = engine.generate([sampled(i, p) for i, p in enumerate(prompts)])
+    again = engine_for(folder, "B").generate([sampled(i, p) for i, p in enumerate(prompts)])
+    assert [r.output_token_ids for r in together] == [r.output_token_ids for r in again]
+    alone = engine.generate([sampled(2, prompts[2])])[0]
+    assert alone.output_token_ids == together[2].output_token_ids
+    # a greedy request keeps its tokens next to sampled ones
+    greedy_alone = engine.generate(greedy([prompts[1]], 6, prefix="g-alone"))[0]
+    mixed = engine.generate([sampled(7, prompts[0]), greedy([prompts[1]], 6, prefix="g-mixed")[0], sampled(8, prompts[3])])
+    assert mixed[1].output_token_ids == greedy_alone.output_token_ids
+    assert len({tuple(r.output_token_ids) for r in together}) > 1

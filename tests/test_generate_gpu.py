@@ -1,0 +1,106 @@
+"""Generation through the Python entry point on the GPU: greedy tokens against the plain model, batched equals
+alone, preemption, HIP-graph decode equals eager decode, sampling, and the command line."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from helpers import PAGE_SIZE, make_folder, random_tokens
+from plain_qwen2 import qwen2_logits, read_model_folder
+from velox_amd import Engine, EngineConfig, Request, SamplingParams
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def engine_for(folder, name, dtype="float32", **overrides):
+    options = dict(model=folder, dtype=dtype, device="cuda", max_model_len=160, max_num_seqs=4, max_num_batched_tokens=32,
+                   max_prefill_chunk_size=7, block_size=PAGE_SIZE[name], num_gpu_blocks=96, enable_cuda_graphs=False, seed=0)
+    options.update(overrides)
+    return Engine.from_pretrained(EngineConfig(**options))
+
+
+def plain_greedy(config, weights, prompt, n):
+    tokens = list(prompt)
+    for _ in range(n):
+        tokens.append(int(qwen2_logits(config, weights, tokens)[-1].argmax()))
+    return tokens[len(prompt):]
+
+
+def greedy(prompts, n, prefix="r"):
+    return [Request(f"{prefix}{i}", p, SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True)) for i, p in enumerate(prompts)]
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_matches_plain(tmp_path, name):
+    folder = make_folder(tmp_path, name)
+    config, weights = read_model_folder(folder)
+    prompts = [random_tokens(config["vocab_size"], n, seed=n) for n in (5, 9, 13, 40)]
+    engine = engine_for(folder, name)
+    together = engine.generate(greedy(prompts, 8))
+    for request, prompt in zip(together, prompts):
+        assert request.output_token_ids == plain_greedy(config, weights, prompt, 8)
+    for i, prompt in enumerate(prompts):
+        assert engine.generate(greedy([prompt], 8, prefix=f"alone{i}-"))[0].output_token_ids == together[i].output_token_ids
+    assert engine.cache.num_used_pages() == 0
+    engine.cache.assert_consistent([])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_decode_equals_eager_decode_and_preemption_keeps_tokens(tmp_path, dtype):
+    folder = make_folder(tmp_path, "B", "float32" if dtype == "float32" else "bfloat16")
+    config, _ = read_model_folder(folder)
+    prompts = [random_tokens(config["vocab_size"], n, seed=40 + n) for n in (20, 31, 12, 25)]
+    eager = engine_for(folder, "B", dtype).generate(greedy(prompts, 30))
+    graph_engine = engine_for(folder, "B", dtype, enable_cuda_graphs=True)
+    assert graph_engine.runner.uses_graphs
+    graphed = graph_engine.generate(greedy(prompts, 30))
+    assert graph_engine.runner.num_graph_replays > 20
+    assert [r.output_token_ids for r in graphed] == [r.output_token_ids for r in eager]
+    # a second round through the same graphs, with other requests in the same slots and pages
+    again = graph_engine.generate(greedy(list(reversed(prompts)), 30, prefix="again"))
+    assert [r.output_token_ids for r in again] == [r.output_token_ids for r in reversed(eager)]
+    tight_engine = engine_for(folder, "B", dtype, num_gpu_blocks=14, enable_cuda_graphs=True)
+    tight = tight_engine.generate(greedy(prompts, 30))
+    assert tight_engine.scheduler.num_preemptions > 0
+    assert [r.output_token_ids for r in tight] == [r.output_token_ids for r in eager]
+    assert tight_engine.cache.num_used_pages() == 0
+
+
+def test_sampling_through_the_engine(tmp_path):
+    folder = make_folder(tmp_path, "B")
+    config, _ = read_model_folder(folder)
+    prompts = [random_tokens(config["vocab_size"], n, seed=70 + n) for n in (1, 17, 40, 8)]
+
+    def sampled(i, prompt, **kw):
+        return Request(f"s{i}", prompt, SamplingParams(temperature=0.8, max_tokens=6, seed=100 + i, ignore_eos=True, **kw))
+
+    engine = engine_for(folder, "B")
+    together = engine.generate([sampled(i, p) for i, p in enumerate(prompts)])
+    again = engine_for(folder, "B").generate([sampled(i, p) for i, p in enumerate(prompts)])
+    assert [r.output_token_ids for r in together] == [r.output_token_ids for r in again]
+    assert engine.generate([sampled(2, prompts[2])])[0].output_token_ids == together[2].output_token_ids
+    greedy_alone = engine.generate(greedy([prompts[1]], 6, prefix="g-alone"))[0]
+    mixed = engine.generate([sampled(7, prompts[0]), greedy([prompts[1]], 6, prefix="g-mixed")[0], sampled(8, prompts[3], top_k=5, top_p=0.9)])
+    assert mixed[1].output_token_ids == greedy_alone.output_token_ids
+    top1 = engine.generate([Request("k1", prompts[1], SamplingParams(temperature=1.5, top_k=1, max_tokens=6, ignore_eos=True))])[0]
+    assert top1.output_token_ids == greedy_alone.output_token_ids
+    penalised = engine.generate([Request("pen", prompts[1], SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True, repetition_penalty=1.3, frequency_penalty=0.4))])[0]
+    assert len(penalised.output_token_ids) == 6
+
+
+def test_command_line(tmp_path):
+    folder = make_folder(tmp_path, "A", "bfloat16")
+    out = tmp_path / "result.json"
+    process = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "benchmark.py"), "--model", folder, "--num-requests", "5", "--max-tokens", "6", "--prompt-len", "11",
+         "--max-model-len", "64", "--max-num-seqs", "4", "--max-num-batched-tokens", "32", "--max-prefill-chunk-size", "8", "--block-size", "4",
+         "--num-gpu-blocks", "64", "--output-json", str(out), "--seed", "3"],
+        capture_output=True, text=True, timeout=600)
+    assert process.returncode == 0, process.stderr[-2000:]
+    result = json.loads(out.read_text())[0]
+    assert result["num_requests"] == 5 and result["generated_tokens"] == 30 and result["prompt_tokens"] == 55
+    assert "Decode throughput" in process.stdout and "TTFT" in process.stdout

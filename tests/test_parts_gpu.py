@@ -1,0 +1,254 @@
+"""Each part of a layer alone against the plain functions, and parts the framework does not have: a toy mixer
+with state of its own, registered, built and stepped from here without touching the framework's files; a
+layer that runs twice; a layer that reads another layer's cache; a windowed layer whose pages go back."""
+import math
+from typing import Dict
+
+import pytest
+import torch
+
+from plain_qwen2 import apply_rope, causal_attention, gated_mlp, rms_norm, rope_tables
+from velox_amd.cache import CacheManager
+from velox_amd.config.model_config import ModelConfig, architecture_name
+from velox_amd.config.registry import config_from_dict, get_architecture, register_architecture
+from velox_amd.engine.batch import StepEntry
+from velox_amd.engine.engine import build_model
+from velox_amd.engine.runner import ModelRunner
+from velox_amd.parts import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, StateNeed, make_part, register_part, single
+from velox_amd.parts.base import Mixer
+from velox_amd.weights import bind_random
+from velox_amd.weights.random_init import random_tensors
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from velox_amd.kernels import load_ops
+
+    return load_ops("cuda")
+
+
+class Ctx:
+    """The few fields a part reads, for calling one part alone."""
+
+    def __init__(self, ops, dtype, **fields):
+        self.ops, self.dtype = ops, dtype
+        self.__dict__.update(fields)
+
+
+def fill(part, seed, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    values = {}
+    for attr, param in part.params().items():
+        t = torch.randn(param.shape, generator=g) * (0.3 if param.role == "matrix" else 0.1)
+        if param.init == "one_plus_normal":
+            t = t + 1
+        held = torch.float32 if param.role == "vector" else dtype
+        setattr(part, attr, t.to(held).cuda())
+        values[attr] = t
+    return values
+
+
+def test_rmsnorm_part_owns_the_residual(ops):
+    norm = make_part("norm", "rmsnorm", prefix="n.", hidden_size=96, eps=1e-5)
+    w = fill(norm, 0)["weight"]
+    ctx = Ctx(ops, torch.float32)
+    residual = torch.randn(7, 96).cuda()
+    delta = torch.randn(7, 96).cuda()
+    before = residual.clone()
+    out = norm.forward(residual, delta, ctx)
+    torch.testing.assert_close(residual, before + delta)
+    torch.testing.assert_close(out.cpu(), rms_norm((before + delta).cpu(), w, 1e-5), rtol=1e-5, atol=1e-6)
+    rows = torch.tensor([6, 2], dtype=torch.int32).cuda()
+    kept = residual.clone()
+    out = norm.forward(residual, delta, ctx, rows=rows)
+    torch.testing.assert_close(residual, kept)
+    torch.testing.assert_close(out.cpu(), rms_norm((kept + delta).cpu()[[6, 2]], w, 1e-5), rtol=1e-5, atol=1e-6)
+
+
+def test_rotary_part_builds_the_reference_tables():
+    rope = make_part("position", "rotary", rotary_dim=32, theta=1e6, max_position=300, scaling_factor=2.0)
+    rope.finalize(torch.device("cuda"), torch.bfloat16)
+    cos, sin = rope.rotary_tables()
+    want_cos, want_sin = rope_tables(32, 1e6, 300, factor=2.0)
+    assert cos.dtype == torch.float32 and cos.shape == (300, 16)
+    torch.testing.assert_close(cos.cpu(), want_cos, rtol=0, atol=0)
+    torch.testing.assert_close(sin.cpu(), want_sin, rtol=0, atol=0)
+    assert make_part("position", "none").rotary_tables() is None
+
+
+def test_gated_mlp_part(ops):
+    ff = make_part("feed_forward", "gated_mlp", prefix="m.", hidden_size=80, intermediate_size=150)
+    w = fill(ff, 1)
+    x = torch.randn(9, 80)
+    got = ff.forward(x.cuda(), Ctx(ops, torch.float32)).cpu()
+    want = gated_mlp(x, w["gate_up_weight"][:150], w["gate_up_weight"][150:], w["down_weight"])
+    torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("nh,nkv,d,hidden,bias,window", [(4, 2, 16, 64, True, None), (6, 2, 48, 80, False, None), (3, 1, 32, 96, True, 5)])
+def test_attention_part_alone(ops, nh, nkv, d, hidden, bias, window):
+    """One attention layer over two sequences cut in two steps each, against plain whole-sequence attention."""
+    rope = make_part("position", "rotary", rotary_dim=d, theta=10000.0, max_position=128)
+    rope.finalize(torch.device("cuda"), torch.float32)
+    mixer = make_part("mixer", "attention", prefix="a.", hidden_size=hidden, num_heads=nh, num_kv_heads=nkv, head_dim=d, position=rope, qkv_bias=bias, window=window)
+    w = fill(mixer, 2)
+    ops.attention_library(d)
+    page = 4
+    cache = CacheManager([mixer.cache_need()], page, 40, 4, torch.float32, "cuda")
+    from velox_amd.engine.batch import BatchBuilder, Workspace
+
+    builder = BatchBuilder(cache, "cuda", 256, 4)
+    workspace = Workspace(torch.device("cuda"))
+    lengths = {"x": 23, "y": 10}
+    xs = {k: torch.randn(n, hidden) for k, n in lengths.items()}
+    seqs = {k: cache.new_sequence() for k in lengths}
+    got: Dict[str, list] = {k: [] for k in lengths}
+    done = {k: 0 for k in lengths}
+    for cuts in ({"x": 9, "y": 10}, {"x": 14}):
+        entries, rows = [], []
+        for k, n in cuts.items():
+            assert cache.append(seqs[k], done[k], n)
+            entries.append(StepEntry(seqs[k], [0] * n, done[k]))
+            rows.append(xs[k][done[k]:done[k] + n])
+        ctx = builder.build(entries, ops, torch.float32, workspace)
+        out = mixer.forward(torch.cat(rows).cuda(), ctx, ctx.cache_view(0), True).cpu()
+        at = 0
+        for k, n in cuts.items():
+            got[k].append(out[at:at + n])
+            at += n
+            done[k] += n
+            cache.release_behind_window(seqs[k], done[k])
+    cos, sin = rope_tables(d, 10000.0, 128)
+    for k, n in lengths.items():
+        qkv = xs[k] @ w["qkv_weight"].T + (w["qkv_bias_vec"] if bias else 0)
+        q = apply_rope(qkv[:, : nh * d].reshape(n, nh, d), cos, sin, torch.arange(n))
+        kk = apply_rope(qkv[:, nh * d:(nh + nkv) * d].reshape(n, nkv, d), cos, sin, torch.arange(n))
+        v = qkv[:, (nh + nkv) * d:].reshape(n, nkv, d)
+        want = causal_attention(q, kk, v, 1 / math.sqrt(d), window).reshape(n, nh * d) @ w["o_weight"].T
+        torch.testing.assert_close(torch.cat(got[k]), want, rtol=2e-4, atol=2e-5)
+    if window is not None:
+        assert seqs["x"].tables[0][0] == 0  # pages behind the window went back while the request was running
+
+
+# ----------------------------------------------------------------------------------------------------
+# a toy architecture defined here: a mixer with per-request state, then an attention layer that runs twice,
+# the second time beside an entry that reads the first run's cache
+# ----------------------------------------------------------------------------------------------------
+class DecayingSumMixer(Mixer):
+    """y_t = W s_t,  s_t = decay * s_{t-1} + x_t, with s kept per request in the cache manager's state slots."""
+
+    def __init__(self, prefix: str, hidden_size: int, decay: float) -> None:
+        super().__init__(prefix)
+        self.hidden_size, self.decay = hidden_size, decay
+        self.weight = None
+
+    def params(self):
+        return {"weight": single("mix.weight", (self.hidden_size, self.hidden_size))}
+
+    def cache_need(self):
+        return StateNeed((("sum", (self.hidden_size,), torch.float32),))
+
+    def forward(self, x, ctx, cache, owns_cache=True):
+        state = cache.tensors["sum"]
+        out = torch.empty_like(x)
+        at = 0
+        for slot, n in zip(ctx.slots.tolist(), ctx.q_lens):
+            s = state[slot]
+            for t in range(at, at + n):
+                s = self.decay * s + x[t].float()
+                out[t] = (self.weight.float() @ s).to(x.dtype)
+            state[slot] = s
+            at += n
+        return out
+
+
+def toy_spec(config, max_position=None) -> ModelSpec:
+    raw = config.raw
+    h = raw["hidden_size"]
+    norm = PartSpec.of("rmsnorm", hidden_size=h, eps=raw["eps"])
+    ff = PartSpec.of("gated_mlp", hidden_size=h, intermediate_size=raw["inter"])
+    attention = PartSpec.of("attention", hidden_size=h, num_heads=4, num_kv_heads=2, head_dim=16, qkv_bias=False)
+    layers = [
+        LayerSpec("layers.0.", PartSpec.of("toy_decaying_sum", hidden_size=h, decay=raw["decay"]), ff, norm, norm, mixer_prefix="mixer."),
+        LayerSpec("layers.1.", attention, ff, norm, norm, position="rope"),
+    ]
+    schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(1, cache_from=1)]
+    return ModelSpec(vocab_size=raw["vocab_size"], hidden_size=h, max_position=256, layers=layers, schedule=schedule, final_norm=norm,
+                     positions={"rope": PartSpec.of("rotary", rotary_dim=16, theta=10000.0, max_position=256)}, tie_head=True)
+
+
+def plain_toy(tensors: Dict[str, torch.Tensor], raw, tokens):
+    h, eps, decay = raw["hidden_size"], raw["eps"], raw["decay"]
+    n = len(tokens)
+    cos, sin = rope_tables(16, 10000.0, n)
+    x = tensors["model.embed_tokens.weight"][torch.tensor(tokens)]
+    kept_kv = {}
+
+    def ff(p, m):
+        return gated_mlp(m, tensors[p + "mlp.gate_proj.weight"], tensors[p + "mlp.up_proj.weight"], tensors[p + "mlp.down_proj.weight"])
+
+    for index, (layer, cache_from) in enumerate([(0, None), (1, None), (0, None), (1, None), (1, 1)]):
+        p = f"layers.{layer}."
+        a = rms_norm(x, tensors[p + "input_layernorm.weight"], eps)
+        if layer == 0:
+            s = torch.zeros(h)
+            rows = []
+            for t in range(n):
+                s = decay * s + a[t]
+                rows.append(tensors[p + "mixer.mix.weight"] @ s)
+            mixed = torch.stack(rows)
+        else:
+            q = apply_rope((a @ tensors[p + "self_attn.q_proj.weight"].T).reshape(n, 4, 16), cos, sin, torch.arange(n))
+            if cache_from is None:
+                k = apply_rope((a @ tensors[p + "self_attn.k_proj.weight"].T).reshape(n, 2, 16), cos, sin, torch.arange(n))
+                v = (a @ tensors[p + "self_attn.v_proj.weight"].T).reshape(n, 2, 16)
+                kept_kv[index] = (k, v)
+            else:
+                k, v = kept_kv[cache_from]
+            mixed = causal_attention(q, k, v, 0.25).reshape(n, 64) @ tensors[p + "self_attn.o_proj.weight"].T
+        x = x + mixed
+        x = x + ff(p, rms_norm(x, tensors[p + "post_attention_layernorm.weight"], eps))
+    return rms_norm(x, tensors["model.norm.weight"], eps) @ tensors["model.embed_tokens.weight"].T
+
+
+def test_toy_architecture_with_state_repeated_layer_and_shared_cache(ops):
+    register_part("mixer", "toy_decaying_sum", DecayingSumMixer)
+    register_architecture("ToyForCausalLM", lambda raw: ModelConfig(architecture_name(raw), dict(raw)), toy_spec)
+    raw = {"architectures": ["ToyForCausalLM"], "hidden_size": 64, "inter": 96, "vocab_size": 101, "eps": 1e-5, "decay": 0.8}
+    config = config_from_dict(raw)
+    model = build_model(config, torch.float32, "cuda")
+    needs = model.cache_needs()
+    assert [type(n).__name__ for n in needs] == ["StateNeed", "PagedNeed", "StateNeed", "PagedNeed", "NoneType"]
+    bind_random(model, 4, torch.float32, "cuda", storage_dtype=torch.float32)
+    tensors = dict(random_tensors(model, 4))
+    ops.prepare(model, torch.float32)
+    cache = CacheManager(needs, 4, 40, 3, torch.float32, "cuda")
+    assert len(cache.groups) == 1 and cache.groups[0].entries == [1, 3]  # both runs of the attention layer own a cache
+    runner = ModelRunner(model, cache, ops, torch.float32, "cuda", 128, 3)
+    g = torch.Generator().manual_seed(0)
+    prompts = {k: torch.randint(0, 101, (n,), generator=g).tolist() for k, n in (("p", 29), ("q", 12), ("r", 40))}
+    seqs = {k: cache.new_sequence() for k in prompts}
+    done = {k: 0 for k in prompts}
+    got = {k: [] for k in prompts}
+    plan = [{"p": 5, "q": 12}, {"p": 1, "r": 17}, {"p": 23, "r": 2}, {"r": 21}]
+    for cuts in plan:
+        entries = []
+        for k, n in cuts.items():
+            assert cache.append(seqs[k], done[k], n)
+            entries.append(StepEntry(seqs[k], prompts[k][done[k]:done[k] + n], done[k], list(range(n))))
+        logits = runner.step(entries).cpu()
+        at = 0
+        for k, n in cuts.items():
+            got[k].append(logits[at:at + n])
+            at += n
+            done[k] += n
+    for k, tokens in prompts.items():
+        torch.testing.assert_close(torch.cat(got[k]), plain_toy(tensors, raw, tokens), rtol=2e-4, atol=2e-5)
+    # a slot that is taken again starts from zero state
+    cache.free_sequence(seqs["q"])
+    again = cache.new_sequence()
+    assert cache.append(again, 0, 12)
+    logits = runner.step([StepEntry(again, prompts["q"], 0, list(range(12)))]).cpu()
+    torch.testing.assert_close(logits, torch.cat(got["q"]), rtol=1e-5, atol=1e-6)

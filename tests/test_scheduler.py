@@ -1,0 +1,219 @@
+"""The scheduler's decisions, driven without a model: what a step would compute is simulated."""
+import pytest
+import torch
+
+from velox_amd.cache import CacheManager
+from velox_amd.engine.request import FinishReason, Request, RequestStatus
+from velox_amd.engine.scheduler import Scheduler, SchedulerConfig
+from velox_amd.parts.base import PagedNeed
+from velox_amd.sampling import SamplingParams
+
+
+def make(pages=33, page=4, seqs=4, budget=16, chunk=8, max_len=128, watermark=0.01):
+    cache = CacheManager([PagedNeed(1, 16)], page, pages, seqs, torch.float32, "cpu", max_model_len=max_len, allocate_tensors=False)
+    return Scheduler(cache, SchedulerConfig(max_num_seqs=seqs, max_num_batched_tokens=budget, max_prefill_chunk_size=chunk, max_model_len=max_len, watermark=watermark))
+
+
+def request(rid, prompt_len, max_tokens=4):
+    return Request(rid, list(range(1, prompt_len + 1)), SamplingParams(temperature=0.0, max_tokens=max_tokens, ignore_eos=True))
+
+
+def run_step(s, out):
+    """What the engine does after a forward: advance, append a token to rows that completed their tokens."""
+    scheduled = out.decode_batch + out.prefill_batch
+    assert len({id(r) for r in scheduled}) == len(scheduled), "a request is in a step twice"
+    assert all(r.cache is not None and r in s.running for r in scheduled), "a scheduled request has no pages"
+    assert not any(r in scheduled for r in out.preempted if r.cache is None)
+    for r in out.decode_batch:
+        s.advance(r, 1)
+    for r in out.prefill_batch:
+        completes = r.num_computed_tokens + r.current_chunk_size >= len(r.all_token_ids)
+        s.advance(r, r.current_chunk_size)
+        r.refresh_status()
+        if not completes:
+            continue
+        out.decode_batch.append(r)  # sampled below
+    for r in out.decode_batch:
+        r.append_token(1000 + len(r.output_token_ids))
+        r.refresh_status()
+        reason = r.should_stop(r.output_token_ids[-1], frozenset())
+        if reason:
+            r.finish(reason)
+
+
+def test_prompt_is_cut_under_budget_and_chunk_then_decodes_first():
+    s = make(budget=16, chunk=8)
+    a, b = request("a", 19), request("b", 5)
+    s.add_request(a)
+    s.add_request(b)
+    out = s.schedule()
+    assert [r.request_id for r in out.prefill_batch] == ["a", "b"] and (a.current_chunk_size, b.current_chunk_size) == (8, 5)
+    assert out.num_batched_tokens == 13 and not out.decode_batch
+    run_step(s, out)
+    assert a.status is RequestStatus.RUNNING_PREFILL and b.status is RequestStatus.RUNNING_DECODE and b.output_token_ids == [1000]
+    out = s.schedule()
+    assert [r.request_id for r in out.decode_batch] == ["b"] and [r.request_id for r in out.prefill_batch] == ["a"] and a.current_chunk_size == 8
+    run_step(s, out)
+    out = s.schedule()
+    assert a.current_chunk_size == 3 and a.num_computed_tokens == 16
+    run_step(s, out)
+    assert a.status is RequestStatus.RUNNING_DECODE and a.output_token_ids == [1000]
+
+
+def test_budget_counts_decodes_before_prompts():
+    s = make(budget=6, chunk=6, seqs=4)
+    for i in range(3):
+        s.add_request(request(f"d{i}", 2, max_tokens=20))
+    run_step(s, s.schedule())
+    s.add_request(request("p", 30))
+    out = s.schedule()
+    assert len(out.decode_batch) == 3 and out.prefill_batch[0].current_chunk_size == 3  # 6 - 3 decodes
+
+
+def test_finish_frees_pages_at_the_next_schedule_and_reasons():
+    s = make()
+    a = request("a", 6, max_tokens=2)
+    s.add_request(a)
+    run_step(s, s.schedule())
+    run_step(s, s.schedule())
+    assert a.finished and a.finish_reason is FinishReason.LENGTH and len(a.output_token_ids) == 2
+    assert s.cache.num_used_pages() > 0 and s.has_work()
+    out = s.schedule()
+    assert out.is_empty() and s.cache.num_used_pages() == 0 and not s.has_work() and s.num_finished == 1
+    s.cache.assert_consistent([])
+    stop = Request("s", [1, 2, 3], SamplingParams(max_tokens=9, stop_token_ids=[77]))
+    assert stop.should_stop(77, frozenset()) is FinishReason.STOP and stop.should_stop(5, frozenset({5})) is FinishReason.STOP
+    assert Request("i", [1], SamplingParams(max_tokens=9, ignore_eos=True)).should_stop(5, frozenset({5})) is None
+
+
+def test_limits_are_refused_at_add():
+    s = make(max_len=32)
+    with pytest.raises(ValueError):
+        s.add_request(request("long", 32))
+    with pytest.raises(ValueError):
+        s.add_request(request("long2", 30, max_tokens=3))
+    s.add_request(request("fits", 30, max_tokens=2))
+    with pytest.raises(ValueError):
+        s.add_request(request("fits", 3))
+    with pytest.raises(ValueError):
+        Request("empty", [], SamplingParams())
+    # the pool bounds the length too: 8 usable pages of 4
+    small = make(pages=9, max_len=4096)
+    assert small.config.max_model_len == 32
+
+
+def test_admission_waits_for_slots_and_keeps_a_watermark_first_come_first_served():
+    s = make(pages=11, seqs=2, budget=64, chunk=64, watermark=0.2)  # 10 usable pages, watermark 2
+    for rid, n in (("a", 12), ("b", 20), ("c", 4)):
+        s.add_request(request(rid, n, max_tokens=2))
+    out = s.schedule()
+    # a takes 3 pages; b wants 5 of the 7 left, headroom 7 - 2 = 5: fits; c finds no slot
+    assert [r.request_id for r in out.prefill_batch] == ["a", "b"] and s.num_waiting == 1
+    run_step(s, out)
+    s2 = make(pages=11, seqs=4, budget=64, chunk=64, watermark=0.2)
+    for rid, n in (("a", 12), ("b", 28), ("c", 4)):
+        s2.add_request(request(rid, n, max_tokens=2))
+    out = s2.schedule()
+    # b needs 7 pages, headroom is 5: it gets a 20-token portion (5 pages); c then sees headroom 0 and waits behind it
+    assert [(r.request_id, r.current_chunk_size) for r in out.prefill_batch] == [("a", 12), ("b", 20)]
+    assert [r.request_id for r in s2.waiting] == ["c"]
+
+
+def test_decode_out_of_pages_preempts_the_newest_and_recomputes_it():
+    s = make(pages=7, page=4, seqs=3, budget=32, chunk=32, watermark=0.01)  # 6 usable pages
+    a, b = request("a", 8, max_tokens=12), request("b", 8, max_tokens=12)
+    s.add_request(a)
+    s.add_request(b)
+    run_step(s, s.schedule())  # 2 pages each, one token sampled each
+    assert s.cache.num_free_pages() == 2
+    run_step(s, s.schedule())  # both decode: position 8 needs a third page each
+    assert s.cache.num_free_pages() == 0 and not s.num_preemptions
+    for _ in range(3):
+        run_step(s, s.schedule())  # positions 9, 10, 11 fit
+    out = s.schedule()  # position 12: a needs a 4th page, none free: b (the newest) is preempted
+    assert [r.request_id for r in out.preempted] == ["b"] and [r.request_id for r in out.decode_batch] == ["a"]
+    assert b.num_preemptions == 1 and s.num_preemptions == 1 and len(b.output_token_ids) == 5  # its tokens are kept
+    # the same scheduling decision admits it again from the front of the queue, from position 0, with what fits
+    assert [r.request_id for r in out.prefill_batch] == ["b"] and b.num_computed_tokens == 0
+    assert b.status is RequestStatus.RUNNING_PREFILL and b.current_chunk_size == 4  # 2 pages free, 1 held back
+    run_step(s, out)
+    s.cache.assert_consistent([a.cache, b.cache])
+    # its recomputation covers prompt and generated tokens (13), then it decodes on: no token is lost or sampled twice
+    guard = 0
+    while b.status is not RequestStatus.RUNNING_DECODE:
+        run_step(s, s.schedule())
+        guard += 1
+        assert guard < 50
+    assert len(b.output_token_ids) == 6 and b.num_computed_tokens == 13
+    while s.has_work():
+        run_step(s, s.schedule())
+    assert len(a.output_token_ids) == 12 and len(b.output_token_ids) == 12 and s.cache.num_used_pages() == 0
+    assert a.output_token_ids == b.output_token_ids == [1000 + i for i in range(12)]
+    s.cache.assert_consistent([])
+
+
+def test_oldest_prefill_may_evict_newer_requests_but_a_newer_prefill_waits():
+    s = make(pages=6, page=4, seqs=3, budget=12, chunk=8, watermark=0.01)  # 5 usable pages
+    a, b = request("a", 18, max_tokens=2), request("b", 12, max_tokens=2)
+    s.add_request(a)
+    s.add_request(b)
+    out = s.schedule()  # a: 8 tokens, 2 pages; b: the 4 tokens the budget leaves, 1 page
+    assert [(r.request_id, r.current_chunk_size) for r in out.prefill_batch] == [("a", 8), ("b", 4)]
+    run_step(s, out)
+    out = s.schedule()  # a takes the last 2 free pages; b finds none and, not being the oldest, just waits
+    assert [(r.request_id, r.current_chunk_size) for r in out.prefill_batch] == [("a", 8)] and not out.preempted
+    run_step(s, out)
+    out = s.schedule()  # a needs one more page: as the oldest prefill it evicts b, the newest request
+    assert [r.request_id for r in out.preempted] == ["b"] and out.prefill_batch[0] is a and a.current_chunk_size == 2
+    assert b.num_preemptions == 1 and b.num_computed_tokens == 0
+    run_step(s, out)
+    while s.has_work():
+        run_step(s, s.schedule())
+    assert len(a.output_token_ids) == 2 and len(b.output_token_ids) == 2 and s.cache.num_used_pages() == 0
+
+
+def test_two_requests_that_cannot_both_fit_still_finish():
+    s = make(pages=5, page=4, seqs=2, budget=32, chunk=32, watermark=0.01)  # 4 usable pages; a alone needs all of them
+    a, b = request("a", 8, max_tokens=8), request("b", 7, max_tokens=8)
+    s.add_request(a)
+    s.add_request(b)
+    guard = 0
+    while s.has_work():
+        out = s.schedule()
+        for victim in out.preempted:
+            assert victim is b  # the older request never yields to the newer one
+        run_step(s, out)
+        s.cache.assert_consistent([r.cache for r in s.running if r.cache is not None])
+        guard += 1
+        assert guard < 200
+    assert s.num_preemptions >= 1 and b.num_preemptions >= 1 and a.num_preemptions == 0
+    assert a.output_token_ids == b.output_token_ids == [1000 + i for i in range(8)]
+    s.cache.assert_consistent([])
+
+
+def test_abort_gives_everything_back_at_once():
+    s = make()
+    a = request("a", 9)
+    s.add_request(a)
+    run_step(s, s.schedule())
+    assert s.abort_request("a") and a.finish_reason is FinishReason.ABORT and a.status is RequestStatus.ABORTED
+    assert s.cache.num_used_pages() == 0 and not s.has_work() and not s.abort_request("a")
+    s.cache.assert_consistent([])
+
+
+def test_a_victim_leaves_the_step_it_was_already_given_a_token_in():
+    # a decodes and b (newer) decodes too; then ... the oldest prefill evicts the newest request, which already sits in the decode batch
+    s = make(pages=7, page=4, seqs=3, budget=16, chunk=8, watermark=0.01)  # 6 usable pages
+    a = request("a", 20, max_tokens=2)
+    b = request("b", 3, max_tokens=9)
+    s.add_request(a)
+    s.add_request(b)
+    run_step(s, s.schedule())  # a: 8 tokens (2 pages); b: whole prompt (1 page), decoding from now on
+    run_step(s, s.schedule())  # b decodes; a: 8 more (4 pages)
+    assert s.cache.num_free_pages() == 1
+    out = s.schedule()  # b decodes (position 4: takes the last page); a then needs a 5th page and evicts b
+    assert [r.request_id for r in out.preempted] == ["b"] and b not in out.decode_batch
+    run_step(s, out)
+    while s.has_work():
+        run_step(s, s.schedule())
+    assert len(a.output_token_ids) == 2 and len(b.output_token_ids) == 9

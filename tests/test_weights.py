@@ -1,0 +1,101 @@
+"""Weights by name from safetensors: one error for everything wrong, dtypes, the random-weights folder."""
+import json
+import os
+
+import pytest
+import torch
+from safetensors.torch import load_file, save_file
+
+from helpers import TINY_A, TINY_B, make_folder
+from velox_amd.config import load_config
+from velox_amd.engine.engine import build_model
+from velox_amd.weights import WeightsError, bind_from_checkpoint, bind_random, held_dtype, write_random_model
+
+
+def _load(folder, dtype=torch.float32):
+    model = build_model(load_config(folder), dtype, "cpu")
+    bind_from_checkpoint(model, folder, dtype, "cpu")
+    return model
+
+
+def test_random_folder_round_trip_and_fusion(tmp_path):
+    folder = make_folder(tmp_path, "B")
+    raw = load_file(os.path.join(folder, "model.safetensors"))
+    assert "lm_head.weight" in raw and raw["model.layers.2.self_attn.k_proj.bias"].shape == (32,)
+    model = _load(folder)
+    mixer = model.blocks[1].mixer
+    p = "model.layers.1.self_attn."
+    want = torch.cat([raw[p + "q_proj.weight"], raw[p + "k_proj.weight"], raw[p + "v_proj.weight"]])
+    assert torch.equal(mixer.qkv_weight, want)
+    assert torch.equal(mixer.qkv_bias_vec, torch.cat([raw[p + "q_proj.bias"], raw[p + "k_proj.bias"], raw[p + "v_proj.bias"]]))
+    ff = model.blocks[1].feed_forward
+    assert torch.equal(ff.gate_up_weight, torch.cat([raw["model.layers.1.mlp.gate_proj.weight"], raw["model.layers.1.mlp.up_proj.weight"]]))
+    assert torch.equal(model.head.weight, raw["lm_head.weight"]) and model.head.weight.data_ptr() != model.embedding.table.data_ptr()
+    # norm weights are around one, everything else around zero
+    assert abs(float(raw["model.norm.weight"].mean()) - 1.0) < 0.05 and abs(float(raw["model.embed_tokens.weight"].mean())) < 0.01
+    assert abs(float(raw["model.embed_tokens.weight"].std()) - 0.02) < 0.002
+
+
+def test_same_seed_same_weights_other_seed_other_weights(tmp_path):
+    a = load_file(os.path.join(write_random_model(TINY_A, str(tmp_path / "a"), 5, "float32"), "model.safetensors"))
+    b = load_file(os.path.join(write_random_model(TINY_A, str(tmp_path / "b"), 5, "float32"), "model.safetensors"))
+    c = load_file(os.path.join(write_random_model(TINY_A, str(tmp_path / "c"), 6, "float32"), "model.safetensors"))
+    assert all(torch.equal(a[k], b[k]) for k in a) and not torch.equal(a["model.norm.weight"], c["model.norm.weight"])
+    # in-memory binding with the host generator gives the folder's values
+    model = build_model(load_config(str(tmp_path / "a")), torch.float32, "cpu")
+    bind_random(model, 5, torch.float32, "cpu", storage_dtype=torch.float32)
+    assert torch.equal(model.embedding.table, a["model.embed_tokens.weight"])
+    assert torch.equal(model.final_norm.weight, a["model.norm.weight"])
+
+
+def test_tied_head_shares_the_table(tmp_path):
+    folder = make_folder(tmp_path, "A")
+    assert "lm_head.weight" not in load_file(os.path.join(folder, "model.safetensors"))
+    model = _load(folder)
+    assert model.head.weight.data_ptr() == model.embedding.table.data_ptr()
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    folder = make_folder(tmp_path, "B")
+    path = os.path.join(folder, "model.safetensors")
+    raw = load_file(path)
+    del raw["model.layers.0.self_attn.q_proj.bias"]
+    del raw["model.norm.weight"]
+    raw["model.layers.7.mlp.up_proj.weight"] = torch.zeros(3, 3)
+    raw["extra.tensor"] = torch.zeros(1)
+    raw["model.layers.1.mlp.down_proj.weight"] = torch.zeros(96, 100)
+    raw["lm_head.weight"] = torch.zeros(320, 95)
+    save_file(raw, path)
+    with pytest.raises(WeightsError) as err:
+        _load(folder)
+    e = err.value
+    assert e.missing == ["model.layers.0.self_attn.q_proj.bias", "model.norm.weight"]
+    assert e.unexpected == ["extra.tensor", "model.layers.7.mlp.up_proj.weight"]
+    assert len(e.wrong_shape) == 2 and any("down_proj" in w and "(96, 100)" in w and "(96, 224)" in w for w in e.wrong_shape)
+    text = str(e)
+    for fragment in ("missing tensors (2)", "unexpected tensors (2)", "wrong shapes (2)", "extra.tensor", "lm_head.weight"):
+        assert fragment in text
+
+
+def test_missing_files(tmp_path):
+    (tmp_path / "config.json").write_text(json.dumps(TINY_A))
+    with pytest.raises(FileNotFoundError):
+        _load(str(tmp_path))
+
+
+def test_dtypes_kept(tmp_path):
+    # stored bfloat16: stays bfloat16 in a bfloat16 run, widened exactly in a float32 run; vectors always float32
+    folder = make_folder(tmp_path, "B", "bfloat16")
+    raw = load_file(os.path.join(folder, "model.safetensors"))
+    bf = _load(folder, torch.bfloat16)
+    assert bf.embedding.table.dtype == torch.bfloat16 and bf.blocks[0].mixer.qkv_weight.dtype == torch.bfloat16
+    assert bf.final_norm.weight.dtype == torch.float32 and bf.blocks[0].mixer.qkv_bias_vec.dtype == torch.float32
+    assert torch.equal(bf.final_norm.weight, raw["model.norm.weight"].float())
+    wide = _load(folder, torch.float32)
+    assert wide.embedding.table.dtype == torch.float32 and torch.equal(wide.embedding.table, raw["model.embed_tokens.weight"].float())
+    # stored float32 stays float32 even in a bfloat16 run
+    folder32 = make_folder(tmp_path, "B", "float32")
+    kept = _load(folder32, torch.bfloat16)
+    assert kept.blocks[0].mixer.qkv_weight.dtype == torch.float32
+    assert held_dtype("matrix", torch.int64, torch.bfloat16) == torch.int32
+    assert held_dtype("matrix", torch.float16, torch.bfloat16) == torch.bfloat16

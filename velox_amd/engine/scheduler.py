@@ -112,7 +112,15 @@ class Scheduler:
             self.cache.free_sequence(request.cache)
             request.cache = None
 
-    def _preempt(self, request: Request) -> None:
+    def _preempt(self, request: Request, output: Optional[SchedulerOutput] = None) -> None:
+        if output is not None:
+            # a victim may already have been given its token of this step (the reference leaves it in the
+            # batch, engine/scheduler.py:241-247): it must not run without its pages
+            if request in output.decode_batch:
+                output.decode_batch.remove(request)
+            if request in output.prefill_batch:
+                output.prefill_batch.remove(request)
+            output.preempted.append(request)
         self._release(request)
         request.num_computed_tokens = 0
         request.status = RequestStatus.PREEMPTED
@@ -127,8 +135,7 @@ class Scheduler:
             if not self.running:
                 return False
             victim = self.running[-1]  # always the newest, even when that is the caller
-            self._preempt(victim)
-            output.preempted.append(victim)
+            self._preempt(victim, output)
             if victim is request:
                 return False
         return True
@@ -164,8 +171,7 @@ class Scheduler:
                 break
             if not self._make_room(request, 1, output) or not self.cache.append(request.cache, request.num_computed_tokens, 1):
                 if request in self.running:
-                    self._preempt(request)
-                    output.preempted.append(request)
+                    self._preempt(request, output)
                 continue
             request.current_chunk_size = 1
             output.decode_batch.append(request)
@@ -183,8 +189,7 @@ class Scheduler:
             chunk = min(wanted, self.cache.max_new_tokens(request.cache, request.num_computed_tokens))
             while chunk <= 0 and oldest and self.running and self.running[-1] is not request:
                 victim = self.running[-1]
-                self._preempt(victim)
-                output.preempted.append(victim)
+                self._preempt(victim, output)
                 chunk = min(wanted, self.cache.max_new_tokens(request.cache, request.num_computed_tokens))
             if chunk <= 0 or not self.cache.append(request.cache, request.num_computed_tokens, chunk):
                 continue

@@ -119,6 +119,7 @@ def bind_from_checkpoint(model, model_dir: str, run_dtype: torch.dtype, device) 
                 plan.append((part, attr, param, None))
                 continue
             missing.extend(absent)
+            used.update(name for name in names if name in checkpoint)
             continue
         ok = True
         for name, want in zip(names, param.source_shapes):
