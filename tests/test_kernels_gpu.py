@@ -309,3 +309,25 @@ def test_penalties(ops, ref):
     ops.apply_penalties(got, tokens, lengths, coeffs)
     ref.apply_penalties(want, tokens, lengths, coeffs)
     torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("m,n,k", [(1, 320, 64), (8, 3584, 3584), (16, 263, 128), (7, 4608, 3584), (17, 100, 192), (32, 1000, 256), (33, 70, 64), (64, 3584, 18944), (50, 152064 // 16, 448)])
+def test_skinny_gemm(ops, ref, out_dtype, m, n, k):
+    x = rand((m, k), torch.bfloat16, 40)
+    w = rand((n, k), torch.bfloat16, 41, 0.05)
+    bias = rand((n,), torch.float32, 42)
+    want = ref.linear(x, w, None, torch.float32)
+    scale = float(want.abs().max())
+    for waves in (None, 4, 8, 16):
+        for b in (None, bias):
+            got = ops.skinny_gemm(x, w, b, out_dtype, waves=waves).float()
+            expect = want + (b if b is not None else 0)
+            atol = 1e-4 * scale if out_dtype == torch.float32 else 1e-2 * scale
+            torch.testing.assert_close(got, expect, rtol=1e-2 if out_dtype == torch.bfloat16 else 1e-4, atol=atol)
+    # the same rows give the same bits whatever else is in the batch, as long as the batch stays in one size class
+    # (up to 16, up to 32, up to 64 rows: the classes split K differently, which changes the order of the sums)
+    fewer = 1 if m <= 16 else 17 if m <= 32 else 33
+    if m > fewer:
+        part = ops.skinny_gemm(x[:fewer].contiguous(), w, None, out_dtype)
+        torch.testing.assert_close(ops.skinny_gemm(x, w, None, out_dtype)[:fewer], part, rtol=0, atol=0)

@@ -1,0 +1,159 @@
+// out[M, N] = A[M, K] * W[N, K]^T (+ bias[N]) for few rows (M <= 64), bfloat16 operands, float32 accumulation: the
+// matrix products of a decode step on gfx950.  Such a product is bound by reading W once from HBM, so the kernel is
+// built around keeping many wide loads of W in flight:
+//
+//  * a workgroup owns 16 * RT consecutive rows of W (output columns) and ALL of K; its waves split K among
+//    themselves and their partial sums are added through LDS in a fixed order (no atomics: the result is the same
+//    on every run and does not depend on the launch);
+//  * a lane reads W in runs of 16 consecutive bfloat16 (32 bytes): for a block of 64 contraction indices, lane
+//    (g = lane / 16, i = lane % 16) holds W[row i][k0 + 16 g .. + 15], the four lane groups cover 128 contiguous
+//    bytes of each row.  The two halves of the run feed two v_mfma_f32_16x16x32_bf16, W as the left operand
+//    (16 rows x 32 indices) and the activations as the right one (32 indices x 16 batch rows) with the same index
+//    assignment, so out^T[n, m] accumulates in the usual 16x16 layout;
+//  * the activations are small (M x K) and come from L2 in the same lane layout; batch rows beyond M are zeros.
+//
+// Requirements checked by the caller: K % 64 == 0, M <= 16 * CT, 16-byte aligned operands.
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float8_raw_t __attribute__((ext_vector_type(8)));
+
+struct Run16 {  // 16 consecutive bfloat16 = two MFMA operands
+  bf16x8_t lo, hi;
+};
+
+__device__ __forceinline__ Run16 load_run(const bf16_t* p) {
+  Run16 r;
+  const float4_t* q = reinterpret_cast<const float4_t*>(p);
+  const float4_t a = q[0], b = q[1];
+  r.lo = __builtin_bit_cast(bf16x8_t, a);
+  r.hi = __builtin_bit_cast(bf16x8_t, b);
+  return r;
+}
+
+__device__ __forceinline__ Run16 zero_run() {
+  Run16 r;
+  const float4_t z = {0.f, 0.f, 0.f, 0.f};
+  r.lo = __builtin_bit_cast(bf16x8_t, z);
+  r.hi = r.lo;
+  return r;
+}
+
+template <int RT, int CT, int WAVES, typename TO>
+__global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
+                                                                 const float* __restrict__ bias, TO* __restrict__ out, int m, int n, int k) {
+  constexpr int UNROLL = 4;  // blocks of 64 indices whose loads are issued together
+  __shared__ float4_t partial[WAVES][RT * CT][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int g = lane >> 4, i = lane & 15;
+  const int n0 = blockIdx.x * 16 * RT;
+
+  // this wave's share of K, in blocks of 64
+  const int blocks_total = k / 64;
+  const int per_wave = (blocks_total + WAVES - 1) / WAVES;
+  const int kb_lo = wave * per_wave;
+  int kb_hi = kb_lo + per_wave;
+  if (kb_hi > blocks_total) kb_hi = blocks_total;
+
+  const bf16_t* w_ptr[RT];
+  bool w_ok[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int row = n0 + 16 * rt + i;
+    w_ok[rt] = row < n;
+    w_ptr[rt] = w + (size_t)(w_ok[rt] ? row : 0) * k + 16 * g;
+  }
+  const bf16_t* a_ptr[CT];
+  bool a_ok[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int row = 16 * ct + i;
+    a_ok[ct] = row < m;
+    a_ptr[ct] = a + (size_t)(a_ok[ct] ? row : 0) * k + 16 * g;
+  }
+
+  float4_t acc[RT][CT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  for (int kb = kb_lo; kb < kb_hi; kb += UNROLL) {
+    Run16 wr[UNROLL][RT];
+    Run16 ar[UNROLL][CT];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const bool in_range = kb + u < kb_hi;
+      const size_t k0 = (size_t)(kb + u) * 64;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) wr[u][rt] = (in_range && w_ok[rt]) ? load_run(w_ptr[rt] + k0) : zero_run();
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) ar[u][ct] = (in_range && a_ok[ct]) ? load_run(a_ptr[ct] + k0) : zero_run();
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+          acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wr[u][rt].lo, ar[u][ct].lo, acc[rt][ct], 0, 0, 0);
+          acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wr[u][rt].hi, ar[u][ct].hi, acc[rt][ct], 0, 0, 0);
+        }
+  }
+
+  // add the waves' partial sums in wave order; each tile's 64 lanes are then spread over the workgroup
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) partial[wave][rt * CT + ct][lane] = acc[rt][ct];
+  __syncthreads();
+  for (int item = threadIdx.x; item < RT * CT * 64; item += WAVES * 64) {
+    const int tile = item >> 6, l = item & 63;
+    float4_t sum = partial[0][tile][l];
+#pragma unroll
+    for (int wv = 1; wv < WAVES; ++wv) sum += partial[wv][tile][l];
+    const int rt = tile / CT, ct = tile % CT;
+    const int col_m = 16 * ct + (l & 15);           // batch row
+    const int row_n = n0 + 16 * rt + 4 * (l >> 4);  // first of four output columns
+    if (col_m >= m) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (row_n + j >= n) break;
+      float v = sum[j];
+      if (bias) v += bias[row_n + j];
+      out[(size_t)col_m * n + row_n + j] = from_f32<TO>(v);
+    }
+  }
+}
+
+template <int RT, int CT, int WAVES>
+static int launch_skinny(const void* a, const void* w, const float* bias, void* out, int m, int n, int k, int out_dtype, hipStream_t stream) {
+  const int blocks = (n + 16 * RT - 1) / (16 * RT);
+  if (out_dtype == VELOX_BF16)
+    skinny_gemm_kernel<RT, CT, WAVES, bf16_t><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (bf16_t*)out, m, n, k);
+  else
+    skinny_gemm_kernel<RT, CT, WAVES, float><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (float*)out, m, n, k);
+  return (int)hipGetLastError();
+}
+
+// waves: how many waves of a workgroup split K (4, 8 or 16; rounded down to what the tile shape allows); the
+// caller picks it so that the launch fills the GPU.
+extern "C" int velox_skinny_gemm_bf16(const void* a, const void* w, const float* bias, void* out, int m, int n, int k, int out_dtype,
+                                      int waves, hipStream_t stream) {
+  if (m <= 0 || n <= 0) return 0;
+  if (k % 64 != 0 || m > 64) return -1;
+#define PICK(RT, CT, W) return launch_skinny<RT, CT, W>(a, w, bias, out, m, n, k, out_dtype, stream)
+  if (m <= 16) {
+    if (waves >= 16) PICK(1, 1, 16);
+    if (waves >= 8) PICK(1, 1, 8);
+    PICK(1, 1, 4);
+  }
+  // more tiles per wave: registers (and the LDS for the final sum) allow 8 waves at most
+  if (m <= 32) {
+    if (waves >= 8) PICK(2, 2, 8);
+    PICK(2, 2, 4);
+  }
+  if (waves >= 8) PICK(2, 4, 8);
+  PICK(2, 4, 4);
+#undef PICK
+}

@@ -56,6 +56,7 @@ class HipOps:
         self._declare_core()
         self.num_cus = torch.cuda.get_device_properties(self.device).multi_processor_count
         self.use_library_gemm = True
+        self.use_skinny_gemm = True
         self._mm_out_dtype_ok: Optional[bool] = None
 
     # -- loading --------------------------------------------------------------------------------
@@ -66,6 +67,8 @@ class HipOps:
         c.velox_silu_mul.argtypes = [_P, _P, _I, _I, _I, _P]
         c.velox_rope_kv_write.argtypes = [_P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_gemm_fma.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_skinny_gemm_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
+        c.velox_skinny_gemm_bf16.restype = _I
         c.velox_argmax.argtypes = [_P, _P, _I, _I, _P]
         c.velox_sample.argtypes = [_P, _P, _P, _I, _I, _P]
         c.velox_apply_penalties.argtypes = [_P, _P, _P, _P, _I, _I, _I, _P]
@@ -159,6 +162,9 @@ class HipOps:
         n = weight.shape[0]
         if bias is not None:
             self._check("bias", bias, torch.float32, (n,))
+        skinny_rows = 16 if n > 8192 else 32  # measured on MI355X: beyond this the library's kernels stream faster
+        if self.use_skinny_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and m <= skinny_rows and k % 64 == 0:
+            return self.skinny_gemm(x, weight, bias, out_dtype)
         if self.use_library_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and bias is None:
             if out_dtype == torch.bfloat16:
                 return torch.nn.functional.linear(x, weight)
@@ -170,6 +176,22 @@ class HipOps:
                 except (RuntimeError, TypeError):
                     self._mm_out_dtype_ok = False
         return self.gemm_fma(x, weight, bias, out_dtype)
+
+    def skinny_gemm(self, x, weight, bias, out_dtype, waves: Optional[int] = None):
+        """Few rows (M <= 64) times a bfloat16 weight: the weight-streaming kernel of the decode step."""
+        m, k = x.shape
+        n = weight.shape[0]
+        if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or m > 64 or k % 64 != 0:
+            raise KernelError(f"skinny_gemm: needs bfloat16 operands, M <= 64 and K % 64 == 0 (M={m}, K={k})")
+        if waves is None:
+            rows_per_block = 16 if m <= 16 else 32
+            blocks = (n + rows_per_block - 1) // rows_per_block
+            wanted = (8 * self.num_cus + blocks - 1) // blocks  # about eight waves per SIMD lane group across the GPU
+            waves = 16 if wanted > 8 else 8 if wanted > 4 else 4
+        out = torch.empty((m, n), dtype=out_dtype, device=self.device)
+        status = self._core.velox_skinny_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), m, n, k, _code(out_dtype), int(waves), self._stream())
+        self._launched(status, "skinny_gemm")
+        return out
 
     def gemm_fma(self, x, weight, bias, out_dtype):
         m, k = x.shape
