@@ -319,9 +319,9 @@ def test_skinny_gemm(ops, ref, out_dtype, m, n, k):
     bias = rand((n,), torch.float32, 42)
     want = ref.linear(x, w, None, torch.float32)
     scale = float(want.abs().max())
-    for waves in (None, 4, 8, 16):
+    for waves, row_tiles in ((None, None), (4, 1), (8, 1), (16, 1), (4, 4), (8, 4)):
         for b in (None, bias):
-            got = ops.skinny_gemm(x, w, b, out_dtype, waves=waves).float()
+            got = ops.skinny_gemm(x, w, b, out_dtype, waves=waves, row_tiles=row_tiles).float()
             expect = want + (b if b is not None else 0)
             atol = 1e-4 * scale if out_dtype == torch.float32 else 1e-2 * scale
             torch.testing.assert_close(got, expect, rtol=1e-2 if out_dtype == torch.bfloat16 else 1e-4, atol=atol)

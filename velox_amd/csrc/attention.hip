@@ -85,7 +85,10 @@ __device__ __forceinline__ void mask_tail(Vec16<bf16_t>& x, int valid) {
   }
 }
 
-template <typename T, int BN>
+// KEY_SPLIT = false: each of the 4 waves owns 16 of the workgroup's 64 rows and visits every key of a tile.
+// KEY_SPLIT = true (at most 16 rows per sequence and KV head, i.e. decode): every wave owns the same rows and
+// visits its own quarter of each tile's keys; the four partial results are merged through LDS at the end.
+template <typename T, int BN, bool KEY_SPLIT>
 __global__ void __launch_bounds__(256) paged_attention_kernel(
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
@@ -97,8 +100,14 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
   constexpr int VEC = 16 / sizeof(T);
   constexpr int NT = BN / 16;
   constexpr int NC = D / 16;
-  __shared__ __attribute__((aligned(16))) T k_tile[BN * KS];
-  __shared__ __attribute__((aligned(16))) T v_tile[D * VS];
+  constexpr int NTW = KEY_SPLIT ? (NT + 3) / 4 : NT;  // key tiles of 16 a wave computes per staged tile
+  constexpr int NCW = KEY_SPLIT ? (NC + 3) / 4 : NC;  // channel blocks a wave writes out
+  constexpr int TILE_BYTES = (BN * KS + D * VS) * (int)sizeof(T);
+  constexpr int MERGE_BYTES = KEY_SPLIT ? (4 * NC * 64 * 16 + 2 * 4 * 16 * 4) : 0;
+  constexpr int SMEM_BYTES = TILE_BYTES > MERGE_BYTES ? TILE_BYTES : MERGE_BYTES;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
+  T* k_tile = reinterpret_cast<T*>(smem);
+  T* v_tile = k_tile + BN * KS;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -116,7 +125,7 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
   const int r0 = blockIdx.x * ROWS_PER_BLOCK;
   if (r0 >= rows_total) return;
 
-  const int r = r0 + wave * 16 + i;
+  const int r = r0 + (KEY_SPLIT ? 0 : wave * 16) + i;
   const bool row_ok = r < rows_total;
   const int tok = row_ok ? r / group : 0;
   const int head = kvh * group + (row_ok ? r % group : 0);
@@ -162,103 +171,126 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
 
   const int* table = block_tables + (size_t)b * table_width;
 
-  for (int tile = tile_lo; tile < tile_hi; ++tile) {
-    const int n0 = n_begin + tile * BN;
-    __syncthreads();
-    // ---- stage K[n0 .. n0+BN) as [key][channel] -------------------------------------------
-    {
-      constexpr int VPR = D / VEC;
-      for (int v = tid; v < BN * VPR; v += 256) {
+  // ---- staging: global -> registers (issued a tile ahead) -> LDS ------------------------------
+  constexpr int VPR = D / VEC;              // vectors per key row of K
+  constexpr int VECS = BN * D / VEC;        // vectors per tile (K and V^T alike)
+  constexpr int ITERS = (VECS + 255) / 256;
+  const int run = page_size < BN ? page_size : BN;  // consecutive keys that are contiguous in a page of V
+  const bool v_by_vectors = run >= VEC;
+  const int vpr_v = v_by_vectors ? run / VEC : 1;
+  const int per_run = D * vpr_v;
+  float4_t k_regs[ITERS], v_regs[ITERS];
+
+  auto fetch = [&](int n0) {
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int v = tid + it * 256;
+      k_regs[it] = float4_t{0.f, 0.f, 0.f, 0.f};
+      v_regs[it] = float4_t{0.f, 0.f, 0.f, 0.f};
+      if (v >= VECS) continue;
+      {
         const int key = v / VPR, vec = v % VPR;
         const int n = n0 + key;
-        Vec16<T> x;
-        x.v = float4_t{0.f, 0.f, 0.f, 0.f};
         if (n < kv_len) {
           const size_t page = (size_t)table[n >> page_shift];
           const int off = n & (page_size - 1);
-          x.v = *reinterpret_cast<const float4_t*>(k_cache + ((page * nkv + kvh) * page_size + off) * D + vec * VEC);
+          k_regs[it] = *reinterpret_cast<const float4_t*>(k_cache + ((page * nkv + kvh) * page_size + off) * D + vec * VEC);
         }
-        *reinterpret_cast<float4_t*>(k_tile + key * KS + vec * VEC) = x.v;
       }
-    }
-    // ---- stage V^T[n0 .. n0+BN) as [channel][key] -----------------------------------------
-    {
-      const int run = page_size < BN ? page_size : BN;  // consecutive keys that are contiguous in a page
-      if (run >= VEC) {
-        const int vpr = run / VEC;
-        const int per_run = D * vpr;
-        for (int v = tid; v < BN * D / VEC; v += 256) {
-          const int rn = v / per_run, rem = v % per_run;
-          const int dd = rem / vpr, vec = rem % vpr;
-          const int nl = rn * run + vec * VEC;
-          const int n = n0 + nl;
+      if (v_by_vectors) {
+        const int rn = v / per_run, rem = v % per_run;
+        const int dd = rem / vpr_v, vec = rem % vpr_v;
+        const int n = n0 + rn * run + vec * VEC;
+        if (n < kv_len) {
+          const size_t page = (size_t)table[n >> page_shift];
+          const int off = n & (page_size - 1);
           Vec16<T> x;
-          x.v = float4_t{0.f, 0.f, 0.f, 0.f};
-          if (n < kv_len) {
-            const size_t page = (size_t)table[n >> page_shift];
-            const int off = n & (page_size - 1);
-            x.v = *reinterpret_cast<const float4_t*>(v_cache + ((page * nkv + kvh) * D + dd) * page_size + off);
-            if (n + VEC > kv_len) mask_tail(x, kv_len - n);
-          }
-          *reinterpret_cast<float4_t*>(v_tile + dd * VS + nl) = x.v;
-        }
-      } else {
-        const int per_run = D * run;
-        for (int v = tid; v < BN * D; v += 256) {
-          const int rn = v / per_run, rem = v % per_run;
-          const int dd = rem / run, e = rem % run;
-          const int nl = rn * run + e;
-          const int n = n0 + nl;
-          T x = from_f32<T>(0.f);
-          if (n < kv_len) {
-            const size_t page = (size_t)table[n >> page_shift];
-            const int off = n & (page_size - 1);
-            x = v_cache[((page * nkv + kvh) * D + dd) * page_size + off];
-          }
-          v_tile[dd * VS + nl] = x;
+          x.v = *reinterpret_cast<const float4_t*>(v_cache + ((page * nkv + kvh) * D + dd) * page_size + off);
+          if (n + VEC > kv_len) mask_tail(x, kv_len - n);
+          v_regs[it] = x.v;
         }
       }
     }
+  };
+  auto commit = [&](int n0) {
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int v = tid + it * 256;
+      if (v >= VECS) continue;
+      *reinterpret_cast<float4_t*>(k_tile + (v / VPR) * KS + (v % VPR) * VEC) = k_regs[it];
+      if (v_by_vectors) {
+        const int rn = v / per_run, rem = v % per_run;
+        *reinterpret_cast<float4_t*>(v_tile + (rem / vpr_v) * VS + rn * run + (rem % vpr_v) * VEC) = v_regs[it];
+      }
+    }
+    if (!v_by_vectors) {  // pages shorter than a vector: element by element, straight from global memory
+      const int per = D * run;
+      for (int v = tid; v < BN * D; v += 256) {
+        const int rn = v / per, rem = v % per;
+        const int dd = rem / run, e = rem % run;
+        const int nl = rn * run + e;
+        const int n = n0 + nl;
+        T x = from_f32<T>(0.f);
+        if (n < kv_len) {
+          const size_t page = (size_t)table[n >> page_shift];
+          x = v_cache[((page * nkv + kvh) * D + dd) * page_size + (n & (page_size - 1))];
+        }
+        v_tile[dd * VS + nl] = x;
+      }
+    }
+  };
+
+  if (tile_lo < tile_hi) fetch(n_begin + tile_lo * BN);
+  for (int tile = tile_lo; tile < tile_hi; ++tile) {
+    const int n0 = n_begin + tile * BN;
+    __syncthreads();  // the previous tile has been read by every wave
+    commit(n0);
     __syncthreads();
-    if (n0 > wave_last_pos) continue;  // nothing this wave may read; it still took part in the staging
+    if (tile + 1 < tile_hi) fetch(n0 + BN);  // in flight while this tile is computed
+    if (n0 > wave_last_pos) continue;        // nothing this wave may read; it still took part in the staging
 
     // ---- S^T = K Q^T ----------------------------------------------------------------------
-    float4_t s[NT];
+    float4_t s[NTW];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      s[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int tt = 0; tt < NTW; ++tt) {
+      const int t = KEY_SPLIT ? wave + 4 * tt : tt;
+      s[tt] = float4_t{0.f, 0.f, 0.f, 0.f};
+      if (t < NT) {
 #pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        const Frag<T> a = load_frag<T>(k_tile + (16 * t + i) * KS + 16 * c + 4 * g);
-        s[t] = mma16(a, qf[c], s[t]);
+        for (int c = 0; c < NC; ++c) {
+          const Frag<T> a = load_frag<T>(k_tile + (16 * t + i) * KS + 16 * c + 4 * g);
+          s[tt] = mma16(a, qf[c], s[tt]);
+        }
       }
     }
     // ---- mask, running maximum ------------------------------------------------------------
     float mx = -INFINITY;
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
+    for (int tt = 0; tt < NTW; ++tt) {
+      const int t = KEY_SPLIT ? wave + 4 * tt : tt;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int n = n0 + 16 * t + 4 * g + j;
-        const bool keep = row_ok && n < kv_len && n <= pos && (window <= 0 || n > pos - window);
-        const float val = keep ? s[t][j] * scale : -INFINITY;
-        s[t][j] = val;
+        const bool keep = row_ok && t < NT && n < kv_len && n <= pos && (window <= 0 || n > pos - window);
+        const float val = keep ? s[tt][j] * scale : -INFINITY;
+        s[tt][j] = val;
         mx = fmaxf(mx, val);
       }
+    }
     mx = fmaxf(mx, __shfl_xor(mx, 16, VELOX_WAVE));
     mx = fmaxf(mx, __shfl_xor(mx, 32, VELOX_WAVE));
     const float m_new = fmaxf(m_i, mx);
     const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
     const float alpha = (m_i == -INFINITY) ? 0.f : softmax_exp<T>(m_i - m_safe);
     float psum = 0.f;
-    Frag<T> pf[NT];
+    Frag<T> pf[NTW];
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
+    for (int tt = 0; tt < NTW; ++tt)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float p = (s[t][j] == -INFINITY) ? 0.f : softmax_exp<T>(s[t][j] - m_safe);
+        const float p = (s[tt][j] == -INFINITY) ? 0.f : softmax_exp<T>(s[tt][j] - m_safe);
         psum += p;
-        set_prob(pf[t], j, p);
+        set_prob(pf[tt], j, p);
       }
     l_i = l_i * alpha + psum;  // partial over this lane's keys; the four lane groups are summed at the end
     m_i = m_new;
@@ -267,32 +299,276 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
     for (int c = 0; c < NC; ++c) {
       acc_o[c] = acc_o[c] * alpha;
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        const Frag<T> a = load_frag<T>(v_tile + (16 * c + i) * VS + 16 * t + 4 * g);
-        acc_o[c] = mma16(a, pf[t], acc_o[c]);
+      for (int tt = 0; tt < NTW; ++tt) {
+        const int t = KEY_SPLIT ? wave + 4 * tt : tt;
+        if (t < NT) {
+          const Frag<T> a = load_frag<T>(v_tile + (16 * c + i) * VS + 16 * t + 4 * g);
+          acc_o[c] = mma16(a, pf[tt], acc_o[c]);
+        }
       }
     }
   }
 
   l_i += __shfl_xor(l_i, 16, VELOX_WAVE);
   l_i += __shfl_xor(l_i, 32, VELOX_WAVE);
+
+  if constexpr (KEY_SPLIT) {
+    // merge the four waves: out = sum_w e^(m_w - m) acc_w / sum_w e^(m_w - m) l_w
+    float4_t* acc_all = reinterpret_cast<float4_t*>(smem);                     // [4][NC][64]
+    float* m_all = reinterpret_cast<float*>(smem + 4 * NC * 64 * 16);          // [4][16]
+    float* l_all = m_all + 4 * 16;                                             // [4][16]
+    __syncthreads();  // the tiles are no longer read
+#pragma unroll
+    for (int c = 0; c < NC; ++c) acc_all[(wave * NC + c) * 64 + lane] = acc_o[c];
+    if (g == 0) { m_all[wave * 16 + i] = m_i; l_all[wave * 16 + i] = l_i; }
+    __syncthreads();
+    float m_tot = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) m_tot = fmaxf(m_tot, m_all[w * 16 + i]);
+    const float m_ref = (m_tot == -INFINITY) ? 0.f : m_tot;
+    float weight[4];
+    float l_tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float mw = m_all[w * 16 + i];
+      weight[w] = (mw == -INFINITY) ? 0.f : softmax_exp<T>(mw - m_ref);
+      l_tot += weight[w] * l_all[w * 16 + i];
+    }
+    m_i = m_tot;
+    l_i = l_tot;
+#pragma unroll
+    for (int cc = 0; cc < NCW; ++cc) {
+      const int c = wave + 4 * cc;
+      if (c < NC) {
+        float4_t sum = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < 4; ++w) sum += acc_all[(w * NC + c) * 64 + lane] * weight[w];
+        acc_o[cc] = sum;  // from here on acc_o[cc] is channel block wave + 4 cc
+      }
+    }
+  }
+
   if (!row_ok) return;
   const float inv = l_i > 0.f ? 1.f / l_i : 1.f;
   const size_t token = (size_t)(q_start + tok);
   if (splits == 1) {
     T* dst = out + (token * nh + head) * D + 4 * g;
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
+    for (int cc = 0; cc < NCW; ++cc) {
+      const int c = KEY_SPLIT ? wave + 4 * cc : cc;
+      if (c < NC) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) dst[16 * c + j] = from_f32<T>(acc_o[c][j] * inv);
+        for (int j = 0; j < 4; ++j) dst[16 * c + j] = from_f32<T>(acc_o[cc][j] * inv);
+      }
     }
   } else {
     const size_t slot = ((size_t)split * total_tokens + token) * nh + head;
     float* dst = part_o + slot * D + 4 * g;
 #pragma unroll
-    for (int c = 0; c < NC; ++c) *reinterpret_cast<float4_t*>(dst + 16 * c) = acc_o[c] * inv;
-    if (g == 0) part_lse[slot] = l_i > 0.f ? m_i + logf(l_i) : -INFINITY;
+    for (int cc = 0; cc < NCW; ++cc) {
+      const int c = KEY_SPLIT ? wave + 4 * cc : cc;
+      if (c < NC) *reinterpret_cast<float4_t*>(dst + 16 * c) = acc_o[cc] * inv;
+    }
+    if (g == 0 && (!KEY_SPLIT || wave == 0)) part_lse[slot] = l_i > 0.f ? m_i + logf(l_i) : -INFINITY;
   }
+}
+
+// Zeroes the elements of a 4-key fragment whose key index is not below `valid`.
+__device__ __forceinline__ void mask_frag(Frag<float>& f, int valid) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) f.v[j] = j < valid ? f.v[j] : 0.f;
+}
+__device__ __forceinline__ void mask_frag(Frag<bf16_t>& f, int valid) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) f.v[j] = j < valid ? f.v[j] : (short)0;
+}
+
+// Decode: every sequence brings one token, and the G <= 16 query heads of a KV head are the 16 columns of the
+// MFMA tiles.  The step is bound by reading the cache once, so nothing is staged: each wave streams its own
+// 16-key tiles straight from global memory into MFMA operands (K rows as [key i][channels 16c + 4g ..], V^T rows
+// as [channel 16c + i][keys 4g ..], both 8- or 16-byte loads of contiguous cache lines), two tiles ahead of the
+// arithmetic, with no barrier in the loop.  The page ids of the workgroup's key range are copied into LDS first, so
+// that a tile's addresses do not wait for a second trip to memory.  The 4 waves of a workgroup interleave the
+// tiles of one (sequence, KV head, split) and merge their running (max, sum, output) through LDS at the end.
+constexpr int DECODE_PAGE_IDS = 2048;
+
+template <typename T>
+__global__ void __launch_bounds__(256) decode_attention_kernel(
+    const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int* __restrict__ block_tables, int table_width, const int* __restrict__ kv_lens,
+    T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
+    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens) {
+  constexpr int NC = D / 16;
+  constexpr int NCW = (NC + 3) / 4;
+  constexpr int DEPTH = sizeof(T) * D <= 256 ? 3 : 2;  // register sets: one being computed, the others in flight
+  __shared__ __attribute__((aligned(16))) float4_t acc_all[4 * NC * 64];
+  __shared__ float m_all[4 * 16];
+  __shared__ float l_all[4 * 16];
+  __shared__ int page_ids[DECODE_PAGE_IDS];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 4, i = lane & 15;
+  const int group = nh / nkv;
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int page_size = 1 << page_shift;
+  const int kv_len = kv_lens[b];
+  const int pos = kv_len - 1;
+  const bool row_ok = i < group;
+  const int head = kvh * group + (row_ok ? i : 0);
+
+  int n_begin = 0;
+  if (window > 0) {
+    n_begin = pos - window + 1;
+    if (n_begin < 0) n_begin = 0;
+    n_begin &= ~15;
+  }
+  const int tiles_total = (kv_len - n_begin + 15) / 16;
+  const int per_split = (tiles_total + splits - 1) / splits;
+  const int t_lo = split * per_split;
+  int t_hi = t_lo + per_split;
+  if (t_hi > tiles_total) t_hi = tiles_total;
+
+  const int* table = block_tables + (size_t)b * table_width;
+  // page ids of keys [n_begin + 16 t_lo, n_begin + 16 t_hi)
+  const int first_page = (n_begin + 16 * t_lo) >> page_shift;
+  const int last_key = n_begin + 16 * t_hi < kv_len ? n_begin + 16 * t_hi : kv_len;
+  const int num_pages = t_hi > t_lo ? ((last_key - 1) >> page_shift) - first_page + 1 : 0;
+  for (int p = tid; p < num_pages && p < DECODE_PAGE_IDS; p += 256) page_ids[p] = table[first_page + p];
+
+  Frag<T> qf[NC];
+  {
+    const T* qp = qkv + (size_t)b * qkv_stride + (size_t)head * D + 4 * g;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) qf[c] = row_ok ? load_frag<T>(qp + 16 * c) : zero_frag<T>();
+  }
+  __syncthreads();
+  auto page_of = [&](int n) -> size_t {
+    const int p = (n >> page_shift) - first_page;
+    return (size_t)(p < DECODE_PAGE_IDS ? page_ids[p] : table[first_page + p]);
+  };
+
+  struct Tile {
+    Frag<T> k[NC];
+    Frag<T> v[NC];
+  };
+  auto load_tile = [&](Tile& tile, int t) {
+    const int n_k = n_begin + 16 * t + i;      // the key whose row this lane reads
+    const int n_v = n_begin + 16 * t + 4 * g;  // the first of the four keys whose values this lane reads
+    if (n_k < kv_len) {
+      const T* kp = k_cache + ((page_of(n_k) * nkv + kvh) * page_size + (n_k & (page_size - 1))) * D + 4 * g;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) tile.k[c] = load_frag<T>(kp + 16 * c);
+    } else {
+#pragma unroll
+      for (int c = 0; c < NC; ++c) tile.k[c] = zero_frag<T>();
+    }
+    if (n_v < kv_len) {
+      const T* vp = v_cache + ((page_of(n_v) * nkv + kvh) * D + i) * page_size + (n_v & (page_size - 1));
+#pragma unroll
+      for (int c = 0; c < NC; ++c) tile.v[c] = load_frag<T>(vp + (size_t)16 * c * page_size);
+      if (n_v + 4 > kv_len) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) mask_frag(tile.v[c], kv_len - n_v);
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < NC; ++c) tile.v[c] = zero_frag<T>();
+    }
+  };
+
+  float m_i = -INFINITY, l_i = 0.f;
+  float4_t acc_o[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) acc_o[c] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  auto compute_tile = [&](const Tile& tile, int t) {
+    float4_t s = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < NC; ++c) s = mma16(tile.k[c], qf[c], s);
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n_begin + 16 * t + 4 * g + j;
+      const bool keep = row_ok && n < kv_len && (window <= 0 || n > pos - window);
+      s[j] = keep ? s[j] * scale : -INFINITY;
+      mx = fmaxf(mx, s[j]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, VELOX_WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, VELOX_WAVE));
+    const float m_new = fmaxf(m_i, mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = (m_i == -INFINITY) ? 0.f : softmax_exp<T>(m_i - m_safe);
+    Frag<T> pf;
+    float psum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float p = (s[j] == -INFINITY) ? 0.f : softmax_exp<T>(s[j] - m_safe);
+      psum += p;
+      set_prob(pf, j, p);
+    }
+    l_i = l_i * alpha + psum;
+    m_i = m_new;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) acc_o[c] = mma16(tile.v[c], pf, acc_o[c] * alpha);
+  };
+
+  // a ring of DEPTH register sets: while a tile is computed the next two are in flight
+  Tile ring[DEPTH];
+  const int t0 = t_lo + wave;
+#pragma unroll
+  for (int s = 0; s < DEPTH - 1; ++s)
+    if (t0 + 4 * s < t_hi) load_tile(ring[s], t0 + 4 * s);
+  for (int t = t0; t < t_hi; t += 4 * DEPTH) {
+#pragma unroll
+    for (int s = 0; s < DEPTH; ++s) {
+      const int tc = t + 4 * s;
+      if (tc < t_hi) {
+        const int tn = tc + 4 * (DEPTH - 1);
+        if (tn < t_hi) load_tile(ring[(s + DEPTH - 1) % DEPTH], tn);
+        compute_tile(ring[s], tc);
+      }
+    }
+  }
+
+  l_i += __shfl_xor(l_i, 16, VELOX_WAVE);
+  l_i += __shfl_xor(l_i, 32, VELOX_WAVE);
+#pragma unroll
+  for (int c = 0; c < NC; ++c) acc_all[(wave * NC + c) * 64 + lane] = acc_o[c];
+  if (g == 0) { m_all[wave * 16 + i] = m_i; l_all[wave * 16 + i] = l_i; }
+  __syncthreads();
+  float m_tot = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) m_tot = fmaxf(m_tot, m_all[w * 16 + i]);
+  const float m_ref = (m_tot == -INFINITY) ? 0.f : m_tot;
+  float weight[4];
+  float l_tot = 0.f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const float mw = m_all[w * 16 + i];
+    weight[w] = (mw == -INFINITY) ? 0.f : softmax_exp<T>(mw - m_ref);
+    l_tot += weight[w] * l_all[w * 16 + i];
+  }
+  if (!row_ok) return;
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 1.f;
+  const size_t slot = ((size_t)split * total_tokens + b) * nh + head;
+#pragma unroll
+  for (int cc = 0; cc < NCW; ++cc) {
+    const int c = wave + 4 * cc;  // this wave writes channel blocks wave, wave + 4, ...
+    if (c >= NC) break;
+    float4_t sum = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) sum += acc_all[(w * NC + c) * 64 + lane] * weight[w];
+    sum = sum * inv;
+    if (splits == 1) {
+      T* dst = out + ((size_t)b * nh + head) * D + 16 * c + 4 * g;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) dst[j] = from_f32<T>(sum[j]);
+    } else {
+      *reinterpret_cast<float4_t*>(part_o + slot * D + 16 * c + 4 * g) = sum;
+    }
+  }
+  if (splits > 1 && wave == 0 && g == 0) part_lse[slot] = l_tot > 0.f ? m_tot + logf(l_tot) : -INFINITY;
 }
 
 // out[token, head, :] = sum_s w_s * o_s / sum_s w_s,  w_s = exp(lse_s - max_s lse_s)
@@ -301,19 +577,23 @@ __global__ void merge_splits_kernel(const float* __restrict__ part_o, const floa
                                     int nh, int splits, int total_tokens) {
   const size_t token = blockIdx.x;
   const int head = blockIdx.y;
+  const size_t stride = (size_t)total_tokens * nh;  // slots per split
+  const size_t slot0 = token * nh + head;
   float mx = -INFINITY;
-  for (int s = 0; s < splits; ++s) mx = fmaxf(mx, part_lse[((size_t)s * total_tokens + token) * nh + head]);
+#pragma unroll 8
+  for (int s = 0; s < splits; ++s) mx = fmaxf(mx, part_lse[s * stride + slot0]);
   const float m_safe = (mx == -INFINITY) ? 0.f : mx;
   for (int dd = threadIdx.x; dd < D; dd += blockDim.x) {
     float acc = 0.f, denom = 0.f;
+#pragma unroll 8
     for (int s = 0; s < splits; ++s) {
-      const size_t slot = ((size_t)s * total_tokens + token) * nh + head;
+      const size_t slot = s * stride + slot0;
       const float lse = part_lse[slot];
       const float w = (lse == -INFINITY) ? 0.f : expf(lse - m_safe);
       acc += w * part_o[slot * D + dd];
       denom += w;
     }
-    out[(token * nh + head) * D + dd] = from_f32<T>(acc / (denom > 0.f ? denom : 1.f));
+    out[slot0 * D + dd] = from_f32<T>(acc / (denom > 0.f ? denom : 1.f));
   }
 }
 
@@ -325,11 +605,26 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
                   int max_q_len, int nh, int nkv, int page_shift, float scale, int window, int splits, hipStream_t stream) {
   constexpr int BN = tile_keys<T>();
   const int group = nh / nkv;
+  if (max_q_len == 1 && total_tokens == num_seqs && group <= 16 && page_shift >= 2 && sizeof(T) * D <= 512) {
+    // every sequence decodes one token: the streaming kernel
+    decode_attention_kernel<T><<<dim3(splits, nkv, num_seqs), 256, 0, stream>>>(
+        (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, kv_lens, (T*)out, part_o, part_lse,
+        nh, nkv, page_shift, scale, window, splits, total_tokens);
+    int status = (int)hipGetLastError();
+    if (status != 0 || splits == 1) return status;
+    merge_splits_kernel<T><<<dim3(total_tokens, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens);
+    return (int)hipGetLastError();
+  }
   const int row_tiles = (max_q_len * group + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
   dim3 grid(row_tiles, nkv, num_seqs * splits);
-  paged_attention_kernel<T, BN><<<grid, 256, 0, stream>>>(
-      (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-      part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
+  if (max_q_len * group <= 16)
+    paged_attention_kernel<T, BN, true><<<grid, 256, 0, stream>>>(
+        (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
+  else
+    paged_attention_kernel<T, BN, false><<<grid, 256, 0, stream>>>(
+        (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
   int status = (int)hipGetLastError();
   if (status != 0 || splits == 1) return status;
   merge_splits_kernel<T><<<dim3(total_tokens, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens);

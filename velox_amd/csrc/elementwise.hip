@@ -60,11 +60,76 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
   }
 }
 
+// Same arithmetic with the row held in registers: one read of residual and delta, 16-byte accesses.  Needs
+// hidden % 4 == 0 and hidden <= 4 * threads * CHUNKS.
+template <typename T> struct Quad;
+template <> struct Quad<float> {
+  float4_t v;
+  __device__ __forceinline__ float get(int i) const { return v[i]; }
+  __device__ __forceinline__ void set(int i, float x) { v[i] = x; }
+};
+template <> struct Quad<bf16_t> {
+  short4_t v;
+  __device__ __forceinline__ float get(int i) const { return __uint_as_float(((uint32_t)(uint16_t)v[i]) << 16); }
+  __device__ __forceinline__ void set(int i, float x) { v[i] = bf16_bits(x); }
+};
+
+template <typename TD, typename TO, int CHUNKS>
+__global__ void add_rmsnorm_rows_in_registers_kernel(float* __restrict__ residual, const TD* __restrict__ delta, const int* __restrict__ rows,
+                                                     const float* __restrict__ weight, TO* __restrict__ out, int hidden, float eps) {
+  __shared__ float scratch[16];
+  const int row = blockIdx.x;
+  const size_t src_row = rows ? (size_t)rows[row] : (size_t)row;
+  float* res = residual + src_row * hidden;
+  const TD* del = delta ? delta + src_row * hidden : nullptr;
+  const bool write_back = (rows == nullptr) && (delta != nullptr);
+  float4_t r[CHUNKS];
+  float sumsq = 0.f;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int at = (threadIdx.x + c * blockDim.x) * 4;
+    r[c] = float4_t{0.f, 0.f, 0.f, 0.f};
+    if (at < hidden) {
+      r[c] = *reinterpret_cast<const float4_t*>(res + at);
+      if (del) {
+        const Quad<TD> d = *reinterpret_cast<const Quad<TD>*>(del + at);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r[c][j] += d.get(j);
+      }
+      if (write_back) *reinterpret_cast<float4_t*>(res + at) = r[c];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sumsq += r[c][j] * r[c][j];
+    }
+  }
+  const float total = block_sum(sumsq, scratch);
+  const float inv = rsqrtf(total / (float)hidden + eps);
+  TO* dst = out + (size_t)row * hidden;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int at = (threadIdx.x + c * blockDim.x) * 4;
+    if (at < hidden) {
+      const float4_t w = *reinterpret_cast<const float4_t*>(weight + at);
+      Quad<TO> o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o.set(j, r[c][j] * inv * w[j]);
+      *reinterpret_cast<Quad<TO>*>(dst + at) = o;
+    }
+  }
+}
+
 extern "C" int velox_add_rmsnorm(float* residual, const void* delta, const int* rows, const float* weight, void* out,
                                  int num_rows, int hidden, float eps, int delta_dtype, int out_dtype, hipStream_t stream) {
   if (num_rows <= 0) return 0;
   const int threads = hidden >= 2048 ? 512 : 256;
-#define LAUNCH(TD, TO) add_rmsnorm_kernel<TD, TO><<<num_rows, threads, 0, stream>>>(residual, (const TD*)delta, rows, weight, (TO*)out, hidden, eps)
+  const bool aligned = (((uintptr_t)residual | (uintptr_t)delta | (uintptr_t)weight | (uintptr_t)out) & 15) == 0;
+  const bool in_registers = aligned && hidden % 4 == 0 && hidden <= 4 * threads * 4;
+#define LAUNCH(TD, TO)                                                                                                                  \
+  do {                                                                                                                                  \
+    if (in_registers)                                                                                                                   \
+      add_rmsnorm_rows_in_registers_kernel<TD, TO, 4><<<num_rows, threads, 0, stream>>>(residual, (const TD*)delta, rows, weight, (TO*)out, hidden, eps); \
+    else                                                                                                                                \
+      add_rmsnorm_kernel<TD, TO><<<num_rows, threads, 0, stream>>>(residual, (const TD*)delta, rows, weight, (TO*)out, hidden, eps);    \
+  } while (0)
   if (delta_dtype == VELOX_BF16 && out_dtype == VELOX_BF16) LAUNCH(bf16_t, bf16_t);
   else if (delta_dtype == VELOX_F32 && out_dtype == VELOX_F32) LAUNCH(float, float);
   else if (delta_dtype == VELOX_BF16 && out_dtype == VELOX_F32) LAUNCH(bf16_t, float);
@@ -88,8 +153,40 @@ __global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ o
   }
 }
 
+// 16-byte accesses; needs inter % (16 / sizeof(T)) == 0.
+template <typename T>
+__global__ void silu_mul_vec_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter) {
+  constexpr int N = 16 / sizeof(T);
+  const int t = blockIdx.y;
+  const T* row = gate_up + (size_t)t * 2 * inter;
+  T* dst = out + (size_t)t * inter;
+  for (int at = (blockIdx.x * blockDim.x + threadIdx.x) * N; at < inter; at += gridDim.x * blockDim.x * N) {
+    const float4_t gv = *reinterpret_cast<const float4_t*>(row + at);
+    const float4_t uv = *reinterpret_cast<const float4_t*>(row + inter + at);
+    float4_t ov;
+    const T* ge = reinterpret_cast<const T*>(&gv);
+    const T* ue = reinterpret_cast<const T*>(&uv);
+    T* oe = reinterpret_cast<T*>(&ov);
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      const float g = to_f32(ge[j]);
+      oe[j] = from_f32<T>(g / (1.f + expf(-g)) * to_f32(ue[j]));
+    }
+    *reinterpret_cast<float4_t*>(dst + at) = ov;
+  }
+}
+
 extern "C" int velox_silu_mul(const void* gate_up, void* out, int tokens, int inter, int dtype, hipStream_t stream) {
   if (tokens <= 0) return 0;
+  const int per = dtype == VELOX_BF16 ? 8 : 4;
+  if (inter % per == 0 && (((uintptr_t)gate_up | (uintptr_t)out) & 15) == 0) {
+    int bx = (inter / per + 255) / 256;
+    if (bx > 32) bx = 32;
+    dim3 grid(bx, tokens);
+    if (dtype == VELOX_BF16) silu_mul_vec_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, inter);
+    else silu_mul_vec_kernel<float><<<grid, 256, 0, stream>>>((const float*)gate_up, (float*)out, inter);
+    VELOX_RETURN_LAUNCH_STATUS();
+  }
   int bx = (inter + 255) / 256;
   if (bx > 64) bx = 64;
   dim3 grid(bx, tokens);
@@ -173,10 +270,88 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
   }
 }
 
+// The same with 16-byte accesses, for the usual case that the whole head rotates (2 * half == d) or nothing does.
+// An item is a run of N = 16 / sizeof(T) channels of the low half of a head together with the matching run of the high half.
+template <typename T>
+__global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, const float* __restrict__ bias, const int* __restrict__ positions,
+                                         const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+                                         const int* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                         int nh, int nkv, int d, int page_size, int write_kv) {
+  constexpr int N = 16 / sizeof(T);
+  const int t = blockIdx.x;
+  const int half = d / 2;
+  const int width = (nh + 2 * nkv) * d;
+  T* row = qkv + (size_t)t * width;
+  const int pos = positions[t];
+  const float* cs = cos_table ? cos_table + (size_t)pos * half : nullptr;
+  const float* sn = sin_table ? sin_table + (size_t)pos * half : nullptr;
+  const int slot = slots[t];
+  const size_t page = (size_t)(slot / page_size);
+  const int offset = slot % page_size;
+  const int runs = half / N;
+  const int q_items = nh * runs;
+  const int k_items = write_kv ? nkv * runs : 0;
+  for (int item = threadIdx.x; item < q_items + k_items; item += blockDim.x) {
+    const bool is_k = item >= q_items;
+    const int local = is_k ? item - q_items : item;
+    const int head = local / runs;
+    const int c0 = (local % runs) * N;
+    const int base = (is_k ? nh * d : 0) + head * d;
+    float4_t lo_v = *reinterpret_cast<const float4_t*>(row + base + c0);
+    float4_t hi_v = *reinterpret_cast<const float4_t*>(row + base + half + c0);
+    T* lo = reinterpret_cast<T*>(&lo_v);
+    T* hi = reinterpret_cast<T*>(&hi_v);
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      float x0 = to_f32(lo[j]), x1 = to_f32(hi[j]);
+      if (bias) { x0 += bias[base + c0 + j]; x1 += bias[base + half + c0 + j]; }
+      float y0 = x0, y1 = x1;
+      if (cs) {
+        const float c = cs[c0 + j], s = sn[c0 + j];
+        y0 = x0 * c - x1 * s;
+        y1 = x0 * s + x1 * c;
+      }
+      lo[j] = from_f32<T>(y0);
+      hi[j] = from_f32<T>(y1);
+    }
+    T* dst = is_k ? k_cache + ((page * nkv + head) * page_size + offset) * d : row + base;
+    *reinterpret_cast<float4_t*>(dst + c0) = lo_v;
+    *reinterpret_cast<float4_t*>(dst + half + c0) = hi_v;
+  }
+  if (write_kv) {
+    const int v_base = (nh + nkv) * d;
+    for (int item = threadIdx.x; item < nkv * d / N; item += blockDim.x) {
+      const int at = item * N;
+      const int head = at / d, c = at % d;
+      float4_t v = *reinterpret_cast<const float4_t*>(row + v_base + at);
+      const T* e = reinterpret_cast<const T*>(&v);
+      T* dst = v_cache + ((page * nkv + head) * d + c) * page_size + offset;
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        float x = to_f32(e[j]);
+        if (bias) x += bias[v_base + at + j];
+        dst[(size_t)j * page_size] = from_f32<T>(x);
+      }
+    }
+  }
+}
+
 extern "C" int velox_rope_kv_write(void* qkv, const float* bias, const int* positions, const float* cos_table, const float* sin_table,
                                    int half, const int* slots, void* k_cache, void* v_cache, int tokens, int nh, int nkv, int d,
                                    int page_size, int write_kv, int dtype, hipStream_t stream) {
   if (tokens <= 0) return 0;
+  const int per = dtype == VELOX_BF16 ? 8 : 4;
+  const bool whole_head = (cos_table == nullptr || 2 * half == d) && (d / 2) % per == 0;
+  const bool aligned = (((uintptr_t)qkv | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0;
+  if (whole_head && aligned) {
+    if (dtype == VELOX_BF16)
+      rope_kv_write_vec_kernel<bf16_t><<<tokens, 256, 0, stream>>>((bf16_t*)qkv, bias, positions, cos_table, sin_table, slots,
+                                                                  (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, page_size, write_kv);
+    else
+      rope_kv_write_vec_kernel<float><<<tokens, 256, 0, stream>>>((float*)qkv, bias, positions, cos_table, sin_table, slots,
+                                                                 (float*)k_cache, (float*)v_cache, nh, nkv, d, page_size, write_kv);
+    VELOX_RETURN_LAUNCH_STATUS();
+  }
   if (dtype == VELOX_BF16)
     rope_kv_write_kernel<bf16_t><<<tokens, 256, 0, stream>>>((bf16_t*)qkv, bias, positions, cos_table, sin_table, half, slots,
                                                             (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, page_size, write_kv);

@@ -48,10 +48,18 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) argmax_kernel(const float* __r
   __shared__ Best scratch[16];
   const float* row = logits + (size_t)blockIdx.x * vocab;
   Best best{-INFINITY, 0x7fffffff};
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-    const float v = row[i];
-    if (v > best.value || best.index == 0x7fffffff) best = Best{v, i};
+  // 16-byte loads over the aligned middle of the row, single elements at its ends
+  const int head = (int)((16 - ((uintptr_t)row & 15)) & 15) / 4;
+  const int first = head < vocab ? head : vocab;
+  const int quads = (vocab - first) / 4;
+  for (int i = threadIdx.x; i < first; i += blockDim.x) best = better(best, Best{row[i], i});
+  const float4_t* body = reinterpret_cast<const float4_t*>(row + first);
+  for (int q = threadIdx.x; q < quads; q += blockDim.x) {
+    const float4_t v = body[q];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) best = better(best, Best{v[j], first + 4 * q + j});
   }
+  for (int i = first + 4 * quads + threadIdx.x; i < vocab; i += blockDim.x) best = better(best, Best{row[i], i});
   best = block_best(best, scratch);
   if (threadIdx.x == 0) out[blockIdx.x] = best.index;
 }

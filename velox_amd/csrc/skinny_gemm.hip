@@ -138,11 +138,17 @@ static int launch_skinny(const void* a, const void* w, const float* bias, void* 
 
 // waves: how many waves of a workgroup split K (4, 8 or 16; rounded down to what the tile shape allows); the
 // caller picks it so that the launch fills the GPU.
+// row_tiles: 16-row tiles of W per wave for M <= 16 (1 or 4).  With 4 a wave reuses each activation fragment for 64 rows
+// of W, which quarters the traffic of the activations; worth it when N is large enough that N / 64 workgroups still fill the GPU.
 extern "C" int velox_skinny_gemm_bf16(const void* a, const void* w, const float* bias, void* out, int m, int n, int k, int out_dtype,
-                                      int waves, hipStream_t stream) {
+                                      int waves, int row_tiles, hipStream_t stream) {
   if (m <= 0 || n <= 0) return 0;
   if (k % 64 != 0 || m > 64) return -1;
 #define PICK(RT, CT, W) return launch_skinny<RT, CT, W>(a, w, bias, out, m, n, k, out_dtype, stream)
+  if (m <= 16 && row_tiles >= 4) {
+    if (waves >= 8) PICK(4, 1, 8);
+    PICK(4, 1, 4);
+  }
   if (m <= 16) {
     if (waves >= 16) PICK(1, 1, 16);
     if (waves >= 8) PICK(1, 1, 8);

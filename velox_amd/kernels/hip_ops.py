@@ -67,7 +67,7 @@ class HipOps:
         c.velox_silu_mul.argtypes = [_P, _P, _I, _I, _I, _P]
         c.velox_rope_kv_write.argtypes = [_P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_gemm_fma.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
-        c.velox_skinny_gemm_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
+        c.velox_skinny_gemm_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
         c.velox_skinny_gemm_bf16.restype = _I
         c.velox_argmax.argtypes = [_P, _P, _I, _I, _P]
         c.velox_sample.argtypes = [_P, _P, _P, _I, _I, _P]
@@ -177,19 +177,21 @@ class HipOps:
                     self._mm_out_dtype_ok = False
         return self.gemm_fma(x, weight, bias, out_dtype)
 
-    def skinny_gemm(self, x, weight, bias, out_dtype, waves: Optional[int] = None):
+    def skinny_gemm(self, x, weight, bias, out_dtype, waves: Optional[int] = None, row_tiles: Optional[int] = None):
         """Few rows (M <= 64) times a bfloat16 weight: the weight-streaming kernel of the decode step."""
         m, k = x.shape
         n = weight.shape[0]
         if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or m > 64 or k % 64 != 0:
             raise KernelError(f"skinny_gemm: needs bfloat16 operands, M <= 64 and K % 64 == 0 (M={m}, K={k})")
+        if row_tiles is None:
+            row_tiles = 4 if (m <= 16 and n >= 64 * 2 * self.num_cus) else 1
         if waves is None:
-            rows_per_block = 16 if m <= 16 else 32
+            rows_per_block = 16 * row_tiles if m <= 16 else 32
             blocks = (n + rows_per_block - 1) // rows_per_block
             wanted = (8 * self.num_cus + blocks - 1) // blocks  # about eight waves per SIMD lane group across the GPU
             waves = 16 if wanted > 8 else 8 if wanted > 4 else 4
         out = torch.empty((m, n), dtype=out_dtype, device=self.device)
-        status = self._core.velox_skinny_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), m, n, k, _code(out_dtype), int(waves), self._stream())
+        status = self._core.velox_skinny_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), m, n, k, _code(out_dtype), int(waves), int(row_tiles), self._stream())
         self._launched(status, "skinny_gemm")
         return out
 
