@@ -39,13 +39,20 @@ def test_head_dim_key_wins_over_quotient():
     ({"hidden_size": 66}, "divisible"),
     ({"vocab_size": None}, "vocab_size"),
     ({"architectures": ["LlamaForCausalLM"]}, "unknown architecture"),
-    ({"architectures": []}, "architectures"),
+    ({"architectures": [], "model_type": None}, "architectures"),
 ])
 def test_refuses_what_it_does_not_implement(change, fragment):
     raw = {**TINY_A, **change}
     with pytest.raises(ConfigError) as err:
         config_from_dict(raw)
     assert fragment in str(err.value)
+
+
+def test_model_type_stands_in_for_a_missing_class_name():
+    raw = {k: v for k, v in TINY_A.items() if k != "architectures"}
+    assert config_from_dict(raw).architecture == "Qwen2ForCausalLM"
+    with pytest.raises(ConfigError):
+        config_from_dict({**raw, "model_type": "other"})
 
 
 def test_unknown_architecture_lists_known_ones():

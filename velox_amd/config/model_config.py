@@ -31,11 +31,18 @@ def read_config_json(model_dir: str) -> Dict[str, Any]:
     return raw
 
 
+# model classes by "model_type", for a config.json that leaves "architectures" out
+_CLASS_OF_MODEL_TYPE = {"qwen2": "Qwen2ForCausalLM"}
+
+
 def architecture_name(raw: Dict[str, Any]) -> str:
     names = raw.get("architectures")
-    if not names or not isinstance(names, (list, tuple)) or not isinstance(names[0], str):
-        raise ConfigError('config.json must name its model class in "architectures"')
-    return names[0]
+    if names and isinstance(names, (list, tuple)) and isinstance(names[0], str):
+        return names[0]
+    model_type = raw.get("model_type")
+    if isinstance(model_type, str) and model_type in _CLASS_OF_MODEL_TYPE:
+        return _CLASS_OF_MODEL_TYPE[model_type]
+    raise ConfigError('config.json must name its model class in "architectures" (or a known "model_type")')
 
 
 def _require(raw: Dict[str, Any], key: str, kind):

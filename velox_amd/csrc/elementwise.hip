@@ -319,19 +319,14 @@ __global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, const float* __res
     *reinterpret_cast<float4_t*>(dst + half + c0) = hi_v;
   }
   if (write_kv) {
+    // values go to [channel][offset]: neighbouring lanes take neighbouring channels, so that a store instruction
+    // touches as few cache lines as the layout allows
     const int v_base = (nh + nkv) * d;
-    for (int item = threadIdx.x; item < nkv * d / N; item += blockDim.x) {
-      const int at = item * N;
-      const int head = at / d, c = at % d;
-      float4_t v = *reinterpret_cast<const float4_t*>(row + v_base + at);
-      const T* e = reinterpret_cast<const T*>(&v);
-      T* dst = v_cache + ((page * nkv + head) * d + c) * page_size + offset;
-#pragma unroll
-      for (int j = 0; j < N; ++j) {
-        float x = to_f32(e[j]);
-        if (bias) x += bias[v_base + at + j];
-        dst[(size_t)j * page_size] = from_f32<T>(x);
-      }
+    for (int item = threadIdx.x; item < nkv * d; item += blockDim.x) {
+      const int head = item / d, c = item % d;
+      float x = to_f32(row[v_base + item]);
+      if (bias) x += bias[v_base + item];
+      v_cache[((page * nkv + head) * d + c) * page_size + offset] = from_f32<T>(x);
     }
   }
 }
