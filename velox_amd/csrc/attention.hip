@@ -85,29 +85,72 @@ __device__ __forceinline__ void mask_tail(Vec16<bf16_t>& x, int valid) {
   }
 }
 
-// KEY_SPLIT = false: each of the 4 waves owns 16 of the workgroup's 64 rows and visits every key of a tile.
-// KEY_SPLIT = true (at most 16 rows per sequence and KV head, i.e. decode): every wave owns the same rows and
-// visits its own quarter of each tile's keys; the four partial results are merged through LDS at the end.
-template <typename T, int BN, bool KEY_SPLIT>
+// ---- the general kernel: portions of prompts, any mix -------------------------------------------------------------
+// Contraction blocks.  A lane always holds 16 bytes of a block: bfloat16 blocks have 32 indices (lane (g, i) holds
+// 8g .. 8g+7, one v_mfma_f32_16x16x32_bf16 per block), float32 blocks 16 (lane holds 4g .. 4g+3, four
+// v_mfma_f32_16x16x4_f32 per block).  Both kinds of operand are one 16-byte LDS read.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+template <typename T> struct Block;
+template <> struct Block<bf16_t> {
+  static constexpr int KB = 32;
+  typedef bf16x8_t Operand;
+  static __device__ __forceinline__ float4_t mma(Operand a, Operand b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Block<float> {
+  static constexpr int KB = 16;
+  typedef float4_t Operand;
+  static __device__ __forceinline__ float4_t mma(Operand a, Operand b, float4_t c) {
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[0], b[0], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[1], b[1], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[2], b[2], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[3], b[3], c, 0, 0, 0);
+    return c;
+  }
+};
+
+template <typename T> __device__ __forceinline__ typename Block<T>::Operand load_operand(const T* p) {
+  return __builtin_bit_cast(typename Block<T>::Operand, *reinterpret_cast<const float4_t*>(p));
+}
+
+// exponent and its unit: a float32 run uses the accurate expf on natural-log scores; a bfloat16 run folds log2(e)
+// into the scale and uses the hardware exp2
+template <typename T> struct Softmax;
+template <> struct Softmax<float> {
+  static constexpr float SCALE = 1.f, LN_UNIT = 1.f;
+  static __device__ __forceinline__ float exp_of(float x) { return expf(x); }
+};
+template <> struct Softmax<bf16_t> {
+  static constexpr float SCALE = 1.44269504088896340736f, LN_UNIT = 0.69314718055994530942f;
+  static __device__ __forceinline__ float exp_of(float x) { return __builtin_amdgcn_exp2f(x); }
+};
+
+constexpr int PREFILL_PAGE_IDS = 2048;
+
+template <typename T, int BN>
 __global__ void __launch_bounds__(256) paged_attention_kernel(
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
     T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
     int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens) {
+  typedef Block<T> B;
+  typedef typename B::Operand Operand;
+  constexpr int KB = B::KB;
+  constexpr int VEC = 16 / sizeof(T);           // elements per 16 bytes = indices of a block a lane holds
+  constexpr int DP = (D + KB - 1) / KB * KB;    // head size padded to whole blocks (zero columns)
   constexpr int PAD = 16 / sizeof(T);
-  constexpr int KS = D + PAD;   // row stride of the K tile   [BN][D]
-  constexpr int VS = BN + PAD;  // row stride of the V^T tile [D][BN]
-  constexpr int VEC = 16 / sizeof(T);
-  constexpr int NT = BN / 16;
-  constexpr int NC = D / 16;
-  constexpr int NTW = KEY_SPLIT ? (NT + 3) / 4 : NT;  // key tiles of 16 a wave computes per staged tile
-  constexpr int NCW = KEY_SPLIT ? (NC + 3) / 4 : NC;  // channel blocks a wave writes out
-  constexpr int TILE_BYTES = (BN * KS + D * VS) * (int)sizeof(T);
-  constexpr int MERGE_BYTES = KEY_SPLIT ? (4 * NC * 64 * 16 + 2 * 4 * 16 * 4) : 0;
-  constexpr int SMEM_BYTES = TILE_BYTES > MERGE_BYTES ? TILE_BYTES : MERGE_BYTES;
-  __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
-  T* k_tile = reinterpret_cast<T*>(smem);
-  T* v_tile = k_tile + BN * KS;
+  constexpr int KS = DP + PAD;                  // row stride of the K tile   [BN][DP]
+  constexpr int VS = BN + PAD;                  // row stride of the V^T tile [D][BN]
+  constexpr int NT = BN / 16;                   // 16-key tiles of S^T per staged tile
+  constexpr int NQB = DP / KB;                  // contraction blocks of Q K^T
+  constexpr int NKB = BN / KB;                  // contraction blocks of P V
+  constexpr int TPB = KB / 16;                  // S^T tiles per key block
+  constexpr int NC = D / 16;                    // 16-channel tiles of the output
+  __shared__ __attribute__((aligned(16))) T k_tile[BN * KS];
+  __shared__ __attribute__((aligned(16))) T v_tile[D * VS];
+  __shared__ int page_ids[PREFILL_PAGE_IDS];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -125,7 +168,7 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
   const int r0 = blockIdx.x * ROWS_PER_BLOCK;
   if (r0 >= rows_total) return;
 
-  const int r = r0 + (KEY_SPLIT ? 0 : wave * 16) + i;
+  const int r = r0 + wave * 16 + i;
   const bool row_ok = r < rows_total;
   const int tok = row_ok ? r / group : 0;
   const int head = kvh * group + (row_ok ? r % group : 0);
@@ -149,64 +192,88 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
   int tile_hi = tile_lo + tiles_per_split;
   if (tile_hi > tiles_total) tile_hi = tiles_total;
 
-  // what this wave can skip: tiles wholly after its last row's position
+  // positions of this wave's rows: tiles after the last one are skipped, tiles before the first one need no mask
   int wave_last_pos = row_ok ? pos : -1;
+  int wave_first_pos = row_ok ? pos : 0x7fffffff;
 #pragma unroll
   for (int offset = 32; offset > 0; offset >>= 1) {
-    const int other = __shfl_xor(wave_last_pos, offset, VELOX_WAVE);
-    wave_last_pos = other > wave_last_pos ? other : wave_last_pos;
+    const int hi = __shfl_xor(wave_last_pos, offset, VELOX_WAVE);
+    const int lo = __shfl_xor(wave_first_pos, offset, VELOX_WAVE);
+    wave_last_pos = hi > wave_last_pos ? hi : wave_last_pos;
+    wave_first_pos = lo < wave_first_pos ? lo : wave_first_pos;
   }
 
-  Frag<T> qf[NC];
+  // page ids of the keys this workgroup visits, and zeros in the padding columns of the K tile
+  const int* table = block_tables + (size_t)b * table_width;
+  const int first_page = (n_begin + tile_lo * BN) >> page_shift;
   {
-    const T* qp = qkv + (size_t)(q_start + tok) * qkv_stride + (size_t)head * D + 4 * g;
+    const int last_key = n_begin + tile_hi * BN < kv_len ? n_begin + tile_hi * BN : kv_len;
+    const int num_pages = tile_hi > tile_lo ? ((last_key - 1) >> page_shift) - first_page + 1 : 0;
+    for (int p = tid; p < num_pages && p < PREFILL_PAGE_IDS; p += 256) page_ids[p] = table[first_page + p];
+    if constexpr (DP > D) {
+      for (int e = tid; e < BN * (DP - D); e += 256) k_tile[(e / (DP - D)) * KS + D + e % (DP - D)] = from_f32<T>(0.f);
+    }
+  }
+  auto page_of = [&](int n) -> size_t {
+    const int p = (n >> page_shift) - first_page;
+    return (size_t)(p < PREFILL_PAGE_IDS ? page_ids[p] : table[first_page + p]);
+  };
+
+  Operand qf[NQB];
+  {
+    const T* qp = qkv + (size_t)(q_start + tok) * qkv_stride + (size_t)head * D + VEC * g;
 #pragma unroll
-    for (int c = 0; c < NC; ++c) qf[c] = row_ok ? load_frag<T>(qp + 16 * c) : zero_frag<T>();
+    for (int cb = 0; cb < NQB; ++cb) {
+      const bool inside = row_ok && (KB * cb + VEC * g < D);
+      qf[cb] = inside ? load_operand<T>(qp + KB * cb) : __builtin_bit_cast(Operand, float4_t{0.f, 0.f, 0.f, 0.f});
+    }
   }
 
   float m_i = -INFINITY, l_i = 0.f;
   float4_t acc_o[NC];
 #pragma unroll
   for (int c = 0; c < NC; ++c) acc_o[c] = float4_t{0.f, 0.f, 0.f, 0.f};
+  const float scale_eff = scale * Softmax<T>::SCALE;
 
-  const int* table = block_tables + (size_t)b * table_width;
-
-  // ---- staging: global -> registers (issued a tile ahead) -> LDS ------------------------------
+  // ---- staging: global -> registers (issued a tile ahead) -> LDS; what does not change from tile to tile is computed once
   constexpr int VPR = D / VEC;              // vectors per key row of K
   constexpr int VECS = BN * D / VEC;        // vectors per tile (K and V^T alike)
   constexpr int ITERS = (VECS + 255) / 256;
   const int run = page_size < BN ? page_size : BN;  // consecutive keys that are contiguous in a page of V
   const bool v_by_vectors = run >= VEC;
-  const int vpr_v = v_by_vectors ? run / VEC : 1;
-  const int per_run = D * vpr_v;
+  const int run_shift = v_by_vectors ? __builtin_ctz(run / VEC) : 0;  // log2(vectors per run and channel)
+  int k_key[ITERS], k_col[ITERS], v_dd[ITERS], v_key[ITERS], v_lds[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int v = tid + it * 256;
+    k_key[it] = v / VPR;
+    k_col[it] = (v % VPR) * VEC;
+    const int rn = (v >> run_shift) / D;            // run index within the tile
+    const int rem = v - ((rn * D) << run_shift);
+    v_dd[it] = rem >> run_shift;
+    v_key[it] = rn * run + (rem & ((1 << run_shift) - 1)) * VEC;  // first key of the vector, local to the tile
+    // column of that key in the V^T tile: inside a block of 32 keys the 8 runs of 4 are interleaved so that lane group g
+    // finds the keys of its two S^T tiles side by side (bfloat16 only; float32 blocks hold one tile)
+    v_lds[it] = v_dd[it] * VS + v_key[it];
+  }
   float4_t k_regs[ITERS], v_regs[ITERS];
 
   auto fetch = [&](int n0) {
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-      const int v = tid + it * 256;
       k_regs[it] = float4_t{0.f, 0.f, 0.f, 0.f};
       v_regs[it] = float4_t{0.f, 0.f, 0.f, 0.f};
-      if (v >= VECS) continue;
-      {
-        const int key = v / VPR, vec = v % VPR;
-        const int n = n0 + key;
-        if (n < kv_len) {
-          const size_t page = (size_t)table[n >> page_shift];
-          const int off = n & (page_size - 1);
-          k_regs[it] = *reinterpret_cast<const float4_t*>(k_cache + ((page * nkv + kvh) * page_size + off) * D + vec * VEC);
-        }
-      }
+      if (tid + it * 256 >= VECS) continue;
+      const int nk = n0 + k_key[it];
+      if (nk < kv_len)
+        k_regs[it] = *reinterpret_cast<const float4_t*>(
+            k_cache + (((page_of(nk) * nkv + kvh) << page_shift) + (nk & (page_size - 1))) * D + k_col[it]);
       if (v_by_vectors) {
-        const int rn = v / per_run, rem = v % per_run;
-        const int dd = rem / vpr_v, vec = rem % vpr_v;
-        const int n = n0 + rn * run + vec * VEC;
-        if (n < kv_len) {
-          const size_t page = (size_t)table[n >> page_shift];
-          const int off = n & (page_size - 1);
+        const int nv = n0 + v_key[it];
+        if (nv < kv_len) {
           Vec16<T> x;
-          x.v = *reinterpret_cast<const float4_t*>(v_cache + ((page * nkv + kvh) * D + dd) * page_size + off);
-          if (n + VEC > kv_len) mask_tail(x, kv_len - n);
+          x.v = *reinterpret_cast<const float4_t*>(v_cache + (((page_of(nv) * nkv + kvh) * D + v_dd[it]) << page_shift) + (nv & (page_size - 1)));
+          if (nv + VEC > kv_len) mask_tail(x, kv_len - nv);
           v_regs[it] = x.v;
         }
       }
@@ -215,12 +282,21 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
   auto commit = [&](int n0) {
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-      const int v = tid + it * 256;
-      if (v >= VECS) continue;
-      *reinterpret_cast<float4_t*>(k_tile + (v / VPR) * KS + (v % VPR) * VEC) = k_regs[it];
+      if (tid + it * 256 >= VECS) continue;
+      *reinterpret_cast<float4_t*>(k_tile + k_key[it] * KS + k_col[it]) = k_regs[it];
       if (v_by_vectors) {
-        const int rn = v / per_run, rem = v % per_run;
-        *reinterpret_cast<float4_t*>(v_tile + (rem / vpr_v) * VS + rn * run + (rem % vpr_v) * VEC) = v_regs[it];
+        if constexpr (KB == 32) {
+          // keys 8m .. 8m+7 of a 32-key block: the first four belong to lane group (2m) % 4 of S^T tile (2m) / 4, the
+          // next four to lane group (2m+1) % 4 of tile (2m+1) / 4; lane group g's column run is 8g + 4 * tile
+          const int base = v_dd[it] * VS + (v_key[it] & ~31);
+          const int m = (v_key[it] & 31) >> 3;
+          const int q0 = 2 * m, q1 = 2 * m + 1;  // quads of 4 keys
+          typedef float float2_t __attribute__((ext_vector_type(2)));
+          *reinterpret_cast<float2_t*>(v_tile + base + 8 * (q0 & 3) + 4 * (q0 >> 2)) = float2_t{v_regs[it][0], v_regs[it][1]};
+          *reinterpret_cast<float2_t*>(v_tile + base + 8 * (q1 & 3) + 4 * (q1 >> 2)) = float2_t{v_regs[it][2], v_regs[it][3]};
+        } else {
+          *reinterpret_cast<float4_t*>(v_tile + v_lds[it]) = v_regs[it];
+        }
       }
     }
     if (!v_by_vectors) {  // pages shorter than a vector: element by element, straight from global memory
@@ -231,15 +307,18 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
         const int nl = rn * run + e;
         const int n = n0 + nl;
         T x = from_f32<T>(0.f);
-        if (n < kv_len) {
-          const size_t page = (size_t)table[n >> page_shift];
-          x = v_cache[((page * nkv + kvh) * D + dd) * page_size + (n & (page_size - 1))];
+        if (n < kv_len) x = v_cache[((page_of(n) * nkv + kvh) * D + dd) * page_size + (n & (page_size - 1))];
+        int col = nl;
+        if constexpr (KB == 32) {
+          const int quad = (nl & 31) >> 2;
+          col = (nl & ~31) + 8 * (quad & 3) + 4 * (quad >> 2) + (nl & 3);
         }
-        v_tile[dd * VS + nl] = x;
+        v_tile[dd * VS + col] = x;
       }
     }
   };
 
+  __syncthreads();  // page ids are in place
   if (tile_lo < tile_hi) fetch(n_begin + tile_lo * BN);
   for (int tile = tile_lo; tile < tile_hi; ++tile) {
     const int n0 = n_begin + tile * BN;
@@ -250,48 +329,58 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
     if (n0 > wave_last_pos) continue;        // nothing this wave may read; it still took part in the staging
 
     // ---- S^T = K Q^T ----------------------------------------------------------------------
-    float4_t s[NTW];
+    float4_t s[NT];
 #pragma unroll
-    for (int tt = 0; tt < NTW; ++tt) {
-      const int t = KEY_SPLIT ? wave + 4 * tt : tt;
-      s[tt] = float4_t{0.f, 0.f, 0.f, 0.f};
-      if (t < NT) {
+    for (int t = 0; t < NT; ++t) {
+      s[t] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
-          const Frag<T> a = load_frag<T>(k_tile + (16 * t + i) * KS + 16 * c + 4 * g);
-          s[tt] = mma16(a, qf[c], s[tt]);
-        }
-      }
+      for (int cb = 0; cb < NQB; ++cb)
+        s[t] = B::mma(load_operand<T>(k_tile + (16 * t + i) * KS + KB * cb + VEC * g), qf[cb], s[t]);
     }
-    // ---- mask, running maximum ------------------------------------------------------------
+    // ---- scale, mask (only where the tile crosses a row's limits), running maximum ----------
+    const bool whole = n0 + BN <= kv_len && n0 + BN - 1 <= wave_first_pos && (window <= 0 || n0 > wave_last_pos - window);
     float mx = -INFINITY;
+    if (whole) {
 #pragma unroll
-    for (int tt = 0; tt < NTW; ++tt) {
-      const int t = KEY_SPLIT ? wave + 4 * tt : tt;
+      for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int n = n0 + 16 * t + 4 * g + j;
-        const bool keep = row_ok && t < NT && n < kv_len && n <= pos && (window <= 0 || n > pos - window);
-        const float val = keep ? s[tt][j] * scale : -INFINITY;
-        s[tt][j] = val;
-        mx = fmaxf(mx, val);
-      }
+        for (int j = 0; j < 4; ++j) {
+          s[t][j] *= scale_eff;
+          mx = fmaxf(mx, s[t][j]);
+        }
+    } else {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int n = n0 + 16 * t + 4 * g + j;
+          const bool keep = row_ok && n < kv_len && n <= pos && (window <= 0 || n > pos - window);
+          s[t][j] = keep ? s[t][j] * scale_eff : -INFINITY;
+          mx = fmaxf(mx, s[t][j]);
+        }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, VELOX_WAVE));
     mx = fmaxf(mx, __shfl_xor(mx, 32, VELOX_WAVE));
     const float m_new = fmaxf(m_i, mx);
     const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = (m_i == -INFINITY) ? 0.f : softmax_exp<T>(m_i - m_safe);
+    const float alpha = (m_i == -INFINITY) ? 0.f : Softmax<T>::exp_of(m_i - m_safe);
     float psum = 0.f;
-    Frag<T> pf[NTW];
+    Operand pf[NKB];
 #pragma unroll
-    for (int tt = 0; tt < NTW; ++tt)
+    for (int kb = 0; kb < NKB; ++kb) {
+      Vec16<T> packed;
+      T* e = reinterpret_cast<T*>(&packed.v);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float p = (s[tt][j] == -INFINITY) ? 0.f : softmax_exp<T>(s[tt][j] - m_safe);
-        psum += p;
-        set_prob(pf[tt], j, p);
-      }
+      for (int u = 0; u < TPB; ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float sv = s[kb * TPB + u][j];
+          const float p = (sv == -INFINITY) ? 0.f : Softmax<T>::exp_of(sv - m_safe);
+          psum += p;
+          e[4 * u + j] = from_f32<T>(p);
+        }
+      pf[kb] = __builtin_bit_cast(Operand, packed.v);
+    }
     l_i = l_i * alpha + psum;  // partial over this lane's keys; the four lane groups are summed at the end
     m_i = m_new;
     // ---- O^T = O^T * alpha + V^T P^T ------------------------------------------------------
@@ -299,77 +388,29 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
     for (int c = 0; c < NC; ++c) {
       acc_o[c] = acc_o[c] * alpha;
 #pragma unroll
-      for (int tt = 0; tt < NTW; ++tt) {
-        const int t = KEY_SPLIT ? wave + 4 * tt : tt;
-        if (t < NT) {
-          const Frag<T> a = load_frag<T>(v_tile + (16 * c + i) * VS + 16 * t + 4 * g);
-          acc_o[c] = mma16(a, pf[tt], acc_o[c]);
-        }
-      }
+      for (int kb = 0; kb < NKB; ++kb)
+        acc_o[c] = B::mma(load_operand<T>(v_tile + (16 * c + i) * VS + KB * kb + VEC * g), pf[kb], acc_o[c]);
     }
   }
 
   l_i += __shfl_xor(l_i, 16, VELOX_WAVE);
   l_i += __shfl_xor(l_i, 32, VELOX_WAVE);
-
-  if constexpr (KEY_SPLIT) {
-    // merge the four waves: out = sum_w e^(m_w - m) acc_w / sum_w e^(m_w - m) l_w
-    float4_t* acc_all = reinterpret_cast<float4_t*>(smem);                     // [4][NC][64]
-    float* m_all = reinterpret_cast<float*>(smem + 4 * NC * 64 * 16);          // [4][16]
-    float* l_all = m_all + 4 * 16;                                             // [4][16]
-    __syncthreads();  // the tiles are no longer read
-#pragma unroll
-    for (int c = 0; c < NC; ++c) acc_all[(wave * NC + c) * 64 + lane] = acc_o[c];
-    if (g == 0) { m_all[wave * 16 + i] = m_i; l_all[wave * 16 + i] = l_i; }
-    __syncthreads();
-    float m_tot = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) m_tot = fmaxf(m_tot, m_all[w * 16 + i]);
-    const float m_ref = (m_tot == -INFINITY) ? 0.f : m_tot;
-    float weight[4];
-    float l_tot = 0.f;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const float mw = m_all[w * 16 + i];
-      weight[w] = (mw == -INFINITY) ? 0.f : softmax_exp<T>(mw - m_ref);
-      l_tot += weight[w] * l_all[w * 16 + i];
-    }
-    m_i = m_tot;
-    l_i = l_tot;
-#pragma unroll
-    for (int cc = 0; cc < NCW; ++cc) {
-      const int c = wave + 4 * cc;
-      if (c < NC) {
-        float4_t sum = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int w = 0; w < 4; ++w) sum += acc_all[(w * NC + c) * 64 + lane] * weight[w];
-        acc_o[cc] = sum;  // from here on acc_o[cc] is channel block wave + 4 cc
-      }
-    }
-  }
-
   if (!row_ok) return;
   const float inv = l_i > 0.f ? 1.f / l_i : 1.f;
   const size_t token = (size_t)(q_start + tok);
   if (splits == 1) {
     T* dst = out + (token * nh + head) * D + 4 * g;
 #pragma unroll
-    for (int cc = 0; cc < NCW; ++cc) {
-      const int c = KEY_SPLIT ? wave + 4 * cc : cc;
-      if (c < NC) {
+    for (int c = 0; c < NC; ++c) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) dst[16 * c + j] = from_f32<T>(acc_o[cc][j] * inv);
-      }
+      for (int j = 0; j < 4; ++j) dst[16 * c + j] = from_f32<T>(acc_o[c][j] * inv);
     }
   } else {
     const size_t slot = ((size_t)split * total_tokens + token) * nh + head;
     float* dst = part_o + slot * D + 4 * g;
 #pragma unroll
-    for (int cc = 0; cc < NCW; ++cc) {
-      const int c = KEY_SPLIT ? wave + 4 * cc : cc;
-      if (c < NC) *reinterpret_cast<float4_t*>(dst + 16 * c) = acc_o[cc] * inv;
-    }
-    if (g == 0 && (!KEY_SPLIT || wave == 0)) part_lse[slot] = l_i > 0.f ? m_i + logf(l_i) : -INFINITY;
+    for (int c = 0; c < NC; ++c) *reinterpret_cast<float4_t*>(dst + 16 * c) = acc_o[c] * inv;
+    if (g == 0) part_lse[slot] = l_i > 0.f ? m_i * Softmax<T>::LN_UNIT + logf(l_i) : -INFINITY;
   }
 }
 
@@ -617,14 +658,9 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
   }
   const int row_tiles = (max_q_len * group + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
   dim3 grid(row_tiles, nkv, num_seqs * splits);
-  if (max_q_len * group <= 16)
-    paged_attention_kernel<T, BN, true><<<grid, 256, 0, stream>>>(
-        (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
-  else
-    paged_attention_kernel<T, BN, false><<<grid, 256, 0, stream>>>(
-        (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
+  paged_attention_kernel<T, BN><<<grid, 256, 0, stream>>>(
+      (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+      part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
   int status = (int)hipGetLastError();
   if (status != 0 || splits == 1) return status;
   merge_splits_kernel<T><<<dim3(total_tokens, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens);
