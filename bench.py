@@ -144,6 +144,7 @@ def main() -> int:
     parser.add_argument("--prefill-tokens", type=int, default=2048)
     parser.add_argument("--no-graphs", action="store_true")
     parser.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    parser.add_argument("--no-tune", action="store_true", help="do not let the matrix library pick its kernels for the prefill shapes")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine (single-GPU tier)")
@@ -161,6 +162,7 @@ def main() -> int:
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
 
     engine = make_engine(model_config, args.dtype, max(batches), args.context, args.prefill_tokens, graphs)
+    tuned = 0 if args.no_tune else engine.tune_matrix_products([args.prefill_tokens])
     step_s, contexts = {}, {}
     for batch in batches:
         steps = args.steps if batch == args.batch else max(8, args.steps // 2)
@@ -190,7 +192,7 @@ def main() -> int:
             "kv_heads": model_config["num_key_value_heads"], "head_dim": model_config["hidden_size"] // model_config["num_attention_heads"],
             "intermediate": model_config["intermediate_size"], "vocab": vocab,
             "global_batch": args.batch, "seq_len": args.context, "mean_context": round(contexts[args.batch], 1), "page_size": 16,
-            "prefill_tokens": args.prefill_tokens, "hip_graphs": graphs, "parallelism": "single-gpu",
+            "prefill_tokens": args.prefill_tokens, "hip_graphs": graphs, "library_gemm_tuned": tuned > 0, "parallelism": "single-gpu",
         },
         "prefill": {
             "value": round(args.prefill_tokens / prefill_s, 1), "tokens": args.prefill_tokens,

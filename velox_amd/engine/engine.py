@@ -121,6 +121,21 @@ class Engine:
         self.runner.capture_decode_graphs()
         torch.cuda.synchronize()
 
+    def tune_matrix_products(self, token_counts: Sequence[int]) -> int:
+        """Optional, bfloat16 only: has the matrix library time its candidate kernels for this model's weight shapes at
+        the given numbers of tokens per step (typically the prefill chunk size) and keep the fastest.  Takes seconds
+        per shape; steps with other token counts are unaffected."""
+        if self.dtype != torch.bfloat16 or self.device.type != "cuda":
+            return 0
+        shapes = set()
+        for part in self.model.all_parts():
+            for attr, param in part.params().items():
+                tensor = getattr(part, attr, None)
+                if param.role == "matrix" and tensor is not None and tensor.dim() == 2 and tensor.dtype == torch.bfloat16 and attr != "table":
+                    shapes.add(tuple(tensor.shape))
+        counts = [m for m in token_counts if m > 64]  # smaller steps run on the engine's own kernels
+        return self.ops.tune_library_products(shapes, counts) if counts else 0
+
     # -- requests -----------------------------------------------------------------------
     def add_request(self, request: Request) -> None:
         bad = [t for t in request.prompt_token_ids if not 0 <= t < self.model.spec.vocab_size]

@@ -13,6 +13,8 @@ a library has no call for.  bfloat16 x bfloat16 products go to the library behin
 from __future__ import annotations
 
 import ctypes
+import os
+import tempfile
 from typing import Dict, Optional
 
 import torch
@@ -93,6 +95,30 @@ class HipOps:
         for need in model.cache_needs():
             if need is not None and hasattr(need, "head_dim"):
                 self.attention_library(need.head_dim)
+
+    def tune_library_products(self, shapes, token_counts, seconds_per_shape: float = 0.2) -> int:
+        """Lets PyTorch's TunableOp time the library's candidate kernels for ``x[M, K] @ w[N, K]^T`` at the given
+        ``(N, K)`` shapes and ``M`` values, and keeps its choices for later calls.  Tuning stays off afterwards, so
+        other shapes keep the library's default choice and never pay for a search.  Returns the number of products tuned."""
+        tunable = torch.cuda.tunable
+        tunable.enable(True)
+        # the library writes what it found to a file when the process ends: keep that out of the working folder
+        tunable.set_filename(os.path.join(tempfile.gettempdir(), f"velox_amd_tunableop_{os.getuid()}_{os.getpid()}.csv"))
+        tunable.set_max_tuning_duration(int(seconds_per_shape * 1000))
+        tunable.tuning_enable(True)
+        done = 0
+        try:
+            for n, k in sorted(set(shapes)):
+                weight = torch.zeros((n, k), dtype=torch.bfloat16, device=self.device)
+                for m in sorted(set(token_counts)):
+                    x = torch.zeros((m, k), dtype=torch.bfloat16, device=self.device)
+                    torch.nn.functional.linear(x, weight)
+                    done += 1
+                del weight
+            torch.cuda.synchronize(self.device)
+        finally:
+            tunable.tuning_enable(False)
+        return done
 
     # -- helpers --------------------------------------------------------------------------------
     def _stream(self):
