@@ -331,3 +331,18 @@ def test_skinny_gemm(ops, ref, out_dtype, m, n, k):
     if m > fewer:
         part = ops.skinny_gemm(x[:fewer].contiguous(), w, None, out_dtype)
         torch.testing.assert_close(ops.skinny_gemm(x, w, None, out_dtype)[:fewer], part, rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("m,inter,k", [(1, 128, 64), (8, 18944, 3584), (16, 150, 128), (7, 1000, 192), (3, 16, 64)])
+def test_skinny_gemm_with_silu_epilogue(ops, ref, m, inter, k):
+    x = rand((m, k), torch.bfloat16, 50)
+    w = rand((2 * inter, k), torch.bfloat16, 51, 0.05)
+    gate_up = ref.linear(x, w, None, torch.float32)
+    want = (torch.nn.functional.silu(gate_up[:, :inter]) * gate_up[:, inter:])
+    scale = float(want.abs().max())
+    for waves, pairs in ((None, None), (4, 1), (8, 1), (4, 2), (8, 2)):
+        got = ops.linear_silu_mul(x, w, torch.bfloat16, waves=waves, pairs=pairs).float()
+        torch.testing.assert_close(got, want, rtol=1e-2, atol=1e-2 * scale)
+    # larger batches take the unfused route and agree with it
+    big = rand((40, k), torch.bfloat16, 52)
+    torch.testing.assert_close(ops.linear_silu_mul(big, w, torch.bfloat16).float(), ref.linear_silu_mul(big, w, torch.bfloat16).float(), rtol=3e-2, atol=3e-2 * scale)

@@ -85,6 +85,9 @@ class TorchOps:
             out = out + bias.float()
         return out.to(out_dtype)
 
+    def linear_silu_mul(self, x, gate_up_weight, out_dtype, **_):
+        return self.silu_mul(self.linear(x, gate_up_weight, None, out_dtype))
+
     def silu_mul(self, gate_up):
         inter = gate_up.shape[-1] // 2
         gate = gate_up[:, :inter].float()

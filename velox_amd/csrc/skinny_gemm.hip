@@ -39,14 +39,18 @@ __device__ __forceinline__ Run16 zero_run() {
   return r;
 }
 
-template <int RT, int CT, int WAVES, typename TO>
+// GLU = true: W holds two stacked matrices, gate rows [0, n) and up rows [n, 2n); the first RT / 2 row tiles of a
+// workgroup are gate rows, the others the up rows of the same output columns, and what is stored is
+// silu(gate) * up, computed on the float32 sums (the [M, 2n] product is never written).
+template <int RT, int CT, int WAVES, typename TO, bool GLU = false>
 __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
                                                                  const float* __restrict__ bias, TO* __restrict__ out, int m, int n, int k) {
   constexpr int UNROLL = 4;  // blocks of 64 indices whose loads are issued together
   __shared__ float4_t partial[WAVES][RT * CT][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int g = lane >> 4, i = lane & 15;
-  const int n0 = blockIdx.x * 16 * RT;
+  constexpr int RTO = GLU ? RT / 2 : RT;  // row tiles that become output columns
+  const int n0 = blockIdx.x * 16 * RTO;
 
   // this wave's share of K, in blocks of 64
   const int blocks_total = k / 64;
@@ -59,9 +63,10 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
   bool w_ok[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int row = n0 + 16 * rt + i;
-    w_ok[rt] = row < n;
-    w_ptr[rt] = w + (size_t)(w_ok[rt] ? row : 0) * k + 16 * g;
+    const int col = n0 + 16 * (rt % RTO) + i;          // output column this row of W contributes to
+    const size_t row = (size_t)col + (rt >= RTO ? n : 0);  // its row in W
+    w_ok[rt] = col < n;
+    w_ptr[rt] = w + (w_ok[rt] ? row : 0) * k + 16 * g;
   }
   const bf16_t* a_ptr[CT];
   bool a_ok[CT];
@@ -107,11 +112,18 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) partial[wave][rt * CT + ct][lane] = acc[rt][ct];
   __syncthreads();
-  for (int item = threadIdx.x; item < RT * CT * 64; item += WAVES * 64) {
+  for (int item = threadIdx.x; item < RTO * CT * 64; item += WAVES * 64) {
     const int tile = item >> 6, l = item & 63;
     float4_t sum = partial[0][tile][l];
 #pragma unroll
     for (int wv = 1; wv < WAVES; ++wv) sum += partial[wv][tile][l];
+    if constexpr (GLU) {
+      float4_t up = partial[0][tile + RTO * CT][l];
+#pragma unroll
+      for (int wv = 1; wv < WAVES; ++wv) up += partial[wv][tile + RTO * CT][l];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sum[j] = sum[j] / (1.f + expf(-sum[j])) * up[j];
+    }
     const int rt = tile / CT, ct = tile % CT;
     const int col_m = 16 * ct + (l & 15);           // batch row
     const int row_n = n0 + 16 * rt + 4 * (l >> 4);  // first of four output columns
@@ -124,6 +136,13 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
       out[(size_t)col_m * n + row_n + j] = from_f32<TO>(v);
     }
   }
+}
+
+template <int RT, int CT, int WAVES>
+static int launch_skinny_glu(const void* a, const void* w, void* out, int m, int n, int k, hipStream_t stream) {
+  const int blocks = (n + 8 * RT - 1) / (8 * RT);
+  skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k);
+  return (int)hipGetLastError();
 }
 
 template <int RT, int CT, int WAVES>
@@ -162,4 +181,21 @@ extern "C" int velox_skinny_gemm_bf16(const void* a, const void* w, const float*
   if (waves >= 8) PICK(2, 4, 8);
   PICK(2, 4, 4);
 #undef PICK
+}
+
+// out[M, n] = silu(A Wgate^T) * (A Wup^T) with W = [Wgate; Wup] of 2n rows, bfloat16 in and out, M <= 32.
+// pairs: gate/up tile pairs per wave (1 or 2).
+extern "C" int velox_skinny_gemm_glu_bf16(const void* a, const void* w, void* out, int m, int n, int k, int waves, int pairs, hipStream_t stream) {
+  if (m <= 0 || n <= 0) return 0;
+  if (k % 64 != 0 || m > 32) return -1;
+  if (m <= 16) {
+    if (pairs >= 2) {
+      if (waves >= 8) return launch_skinny_glu<4, 1, 8>(a, w, out, m, n, k, stream);
+      return launch_skinny_glu<4, 1, 4>(a, w, out, m, n, k, stream);
+    }
+    if (waves >= 8) return launch_skinny_glu<2, 1, 8>(a, w, out, m, n, k, stream);
+    return launch_skinny_glu<2, 1, 4>(a, w, out, m, n, k, stream);
+  }
+  if (waves >= 8) return launch_skinny_glu<2, 2, 8>(a, w, out, m, n, k, stream);
+  return launch_skinny_glu<2, 2, 4>(a, w, out, m, n, k, stream);
 }

@@ -71,6 +71,8 @@ class HipOps:
         c.velox_gemm_fma.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
         c.velox_skinny_gemm_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
         c.velox_skinny_gemm_bf16.restype = _I
+        c.velox_skinny_gemm_glu_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P]
+        c.velox_skinny_gemm_glu_bf16.restype = _I
         c.velox_argmax.argtypes = [_P, _P, _I, _I, _P]
         c.velox_sample.argtypes = [_P, _P, _P, _I, _I, _P]
         c.velox_apply_penalties.argtypes = [_P, _P, _P, _P, _I, _I, _I, _P]
@@ -219,6 +221,29 @@ class HipOps:
         out = torch.empty((m, n), dtype=out_dtype, device=self.device)
         status = self._core.velox_skinny_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), m, n, k, _code(out_dtype), int(waves), int(row_tiles), self._stream())
         self._launched(status, "skinny_gemm")
+        return out
+
+    def linear_silu_mul(self, x: torch.Tensor, gate_up_weight: torch.Tensor, out_dtype: torch.dtype, waves: Optional[int] = None, pairs: Optional[int] = None) -> torch.Tensor:
+        """``silu(x Wgate^T) * (x Wup^T)`` for ``W = [Wgate; Wup]``.  Decode-sized bfloat16 batches run as one kernel that
+        never writes the [M, 2I] product; everything else is the product followed by the SiLU kernel."""
+        m, k = x.shape
+        two_n = gate_up_weight.shape[0]
+        fused = (self.use_skinny_gemm and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16 and out_dtype == torch.bfloat16
+                 and m <= 16 and k % 64 == 0 and two_n % 2 == 0 and x.dim() == 2 and gate_up_weight.shape[1] == k)
+        if not fused:
+            return self.silu_mul(self.linear(x, gate_up_weight, None, out_dtype))
+        self._check("x", x, align=16)
+        self._check("gate_up_weight", gate_up_weight, align=16)
+        n = two_n // 2
+        if pairs is None:
+            pairs = 2 if n >= 32 * 2 * self.num_cus else 1
+        if waves is None:
+            blocks = (n + 16 * pairs - 1) // (16 * pairs)
+            wanted = (8 * self.num_cus + blocks - 1) // blocks
+            waves = 8 if wanted > 4 else 4
+        out = torch.empty((m, n), dtype=out_dtype, device=self.device)
+        status = self._core.velox_skinny_gemm_glu_bf16(_ptr(x), _ptr(gate_up_weight), _ptr(out), m, n, k, int(waves), int(pairs), self._stream())
+        self._launched(status, "skinny_gemm_glu")
         return out
 
     def gemm_fma(self, x, weight, bias, out_dtype):

@@ -2,8 +2,9 @@
 
 Reference ``src/mlp.py:9-15``: one fused product with rows ``[Wgate; Wup]`` (no bias),
 ``act(gate) * up``, down product (no bias); ``silu(x) = x * sigmoid(x)``.  The
-activation and the product are one kernel here and are computed in float32
-from the stored gate/up values, with one rounding at the store.
+activation and the product ``act(gate) * up`` are computed in float32 with one
+rounding at the store; for decode-sized batches they are the epilogue of the
+gate/up product itself, which then never writes its ``[T, 2I]`` result.
 """
 from __future__ import annotations
 
@@ -33,8 +34,7 @@ class GatedMLP(FeedForward):
 
     def forward(self, x, ctx):
         ops = ctx.ops
-        gate_up = ops.linear(x, self.gate_up_weight, None, ctx.dtype)
-        act = ops.silu_mul(gate_up)
+        act = ops.linear_silu_mul(x, self.gate_up_weight, ctx.dtype)
         return ops.linear(act, self.down_weight, None, ctx.dtype)
 
 
