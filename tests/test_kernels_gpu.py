@@ -346,3 +346,27 @@ def test_skinny_gemm_with_silu_epilogue(ops, ref, m, inter, k):
     # larger batches take the unfused route and agree with it
     big = rand((40, k), torch.bfloat16, 52)
     torch.testing.assert_close(ops.linear_silu_mul(big, w, torch.bfloat16).float(), ref.linear_silu_mul(big, w, torch.bfloat16).float(), rtol=3e-2, atol=3e-2 * scale)
+
+
+@pytest.mark.parametrize("m,n,k", [(17, 3584, 18944), (64, 3584, 3584), (33, 100, 640), (64, 4608, 3584), (40, 260, 128)])
+def test_skinny_gemm_splitk_and_norm_that_adds_the_partials(ops, ref, m, n, k):
+    x = rand((m, k), torch.bfloat16, 60)
+    w = rand((n, k), torch.bfloat16, 61, 0.05)
+    want = ref.linear(x, w, None, torch.float32)
+    scale = float(want.abs().max())
+    for splits in (None, 1, 2, 5):
+        part = ops.skinny_gemm_splitk(x, w, splits=splits)
+        assert part.dim() == 3 and part.shape[1:] == (m, n) and part.dtype == torch.float32
+        torch.testing.assert_close(part.sum(0), want, rtol=1e-4, atol=1e-4 * scale)
+    part = ops.skinny_gemm_splitk(x, w)
+    if n % 4 == 0:
+        residual = rand((m, n), torch.float32, 62)
+        weight = 1 + rand((n,), torch.float32, 63, 0.02)
+        r_hip, r_ref = residual.clone(), residual.clone()
+        got = ops.add_rmsnorm(r_hip, part, weight, 1e-6, torch.bfloat16)
+        ref_out = ref.add_rmsnorm(r_ref, part, weight, 1e-6, torch.bfloat16)
+        torch.testing.assert_close(r_hip, r_ref, rtol=1e-5, atol=1e-5 * scale)
+        torch.testing.assert_close(got.float(), ref_out.float(), rtol=2e-2, atol=2e-2)
+        rows = torch.tensor([m - 1, 0, 3], dtype=torch.int32).cuda()
+        torch.testing.assert_close(ops.add_rmsnorm_rows(r_hip, part, rows, weight, 1e-6, torch.float32),
+                                   ref.add_rmsnorm_rows(r_ref, part, rows, weight, 1e-6, torch.float32), rtol=1e-4, atol=1e-4)

@@ -66,12 +66,16 @@ class TorchOps:
         return table[token_ids.long()].float()
 
     def add_rmsnorm(self, residual, delta, weight, eps, out_dtype):
+        if delta is not None and delta.dim() == 3:
+            delta = delta.float().sum(0)
         if delta is not None:
             residual += delta.float()
         var = (residual * residual).sum(-1, keepdim=True) / residual.shape[-1]
         return (residual * torch.rsqrt(var + eps) * weight.float()).to(out_dtype)
 
     def add_rmsnorm_rows(self, residual, delta, rows, weight, eps, out_dtype):
+        if delta is not None and delta.dim() == 3:
+            delta = delta.float().sum(0)
         x = residual[rows.long()]
         if delta is not None:
             x = x + delta[rows.long()].float()
@@ -79,7 +83,7 @@ class TorchOps:
         return (x * torch.rsqrt(var + eps) * weight.float()).to(out_dtype)
 
     # -- matrix products ----------------------------------------------------------------
-    def linear(self, x, weight, bias, out_dtype):
+    def linear(self, x, weight, bias, out_dtype, partials_ok=False):
         out = x.float() @ weight.float().T
         if bias is not None:
             out = out + bias.float()

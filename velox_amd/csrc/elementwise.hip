@@ -34,9 +34,12 @@ extern "C" int velox_embed(const int* ids, const void* table, float* out, int to
 //   rows != nullptr: r = residual[rows[row]] (+ delta[rows[row]]); out[row] = norm(r); nothing else is written
 //   norm(r) = r * rsqrt(sum(r^2) / H + eps) * w
 // ---------------------------------------------------------------------------------------------
+//   delta may be `partials` stacked tensors (partial sums of a split product), `partial_stride` elements apart: they are
+//   added in order, first to last.
 template <typename TD, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta, const int* __restrict__ rows,
-                                   const float* __restrict__ weight, TO* __restrict__ out, int hidden, float eps) {
+                                   const float* __restrict__ weight, TO* __restrict__ out, int hidden, float eps,
+                                   int partials, size_t partial_stride) {
   __shared__ float scratch[16];
   const int row = blockIdx.x;
   const size_t src_row = rows ? (size_t)rows[row] : (size_t)row;
@@ -46,7 +49,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
   float sumsq = 0.f;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float r = res[i];
-    if (del) r += to_f32(del[i]);
+    if (del)
+      for (int p = 0; p < partials; ++p) r += to_f32(del[p * partial_stride + i]);
     if (write_back) res[i] = r;
     sumsq += r * r;
   }
@@ -55,7 +59,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
   TO* dst = out + (size_t)row * hidden;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float r = res[i];
-    if (del && !write_back) r += to_f32(del[i]);
+    if (del && !write_back)
+      for (int p = 0; p < partials; ++p) r += to_f32(del[p * partial_stride + i]);
     dst[i] = from_f32<TO>(r * inv * weight[i]);
   }
 }
@@ -76,7 +81,8 @@ template <> struct Quad<bf16_t> {
 
 template <typename TD, typename TO, int CHUNKS>
 __global__ void add_rmsnorm_rows_in_registers_kernel(float* __restrict__ residual, const TD* __restrict__ delta, const int* __restrict__ rows,
-                                                     const float* __restrict__ weight, TO* __restrict__ out, int hidden, float eps) {
+                                                     const float* __restrict__ weight, TO* __restrict__ out, int hidden, float eps,
+                                                     int partials, size_t partial_stride) {
   __shared__ float scratch[16];
   const int row = blockIdx.x;
   const size_t src_row = rows ? (size_t)rows[row] : (size_t)row;
@@ -92,9 +98,11 @@ __global__ void add_rmsnorm_rows_in_registers_kernel(float* __restrict__ residua
     if (at < hidden) {
       r[c] = *reinterpret_cast<const float4_t*>(res + at);
       if (del) {
-        const Quad<TD> d = *reinterpret_cast<const Quad<TD>*>(del + at);
+        for (int p = 0; p < partials; ++p) {
+          const Quad<TD> d = *reinterpret_cast<const Quad<TD>*>(del + p * partial_stride + at);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) r[c][j] += d.get(j);
+          for (int j = 0; j < 4; ++j) r[c][j] += d.get(j);
+        }
       }
       if (write_back) *reinterpret_cast<float4_t*>(res + at) = r[c];
 #pragma unroll
@@ -118,17 +126,19 @@ __global__ void add_rmsnorm_rows_in_registers_kernel(float* __restrict__ residua
 }
 
 extern "C" int velox_add_rmsnorm(float* residual, const void* delta, const int* rows, const float* weight, void* out,
-                                 int num_rows, int hidden, float eps, int delta_dtype, int out_dtype, hipStream_t stream) {
+                                 int num_rows, int hidden, float eps, int delta_dtype, int out_dtype, int partials,
+                                 long long partial_stride, hipStream_t stream) {
   if (num_rows <= 0) return 0;
+  if (partials < 1 || (partials > 1 && partial_stride % 4 != 0)) return -1;
   const int threads = hidden >= 2048 ? 512 : 256;
   const bool aligned = (((uintptr_t)residual | (uintptr_t)delta | (uintptr_t)weight | (uintptr_t)out) & 15) == 0;
   const bool in_registers = aligned && hidden % 4 == 0 && hidden <= 4 * threads * 4;
 #define LAUNCH(TD, TO)                                                                                                                  \
   do {                                                                                                                                  \
     if (in_registers)                                                                                                                   \
-      add_rmsnorm_rows_in_registers_kernel<TD, TO, 4><<<num_rows, threads, 0, stream>>>(residual, (const TD*)delta, rows, weight, (TO*)out, hidden, eps); \
+      add_rmsnorm_rows_in_registers_kernel<TD, TO, 4><<<num_rows, threads, 0, stream>>>(residual, (const TD*)delta, rows, weight, (TO*)out, hidden, eps, partials, (size_t)partial_stride); \
     else                                                                                                                                \
-      add_rmsnorm_kernel<TD, TO><<<num_rows, threads, 0, stream>>>(residual, (const TD*)delta, rows, weight, (TO*)out, hidden, eps);    \
+      add_rmsnorm_kernel<TD, TO><<<num_rows, threads, 0, stream>>>(residual, (const TD*)delta, rows, weight, (TO*)out, hidden, eps, partials, (size_t)partial_stride); \
   } while (0)
   if (delta_dtype == VELOX_BF16 && out_dtype == VELOX_BF16) LAUNCH(bf16_t, bf16_t);
   else if (delta_dtype == VELOX_F32 && out_dtype == VELOX_F32) LAUNCH(float, float);

@@ -199,3 +199,102 @@ extern "C" int velox_skinny_gemm_glu_bf16(const void* a, const void* w, void* ou
   if (waves >= 8) return launch_skinny_glu<2, 2, 8>(a, w, out, m, n, k, stream);
   return launch_skinny_glu<2, 2, 4>(a, w, out, m, n, k, stream);
 }
+
+// ---------------------------------------------------------------------------------------------------------------
+// Split-K variant for 17 .. 64 rows and matrices with few rows of W but a long K (the output and down projections):
+// partial[s, M, N] = A[:, K_s] * W[:, K_s]^T in float32 for each of S slices K_s of K; whoever consumes the result adds the
+// S partial sums (the residual-add + norm kernel does, in a fixed order).  A workgroup owns 64 rows of W (one 16-row
+// tile per wave) and one slice of K.  W streams through registers a chunk (4 blocks of 64 indices) ahead; the
+// activations of a chunk (up to 64 rows x 256 indices) are staged in LDS once per workgroup and read by all four waves.
+// ---------------------------------------------------------------------------------------------------------------
+template <int CT>
+__global__ void __launch_bounds__(256) skinny_gemm_splitk_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
+                                                                float* __restrict__ partial, int m, int n, int k, int blocks_per_split) {
+  constexpr int CHUNK = 4;                 // blocks of 64 indices per staging step
+  constexpr int ROWS = 16 * CT;            // activation rows held in LDS
+  constexpr int AS = 64 + 8;               // row stride of one block of activations, in elements
+  constexpr int A_VECS = ROWS * CHUNK * 8; // 16-byte vectors per chunk of activations
+  constexpr int A_ITERS = (A_VECS + 255) / 256;
+  __shared__ __attribute__((aligned(16))) bf16_t a_tile[CHUNK * ROWS * AS];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 4, i = lane & 15;
+  const int row = blockIdx.x * 64 + 16 * wave + i;
+  const bool w_ok = row < n;
+  const bf16_t* w_ptr = w + (size_t)(w_ok ? row : 0) * k + 16 * g;
+  const int blocks_total = k / 64;
+  const int kb_lo = blockIdx.y * blocks_per_split;
+  int kb_hi = kb_lo + blocks_per_split;
+  if (kb_hi > blocks_total) kb_hi = blocks_total;
+
+  float4_t acc[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) acc[ct] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  Run16 w_next[CHUNK];
+  float4_t a_next[A_ITERS];
+  auto fetch = [&](int kb) {
+#pragma unroll
+    for (int u = 0; u < CHUNK; ++u) w_next[u] = (w_ok && kb + u < kb_hi) ? load_run(w_ptr + (size_t)(kb + u) * 64) : zero_run();
+#pragma unroll
+    for (int it = 0; it < A_ITERS; ++it) {
+      const int v = tid + it * 256;           // vector index: (block u, row r, 16-byte piece p)
+      const int u = v / (ROWS * 8), r = (v / 8) % ROWS, p = v % 8;
+      a_next[it] = float4_t{0.f, 0.f, 0.f, 0.f};
+      if (v < A_VECS && r < m && kb + u < kb_hi)
+        a_next[it] = *reinterpret_cast<const float4_t*>(a + (size_t)r * k + (size_t)(kb + u) * 64 + p * 8);
+    }
+  };
+
+  if (kb_lo < kb_hi) fetch(kb_lo);
+  for (int kb = kb_lo; kb < kb_hi; kb += CHUNK) {
+    __syncthreads();  // the previous chunk has been read by every wave
+#pragma unroll
+    for (int it = 0; it < A_ITERS; ++it) {
+      const int v = tid + it * 256;
+      if (v < A_VECS) {
+        const int u = v / (ROWS * 8), r = (v / 8) % ROWS, p = v % 8;
+        *reinterpret_cast<float4_t*>(a_tile + (u * ROWS + r) * AS + p * 8) = a_next[it];
+      }
+    }
+    Run16 w_cur[CHUNK];
+#pragma unroll
+    for (int u = 0; u < CHUNK; ++u) w_cur[u] = w_next[u];
+    __syncthreads();
+    if (kb + CHUNK < kb_hi) fetch(kb + CHUNK);  // in flight while this chunk is multiplied
+#pragma unroll
+    for (int u = 0; u < CHUNK; ++u)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+        const bf16_t* src = a_tile + (u * ROWS + 16 * ct + i) * AS + 16 * g;
+        const bf16x8_t lo = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const float4_t*>(src));
+        const bf16x8_t hi = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const float4_t*>(src + 8));
+        acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[u].lo, lo, acc[ct], 0, 0, 0);
+        acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[u].hi, hi, acc[ct], 0, 0, 0);
+      }
+  }
+  float* dst = partial + (size_t)blockIdx.y * m * n;
+  const int col_n = blockIdx.x * 64 + 16 * wave + 4 * g;
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int col_m = 16 * ct + i;
+    if (col_m >= m) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (col_n + j < n) dst[(size_t)col_m * n + col_n + j] = acc[ct][j];
+  }
+}
+
+// partial: float32 [splits, M, N].  blocks_per_split * splits must cover K / 64.
+extern "C" int velox_skinny_gemm_splitk_bf16(const void* a, const void* w, float* partial, int m, int n, int k, int splits, hipStream_t stream) {
+  if (m <= 0 || n <= 0) return 0;
+  if (k % 64 != 0 || m > 64 || splits < 1) return -1;
+  const int blocks_total = k / 64;
+  const int per_split = (blocks_total + splits - 1) / splits;
+  dim3 grid((n + 63) / 64, splits);
+  if (m <= 32)
+    skinny_gemm_splitk_kernel<2><<<grid, 256, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, partial, m, n, k, per_split);
+  else
+    skinny_gemm_splitk_kernel<4><<<grid, 256, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, partial, m, n, k, per_split);
+  return (int)hipGetLastError();
+}

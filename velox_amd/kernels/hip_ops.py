@@ -65,7 +65,7 @@ class HipOps:
     def _declare_core(self) -> None:
         c = self._core
         c.velox_embed.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
-        c.velox_add_rmsnorm.argtypes = [_P, _P, _P, _P, _P, _I, _I, _F, _I, _I, _P]
+        c.velox_add_rmsnorm.argtypes = [_P, _P, _P, _P, _P, _I, _I, _F, _I, _I, _I, ctypes.c_longlong, _P]
         c.velox_silu_mul.argtypes = [_P, _P, _I, _I, _I, _P]
         c.velox_rope_kv_write.argtypes = [_P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_gemm_fma.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
@@ -73,6 +73,8 @@ class HipOps:
         c.velox_skinny_gemm_bf16.restype = _I
         c.velox_skinny_gemm_glu_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P]
         c.velox_skinny_gemm_glu_bf16.restype = _I
+        c.velox_skinny_gemm_splitk_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
+        c.velox_skinny_gemm_splitk_bf16.restype = _I
         c.velox_argmax.argtypes = [_P, _P, _I, _I, _P]
         c.velox_sample.argtypes = [_P, _P, _P, _I, _I, _P]
         c.velox_apply_penalties.argtypes = [_P, _P, _P, _P, _I, _I, _I, _P]
@@ -161,8 +163,13 @@ class HipOps:
             raise KernelError("add_rmsnorm: residual must be [T, H]")
         tokens, hidden = residual.shape
         self._check("weight", weight, torch.float32, (hidden,))
+        partials, partial_stride = 1, 0
         if delta is not None:
-            self._check("delta", delta, None, (tokens, hidden))
+            if delta.dim() == 3:  # partial sums of a split product, added here
+                partials, partial_stride = delta.shape[0], tokens * hidden
+                self._check("delta", delta, torch.float32, (partials, tokens, hidden), align=16)
+            else:
+                self._check("delta", delta, None, (tokens, hidden))
         if rows is not None:
             self._check("rows", rows, torch.int32)
             count = rows.shape[0]
@@ -170,7 +177,7 @@ class HipOps:
             count = tokens
         out = torch.empty((count, hidden), dtype=out_dtype, device=self.device)
         delta_code = _code(delta.dtype) if delta is not None else _code(out_dtype)
-        status = self._core.velox_add_rmsnorm(_ptr(residual), _ptr(delta), _ptr(rows), _ptr(weight), _ptr(out), count, hidden, float(eps), delta_code, _code(out_dtype), self._stream())
+        status = self._core.velox_add_rmsnorm(_ptr(residual), _ptr(delta), _ptr(rows), _ptr(weight), _ptr(out), count, hidden, float(eps), delta_code, _code(out_dtype), partials, partial_stride, self._stream())
         self._launched(status, "add_rmsnorm")
         return out
 
@@ -181,7 +188,9 @@ class HipOps:
         return self._norm(residual, delta, rows, weight, eps, out_dtype)
 
     # -- matrix products --------------------------------------------------------------------------
-    def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype) -> torch.Tensor:
+    def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype, partials_ok: bool = False) -> torch.Tensor:
+        """``x @ weight^T (+ bias)`` as ``[M, N]`` in ``out_dtype``.  With ``partials_ok`` the result may instead come back as
+        float32 partial sums ``[S, M, N]`` that the consumer adds (``add_rmsnorm`` does)."""
         self._check("x", x, align=16)
         self._check("weight", weight, align=16)
         if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
@@ -190,6 +199,9 @@ class HipOps:
         n = weight.shape[0]
         if bias is not None:
             self._check("bias", bias, torch.float32, (n,))
+        if (partials_ok and bias is None and self.use_skinny_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+                and 16 < m <= 64 and k % 64 == 0 and n <= 8192 and n % 4 == 0):
+            return self.skinny_gemm_splitk(x, weight)
         skinny_rows = 16 if n > 8192 else 32  # measured on MI355X: beyond this the library's kernels stream faster
         if self.use_skinny_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and m <= skinny_rows and k % 64 == 0:
             return self.skinny_gemm(x, weight, bias, out_dtype)
@@ -244,6 +256,24 @@ class HipOps:
         out = torch.empty((m, n), dtype=out_dtype, device=self.device)
         status = self._core.velox_skinny_gemm_glu_bf16(_ptr(x), _ptr(gate_up_weight), _ptr(out), m, n, k, int(waves), int(pairs), self._stream())
         self._launched(status, "skinny_gemm_glu")
+        return out
+
+    def skinny_gemm_splitk(self, x, weight, splits: Optional[int] = None) -> torch.Tensor:
+        """17 .. 64 rows times a bfloat16 weight with few rows and a long K: float32 partial sums ``[S, M, N]``."""
+        m, k = x.shape
+        n = weight.shape[0]
+        if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or m > 64 or k % 64 != 0:
+            raise KernelError(f"skinny_gemm_splitk: needs bfloat16 operands, M <= 64 and K % 64 == 0 (M={m}, K={k})")
+        self._check("x", x, align=16)
+        self._check("weight", weight, align=16)
+        if splits is None:
+            blocks = (n + 63) // 64
+            splits = max(1, min((2 * self.num_cus + blocks - 1) // blocks, k // 512, 16))
+        per_split = (k // 64 + splits - 1) // splits
+        splits = (k // 64 + per_split - 1) // per_split  # no empty slice
+        out = torch.empty((splits, m, n), dtype=torch.float32, device=self.device)
+        status = self._core.velox_skinny_gemm_splitk_bf16(_ptr(x), _ptr(weight), _ptr(out), m, n, k, splits, self._stream())
+        self._launched(status, "skinny_gemm_splitk")
         return out
 
     def gemm_fma(self, x, weight, bias, out_dtype):

@@ -92,7 +92,7 @@ class AttentionMixer(Mixer):
             ctx.max_q_len, meta.max_kv_len, self.scale, self.window,
             ctx.all_decode, ctx.workspace,
         )
-        return ops.linear(attn, self.o_weight, None, ctx.dtype)
+        return ops.linear(attn, self.o_weight, None, ctx.dtype, partials_ok=True)
 
 
 register_part("mixer", "attention", AttentionMixer)

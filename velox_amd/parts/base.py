@@ -107,7 +107,8 @@ class Mixer(Part):
         return None
 
     def forward(self, x: torch.Tensor, ctx, cache, owns_cache: bool = True) -> torch.Tensor:
-        """``x`` [T, H] in the run dtype -> [T, H].
+        """``x`` [T, H] in the run dtype -> [T, H] (or float32 partial sums [S, T, H] that the next norm adds up: what
+        ``ops.linear(..., partials_ok=True)`` returns may be handed on as it is).
 
         ``cache`` is this schedule entry's view of the cache (or the entry's it reads
         from when ``owns_cache`` is false: then nothing may be written to it).
@@ -117,6 +118,7 @@ class Mixer(Part):
 
 class FeedForward(Part):
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        """[T, H] -> [T, H], or float32 partial sums [S, T, H] (see ``Mixer.forward``)."""
         raise NotImplementedError
 
 
@@ -124,6 +126,7 @@ class Norm(Part):
     def forward(self, residual: torch.Tensor, delta: Optional[torch.Tensor], ctx, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``residual`` [T, H] float32.
 
+        ``delta`` is [T, H] or float32 partial sums [S, T, H], which are added first to last.
         With ``rows`` None: ``residual += delta`` in place (delta may be None) and the
         normalised residual comes back in the run dtype, [T, H].  With ``rows`` (int32
         [R]): nothing is changed and ``normalise(residual[rows] + delta[rows])`` comes back.

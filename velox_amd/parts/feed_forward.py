@@ -35,7 +35,7 @@ class GatedMLP(FeedForward):
     def forward(self, x, ctx):
         ops = ctx.ops
         act = ops.linear_silu_mul(x, self.gate_up_weight, ctx.dtype)
-        return ops.linear(act, self.down_weight, None, ctx.dtype)
+        return ops.linear(act, self.down_weight, None, ctx.dtype, partials_ok=True)
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)
