@@ -325,12 +325,42 @@ def test_skinny_gemm(ops, ref, out_dtype, m, n, k):
             expect = want + (b if b is not None else 0)
             atol = 1e-4 * scale if out_dtype == torch.float32 else 1e-2 * scale
             torch.testing.assert_close(got, expect, rtol=1e-2 if out_dtype == torch.bfloat16 else 1e-4, atol=atol)
+    # the weight in the order the lanes read it gives the same bits as the row-major weight
+    packed = ops.pack_rows(w)
+    got = ops.skinny_gemm(x, None, bias, out_dtype, packed=packed, n=n).float()  # with its own choice of waves and tiles
+    torch.testing.assert_close(got, want + bias, rtol=1e-2 if out_dtype == torch.bfloat16 else 1e-4, atol=atol)
+    for waves, row_tiles in ((4, 1), (16, 1), (4, 4)):
+        torch.testing.assert_close(ops.skinny_gemm(x, None, bias, out_dtype, waves=waves, row_tiles=row_tiles, packed=packed, n=n),
+                                   ops.skinny_gemm(x, w, bias, out_dtype, waves=waves, row_tiles=row_tiles), rtol=0, atol=0)
     # the same rows give the same bits whatever else is in the batch, as long as the batch stays in one size class
     # (up to 16, up to 32, up to 64 rows: the classes split K differently, which changes the order of the sums)
     fewer = 1 if m <= 16 else 17 if m <= 32 else 33
     if m > fewer:
         part = ops.skinny_gemm(x[:fewer].contiguous(), w, None, out_dtype)
         torch.testing.assert_close(ops.skinny_gemm(x, w, None, out_dtype)[:fewer], part, rtol=0, atol=0)
+
+
+def test_registered_weight_copies_die_with_their_weight(ops, ref):
+    """The lane-ordered copy belongs to one tensor object: another weight that later lands on the same address, or the
+    same weight after a change in place, must not be multiplied with the old copy."""
+    x = rand((4, 128), torch.bfloat16, 60)
+    first = rand((96, 128), torch.bfloat16, 61, 0.05)
+    ops.register_weight(first)
+    assert ops.packed_weight(first) is not None
+    address = first.data_ptr()
+    del first
+    for seed in range(62, 70):
+        other = rand((96, 128), torch.bfloat16, seed, 0.05)
+        assert ops.packed_weight(other) is None
+        torch.testing.assert_close(ops.linear(x, other, None, torch.float32), ref.linear(x, other, None, torch.float32), rtol=1e-4, atol=1e-4)
+        if other.data_ptr() == address:
+            break
+    ops.register_weight(other)
+    other.mul_(2.0)
+    assert ops.packed_weight(other) is None
+    torch.testing.assert_close(ops.linear(x, other, None, torch.float32), ref.linear(x, other, None, torch.float32), rtol=1e-4, atol=1e-4)
+    ops.register_weight(other, stacked=2)
+    assert ops.packed_weight(other, 2) is not None and ops.packed_weight(other, 1) is None
 
 
 @pytest.mark.parametrize("m,inter,k", [(1, 128, 64), (8, 18944, 3584), (16, 150, 128), (7, 1000, 192), (3, 16, 64)])
@@ -343,6 +373,10 @@ def test_skinny_gemm_with_silu_epilogue(ops, ref, m, inter, k):
     for waves, pairs in ((None, None), (4, 1), (8, 1), (4, 2), (8, 2)):
         got = ops.linear_silu_mul(x, w, torch.bfloat16, waves=waves, pairs=pairs).float()
         torch.testing.assert_close(got, want, rtol=1e-2, atol=1e-2 * scale)
+    packed = ops.pack_rows(w, matrices=2)
+    for waves, pairs in ((None, None), (4, 1), (8, 2)):
+        torch.testing.assert_close(ops.linear_silu_mul(x, w, torch.bfloat16, waves=waves, pairs=pairs, packed=packed),
+                                   ops.linear_silu_mul(x, w, torch.bfloat16, waves=waves, pairs=pairs), rtol=0, atol=0)
     # larger batches take the unfused route and agree with it
     big = rand((40, k), torch.bfloat16, 52)
     torch.testing.assert_close(ops.linear_silu_mul(big, w, torch.bfloat16).float(), ref.linear_silu_mul(big, w, torch.bfloat16).float(), rtol=3e-2, atol=3e-2 * scale)

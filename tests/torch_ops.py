@@ -61,6 +61,9 @@ class TorchOps:
     def prepare(self, model, dtype) -> None:
         pass
 
+    def register_weight(self, weight, stacked=1) -> None:
+        pass
+
     # -- embedding and norms ------------------------------------------------------------
     def embed(self, token_ids, table):
         return table[token_ids.long()].float()

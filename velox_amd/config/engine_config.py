@@ -53,6 +53,9 @@ class EngineConfig:
 
     enable_prefix_caching: bool = False
     enable_cuda_graphs: bool = True
+    # a second copy of every bfloat16 weight in the order the decode kernels read it: faster decoding for the
+    # weights' size again in memory (not a reference option)
+    pack_decode_weights: bool = True
     watermark: float = 0.01
 
     seed: Optional[int] = None

@@ -42,7 +42,10 @@ __device__ __forceinline__ Run16 zero_run() {
 // GLU = true: W holds two stacked matrices, gate rows [0, n) and up rows [n, 2n); the first RT / 2 row tiles of a
 // workgroup are gate rows, the others the up rows of the same output columns, and what is stored is
 // silu(gate) * up, computed on the float32 sums (the [M, 2n] product is never written).
-template <int RT, int CT, int WAVES, typename TO, bool GLU = false>
+// PACKED = true: W is stored tile by tile in the order the lanes read it, [row tile of 16][block of 64 indices][lane][16
+// elements] (rows padded with zeros to a multiple of 16; for GLU gate and up are padded separately), so that a wave's
+// load is one contiguous kilobyte.
+template <int RT, int CT, int WAVES, typename TO, bool GLU = false, bool PACKED = false>
 __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
                                                                  const float* __restrict__ bias, TO* __restrict__ out, int m, int n, int k) {
   constexpr int UNROLL = 4;  // blocks of 64 indices whose loads are issued together
@@ -64,9 +67,16 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     const int col = n0 + 16 * (rt % RTO) + i;          // output column this row of W contributes to
-    const size_t row = (size_t)col + (rt >= RTO ? n : 0);  // its row in W
     w_ok[rt] = col < n;
-    w_ptr[rt] = w + (w_ok[rt] ? row : 0) * k + 16 * g;
+    if constexpr (PACKED) {
+      const size_t tiles_per_matrix = (size_t)(n + 15) / 16;
+      const size_t tile = (size_t)(n0 / 16 + rt % RTO) + (rt >= RTO ? tiles_per_matrix : 0);
+      w_ok[rt] = n0 + 16 * (rt % RTO) < n;  // padded rows are zeros in memory
+      w_ptr[rt] = w + (w_ok[rt] ? tile : 0) * (size_t)(k / 64) * 1024 + lane * 16;
+    } else {
+      const size_t row = (size_t)col + (rt >= RTO ? n : 0);  // its row in W
+      w_ptr[rt] = w + (w_ok[rt] ? row : 0) * k + 16 * g;
+    }
   }
   const bf16_t* a_ptr[CT];
   bool a_ok[CT];
@@ -90,8 +100,9 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
     for (int u = 0; u < UNROLL; ++u) {
       const bool in_range = kb + u < kb_hi;
       const size_t k0 = (size_t)(kb + u) * 64;
+      const size_t w0 = PACKED ? (size_t)(kb + u) * 1024 : k0;
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) wr[u][rt] = (in_range && w_ok[rt]) ? load_run(w_ptr[rt] + k0) : zero_run();
+      for (int rt = 0; rt < RT; ++rt) wr[u][rt] = (in_range && w_ok[rt]) ? load_run(w_ptr[rt] + w0) : zero_run();
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) ar[u][ct] = (in_range && a_ok[ct]) ? load_run(a_ptr[ct] + k0) : zero_run();
     }
@@ -139,15 +150,25 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
 }
 
 template <int RT, int CT, int WAVES>
-static int launch_skinny_glu(const void* a, const void* w, void* out, int m, int n, int k, hipStream_t stream) {
+static int launch_skinny_glu(const void* a, const void* w, void* out, int m, int n, int k, bool packed, hipStream_t stream) {
   const int blocks = (n + 8 * RT - 1) / (8 * RT);
-  skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k);
+  if (packed)
+    skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k);
+  else
+    skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k);
   return (int)hipGetLastError();
 }
 
 template <int RT, int CT, int WAVES>
-static int launch_skinny(const void* a, const void* w, const float* bias, void* out, int m, int n, int k, int out_dtype, hipStream_t stream) {
+static int launch_skinny(const void* a, const void* w, const float* bias, void* out, int m, int n, int k, int out_dtype, bool packed, hipStream_t stream) {
   const int blocks = (n + 16 * RT - 1) / (16 * RT);
+  if (packed) {
+    if (out_dtype == VELOX_BF16)
+      skinny_gemm_kernel<RT, CT, WAVES, bf16_t, false, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (bf16_t*)out, m, n, k);
+    else
+      skinny_gemm_kernel<RT, CT, WAVES, float, false, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (float*)out, m, n, k);
+    return (int)hipGetLastError();
+  }
   if (out_dtype == VELOX_BF16)
     skinny_gemm_kernel<RT, CT, WAVES, bf16_t><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (bf16_t*)out, m, n, k);
   else
@@ -160,10 +181,10 @@ static int launch_skinny(const void* a, const void* w, const float* bias, void* 
 // row_tiles: 16-row tiles of W per wave for M <= 16 (1 or 4).  With 4 a wave reuses each activation fragment for 64 rows
 // of W, which quarters the traffic of the activations; worth it when N is large enough that N / 64 workgroups still fill the GPU.
 extern "C" int velox_skinny_gemm_bf16(const void* a, const void* w, const float* bias, void* out, int m, int n, int k, int out_dtype,
-                                      int waves, int row_tiles, hipStream_t stream) {
+                                      int waves, int row_tiles, int packed, hipStream_t stream) {
   if (m <= 0 || n <= 0) return 0;
   if (k % 64 != 0 || m > 64) return -1;
-#define PICK(RT, CT, W) return launch_skinny<RT, CT, W>(a, w, bias, out, m, n, k, out_dtype, stream)
+#define PICK(RT, CT, W) return launch_skinny<RT, CT, W>(a, w, bias, out, m, n, k, out_dtype, packed != 0, stream)
   if (m <= 16 && row_tiles >= 4) {
     if (waves >= 8) PICK(4, 1, 8);
     PICK(4, 1, 4);
@@ -185,19 +206,19 @@ extern "C" int velox_skinny_gemm_bf16(const void* a, const void* w, const float*
 
 // out[M, n] = silu(A Wgate^T) * (A Wup^T) with W = [Wgate; Wup] of 2n rows, bfloat16 in and out, M <= 32.
 // pairs: gate/up tile pairs per wave (1 or 2).
-extern "C" int velox_skinny_gemm_glu_bf16(const void* a, const void* w, void* out, int m, int n, int k, int waves, int pairs, hipStream_t stream) {
+extern "C" int velox_skinny_gemm_glu_bf16(const void* a, const void* w, void* out, int m, int n, int k, int waves, int pairs, int packed, hipStream_t stream) {
   if (m <= 0 || n <= 0) return 0;
   if (k % 64 != 0 || m > 32) return -1;
   if (m <= 16) {
     if (pairs >= 2) {
-      if (waves >= 8) return launch_skinny_glu<4, 1, 8>(a, w, out, m, n, k, stream);
-      return launch_skinny_glu<4, 1, 4>(a, w, out, m, n, k, stream);
+      if (waves >= 8) return launch_skinny_glu<4, 1, 8>(a, w, out, m, n, k, packed != 0, stream);
+      return launch_skinny_glu<4, 1, 4>(a, w, out, m, n, k, packed != 0, stream);
     }
-    if (waves >= 8) return launch_skinny_glu<2, 1, 8>(a, w, out, m, n, k, stream);
-    return launch_skinny_glu<2, 1, 4>(a, w, out, m, n, k, stream);
+    if (waves >= 8) return launch_skinny_glu<2, 1, 8>(a, w, out, m, n, k, packed != 0, stream);
+    return launch_skinny_glu<2, 1, 4>(a, w, out, m, n, k, packed != 0, stream);
   }
-  if (waves >= 8) return launch_skinny_glu<2, 2, 8>(a, w, out, m, n, k, stream);
-  return launch_skinny_glu<2, 2, 4>(a, w, out, m, n, k, stream);
+  if (waves >= 8) return launch_skinny_glu<2, 2, 8>(a, w, out, m, n, k, packed != 0, stream);
+  return launch_skinny_glu<2, 2, 4>(a, w, out, m, n, k, packed != 0, stream);
 }
 
 // ---------------------------------------------------------------------------------------------------------------

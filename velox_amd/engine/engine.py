@@ -101,6 +101,8 @@ class Engine:
         model = build_model(model_config, dtype, device, max_position=max_model_len)
         bind(model, dtype, device)
         needs = model.cache_needs()
+        if hasattr(ops, "pack_decode_weights"):
+            ops.pack_decode_weights = config.pack_decode_weights
         ops.prepare(model, dtype)
         num_pages = config.num_gpu_blocks
         if num_pages is None:

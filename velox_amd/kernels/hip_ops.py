@@ -59,6 +59,7 @@ class HipOps:
         self.num_cus = torch.cuda.get_device_properties(self.device).multi_processor_count
         self.use_library_gemm = True
         self.use_skinny_gemm = True
+        self.pack_decode_weights = True
         self._mm_out_dtype_ok: Optional[bool] = None
 
     # -- loading --------------------------------------------------------------------------------
@@ -69,9 +70,9 @@ class HipOps:
         c.velox_silu_mul.argtypes = [_P, _P, _I, _I, _I, _P]
         c.velox_rope_kv_write.argtypes = [_P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_gemm_fma.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
-        c.velox_skinny_gemm_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_skinny_gemm_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_skinny_gemm_bf16.restype = _I
-        c.velox_skinny_gemm_glu_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P]
+        c.velox_skinny_gemm_glu_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
         c.velox_skinny_gemm_glu_bf16.restype = _I
         c.velox_skinny_gemm_splitk_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
         c.velox_skinny_gemm_splitk_bf16.restype = _I
@@ -95,10 +96,39 @@ class HipOps:
         return lib
 
     def prepare(self, model, dtype) -> None:
-        """Builds (at first use) and loads what this model's mixers need."""
+        """Builds (at first use) and loads what this model's mixers need, and lets every part register the weights
+        that decode-sized products read (``Part.prepare_kernels``)."""
         for need in model.cache_needs():
             if need is not None and hasattr(need, "head_dim"):
                 self.attention_library(need.head_dim)
+        for part in model.all_parts():
+            part.prepare_kernels(self)
+
+    def register_weight(self, weight: torch.Tensor, stacked: int = 1) -> None:
+        """Keeps a second copy of a bfloat16 ``[N, K]`` weight in the order the skinny kernels' lanes read it (see
+        ``pack_rows``): decode-sized products then stream contiguous kilobytes.  ``stacked`` = 2 marks ``[Wgate; Wup]``.
+        Costs the weight's size again in memory; ``pack_decode_weights = False`` turns it off.  The copy hangs on the
+        tensor object itself, so it lives exactly as long as the weight and is found only through that object."""
+        if (not self.pack_decode_weights or weight is None or weight.dtype != torch.bfloat16 or weight.dim() != 2
+                or weight.shape[1] % 64 != 0 or weight.shape[0] % stacked != 0 or weight.device != self.device):
+            return
+        copies = getattr(weight, "_velox_packed", None)
+        if copies is None or copies["version"] != weight._version:
+            copies = {"version": weight._version}
+            weight._velox_packed = copies
+        if stacked in copies:
+            return
+        per_matrix = weight.shape[0] // stacked
+        whole_tiles = [c for key, c in copies.items() if key != "version"] if per_matrix % 16 == 0 else []
+        # with whole tiles every stacking gives the same bytes
+        copies[stacked] = whole_tiles[0] if whole_tiles else self.pack_rows(weight, stacked)
+
+    @staticmethod
+    def packed_weight(weight: torch.Tensor, stacked: int = 1) -> Optional[torch.Tensor]:
+        copies = getattr(weight, "_velox_packed", None)
+        if copies is None or copies["version"] != weight._version:
+            return None
+        return copies.get(stacked)
 
     def tune_library_products(self, shapes, token_counts, seconds_per_shape: float = 0.2) -> int:
         """Lets PyTorch's TunableOp time the library's candidate kernels for ``x[M, K] @ w[N, K]^T`` at the given
@@ -204,7 +234,7 @@ class HipOps:
             return self.skinny_gemm_splitk(x, weight)
         skinny_rows = 16 if n > 8192 else 32  # measured on MI355X: beyond this the library's kernels stream faster
         if self.use_skinny_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and m <= skinny_rows and k % 64 == 0:
-            return self.skinny_gemm(x, weight, bias, out_dtype)
+            return self.skinny_gemm(x, weight, bias, out_dtype, packed=self.packed_weight(weight))
         if self.use_library_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and bias is None:
             if out_dtype == torch.bfloat16:
                 return torch.nn.functional.linear(x, weight)
@@ -217,25 +247,48 @@ class HipOps:
                     self._mm_out_dtype_ok = False
         return self.gemm_fma(x, weight, bias, out_dtype)
 
-    def skinny_gemm(self, x, weight, bias, out_dtype, waves: Optional[int] = None, row_tiles: Optional[int] = None):
-        """Few rows (M <= 64) times a bfloat16 weight: the weight-streaming kernel of the decode step."""
+    @staticmethod
+    def pack_rows(weight: torch.Tensor, matrices: int = 1) -> torch.Tensor:
+        """``weight`` [N, K] bfloat16 (``matrices`` stacked matrices of N / matrices rows each) in the order the skinny
+        kernels' lanes read it: [row tile of 16][block of 64 indices][lane = 16 * (index / 16) + row][16 elements], each
+        matrix padded with zero rows to whole tiles.  A wave's load of a block is then one contiguous kilobyte."""
+        n_all, k = weight.shape
+        n = n_all // matrices
+        tiles = (n + 15) // 16
+        padded = torch.zeros((matrices, tiles * 16, k), dtype=weight.dtype, device=weight.device)
+        padded[:, :n] = weight.view(matrices, n, k)
+        # [matrix, tile, row i, block, group g, 16] -> [matrix, tile, block, g, i, 16]
+        return padded.view(matrices, tiles, 16, k // 64, 4, 16).permute(0, 1, 3, 4, 2, 5).contiguous().view(-1)
+
+    def skinny_gemm(self, x, weight, bias, out_dtype, waves: Optional[int] = None, row_tiles: Optional[int] = None, packed: Optional[torch.Tensor] = None, n: Optional[int] = None):
+        """Few rows (M <= 64) times a bfloat16 weight: the weight-streaming kernel of the decode step.  ``packed`` is
+        ``pack_rows(weight)``, used instead of ``weight`` when given (``n`` = rows of the weight)."""
         m, k = x.shape
-        n = weight.shape[0]
-        if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or m > 64 or k % 64 != 0:
+        n = weight.shape[0] if weight is not None else n
+        if packed is not None:
+            weight_arg = packed
+            if packed.dtype != torch.bfloat16 or packed.numel() != ((n + 15) // 16) * 16 * k:
+                raise KernelError("skinny_gemm: the packed weight does not match N and K")
+        else:
+            weight_arg = weight
+        if x.dtype != torch.bfloat16 or weight_arg.dtype != torch.bfloat16 or m > 64 or k % 64 != 0:
             raise KernelError(f"skinny_gemm: needs bfloat16 operands, M <= 64 and K % 64 == 0 (M={m}, K={k})")
         if row_tiles is None:
-            row_tiles = 4 if (m <= 16 and n >= 64 * 2 * self.num_cus) else 1
+            # 64 rows per wave quarter the activation traffic, which pays for the row-major weight only
+            row_tiles = 4 if (m <= 16 and n >= 64 * 2 * self.num_cus and (packed is None or m > 8)) else 1
+        if waves is None and packed is not None and row_tiles == 1 and m <= 16:
+            waves = 8
         if waves is None:
             rows_per_block = 16 * row_tiles if m <= 16 else 32
             blocks = (n + rows_per_block - 1) // rows_per_block
             wanted = (8 * self.num_cus + blocks - 1) // blocks  # about eight waves per SIMD lane group across the GPU
             waves = 16 if wanted > 8 else 8 if wanted > 4 else 4
         out = torch.empty((m, n), dtype=out_dtype, device=self.device)
-        status = self._core.velox_skinny_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), m, n, k, _code(out_dtype), int(waves), int(row_tiles), self._stream())
+        status = self._core.velox_skinny_gemm_bf16(_ptr(x), _ptr(weight_arg), _ptr(bias), _ptr(out), m, n, k, _code(out_dtype), int(waves), int(row_tiles), 1 if packed is not None else 0, self._stream())
         self._launched(status, "skinny_gemm")
         return out
 
-    def linear_silu_mul(self, x: torch.Tensor, gate_up_weight: torch.Tensor, out_dtype: torch.dtype, waves: Optional[int] = None, pairs: Optional[int] = None) -> torch.Tensor:
+    def linear_silu_mul(self, x: torch.Tensor, gate_up_weight: torch.Tensor, out_dtype: torch.dtype, waves: Optional[int] = None, pairs: Optional[int] = None, packed: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``silu(x Wgate^T) * (x Wup^T)`` for ``W = [Wgate; Wup]``.  Decode-sized bfloat16 batches run as one kernel that
         never writes the [M, 2I] product; everything else is the product followed by the SiLU kernel."""
         m, k = x.shape
@@ -244,17 +297,17 @@ class HipOps:
                  and m <= 16 and k % 64 == 0 and two_n % 2 == 0 and x.dim() == 2 and gate_up_weight.shape[1] == k)
         if not fused:
             return self.silu_mul(self.linear(x, gate_up_weight, None, out_dtype))
+        if packed is None:
+            packed = self.packed_weight(gate_up_weight, 2)
         self._check("x", x, align=16)
         self._check("gate_up_weight", gate_up_weight, align=16)
         n = two_n // 2
         if pairs is None:
-            pairs = 2 if n >= 32 * 2 * self.num_cus else 1
+            pairs = 1  # measured on MI355X: two pairs per wave never paid, packed or not
         if waves is None:
-            blocks = (n + 16 * pairs - 1) // (16 * pairs)
-            wanted = (8 * self.num_cus + blocks - 1) // blocks
-            waves = 8 if wanted > 4 else 4
+            waves = 8
         out = torch.empty((m, n), dtype=out_dtype, device=self.device)
-        status = self._core.velox_skinny_gemm_glu_bf16(_ptr(x), _ptr(gate_up_weight), _ptr(out), m, n, k, int(waves), int(pairs), self._stream())
+        status = self._core.velox_skinny_gemm_glu_bf16(_ptr(x), _ptr(packed if packed is not None else gate_up_weight), _ptr(out), m, n, k, int(waves), int(pairs), 1 if packed is not None else 0, self._stream())
         self._launched(status, "skinny_gemm_glu")
         return out
 

@@ -71,6 +71,10 @@ class AttentionMixer(Mixer):
     def cache_need(self):
         return PagedNeed(self.num_kv_heads, self.head_dim, self.window)
 
+    def prepare_kernels(self, ops) -> None:
+        ops.register_weight(self.qkv_weight)
+        ops.register_weight(self.o_weight)
+
     def forward(self, x, ctx, cache, owns_cache: bool = True):
         ops = ctx.ops
         # the bias is added (in float32) by the kernel that rotates and stores, which reads qkv anyway

@@ -76,6 +76,10 @@ class Part:
     def finalize(self, device: torch.device, dtype: torch.dtype) -> None:
         """Called once after the weights are bound (build tables, derived tensors)."""
 
+    def prepare_kernels(self, ops) -> None:
+        """Called once with the kernels' handle: a part may register the weights its decode-sized products read
+        (``ops.register_weight``).  Nothing has to be done here."""
+
 
 # ----------------------------------------------------------------------------------------
 # what a mixer needs of the cache manager

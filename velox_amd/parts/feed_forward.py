@@ -32,6 +32,10 @@ class GatedMLP(FeedForward):
             "down_weight": single("down_proj.weight", (h, i)),
         }
 
+    def prepare_kernels(self, ops) -> None:
+        ops.register_weight(self.gate_up_weight, stacked=2)
+        ops.register_weight(self.down_weight)
+
     def forward(self, x, ctx):
         ops = ctx.ops
         act = ops.linear_silu_mul(x, self.gate_up_weight, ctx.dtype)

@@ -106,6 +106,9 @@ class OutputHead(Part):
             return {"weight": base}
         return {"weight": Param(base.shape, base.sources, base.source_shapes, base.role, base.init, alias_of=self.tied_to)}
 
+    def prepare_kernels(self, ops) -> None:
+        ops.register_weight(self.weight)
+
     def forward(self, hidden_rows: torch.Tensor, ctx) -> torch.Tensor:
         return ctx.ops.linear(hidden_rows, self.weight, None, torch.float32)
 
