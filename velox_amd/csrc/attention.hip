@@ -30,7 +30,6 @@
 
 constexpr int D = VELOX_HEAD_DIM;
 static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple of 16 between 16 and 256");
-constexpr int ROWS_PER_BLOCK = 64;
 
 template <typename T> struct Frag;
 template <> struct Frag<float> { float4_t v; };
@@ -129,7 +128,9 @@ template <> struct Softmax<bf16_t> {
 
 constexpr int PREFILL_PAGE_IDS = 2048;
 
-template <typename T, int BN>
+// CT = 16-row tiles per wave: a workgroup owns 64 * CT rows.  With CT = 2 every K and V^T operand read from LDS feeds
+// two matrix instructions, which is what long portions of prompts need; a row's arithmetic is the same for every CT.
+template <typename T, int BN, int CT>
 __global__ void __launch_bounds__(256) paged_attention_kernel(
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
@@ -148,6 +149,7 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
   constexpr int NKB = BN / KB;                  // contraction blocks of P V
   constexpr int TPB = KB / 16;                  // S^T tiles per key block
   constexpr int NC = D / 16;                    // 16-channel tiles of the output
+  constexpr int ROWS_PER_BLOCK = 64 * CT;
   __shared__ __attribute__((aligned(16))) T k_tile[BN * KS];
   __shared__ __attribute__((aligned(16))) T v_tile[D * VS];
   __shared__ int page_ids[PREFILL_PAGE_IDS];
@@ -165,14 +167,20 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
   const int kv_len = kv_lens[b];
   const int ctx = kv_len - q_len;
   const int rows_total = q_len * group;
-  const int r0 = blockIdx.x * ROWS_PER_BLOCK;
+  // late rows read the most keys: they go first, so that the long workgroups do not start last
+  const int r0 = (gridDim.x - 1 - blockIdx.x) * ROWS_PER_BLOCK;
   if (r0 >= rows_total) return;
 
-  const int r = r0 + wave * 16 + i;
-  const bool row_ok = r < rows_total;
-  const int tok = row_ok ? r / group : 0;
-  const int head = kvh * group + (row_ok ? r % group : 0);
-  const int pos = ctx + tok;
+  bool row_ok[CT];
+  int tok[CT], head[CT], pos[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int r = r0 + (wave * CT + ct) * 16 + i;
+    row_ok[ct] = r < rows_total;
+    tok[ct] = row_ok[ct] ? r / group : 0;
+    head[ct] = kvh * group + (row_ok[ct] ? r % group : 0);
+    pos[ct] = ctx + tok[ct];
+  }
 
   // keys this workgroup has to visit
   const int first_tok = r0 / group;
@@ -193,8 +201,12 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
   if (tile_hi > tiles_total) tile_hi = tiles_total;
 
   // positions of this wave's rows: tiles after the last one are skipped, tiles before the first one need no mask
-  int wave_last_pos = row_ok ? pos : -1;
-  int wave_first_pos = row_ok ? pos : 0x7fffffff;
+  int wave_last_pos = -1, wave_first_pos = 0x7fffffff;
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    if (row_ok[ct] && pos[ct] > wave_last_pos) wave_last_pos = pos[ct];
+    if (row_ok[ct] && pos[ct] < wave_first_pos) wave_first_pos = pos[ct];
+  }
 #pragma unroll
   for (int offset = 32; offset > 0; offset >>= 1) {
     const int hi = __shfl_xor(wave_last_pos, offset, VELOX_WAVE);
@@ -203,36 +215,38 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
     wave_first_pos = lo < wave_first_pos ? lo : wave_first_pos;
   }
 
-  // page ids of the keys this workgroup visits, and zeros in the padding columns of the K tile
+  // Page ids of the keys this workgroup visits are kept in LDS, a window of PREFILL_PAGE_IDS pages at a time (the tile
+  // loop moves the window on when the next tile would leave it); zeros go to the padding columns of the K tile.
   const int* table = block_tables + (size_t)b * table_width;
-  const int first_page = (n_begin + tile_lo * BN) >> page_shift;
-  {
-    const int last_key = n_begin + tile_hi * BN < kv_len ? n_begin + tile_hi * BN : kv_len;
-    const int num_pages = tile_hi > tile_lo ? ((last_key - 1) >> page_shift) - first_page + 1 : 0;
+  const int last_key = n_begin + tile_hi * BN < kv_len ? n_begin + tile_hi * BN : kv_len;
+  const int last_page = tile_hi > tile_lo ? (last_key - 1) >> page_shift : -1;
+  int first_page = (n_begin + tile_lo * BN) >> page_shift;  // first page of the window
+  auto load_page_ids = [&]() {
+    const int num_pages = last_page - first_page + 1;
     for (int p = tid; p < num_pages && p < PREFILL_PAGE_IDS; p += 256) page_ids[p] = table[first_page + p];
-    if constexpr (DP > D) {
-      for (int e = tid; e < BN * (DP - D); e += 256) k_tile[(e / (DP - D)) * KS + D + e % (DP - D)] = from_f32<T>(0.f);
-    }
-  }
-  auto page_of = [&](int n) -> size_t {
-    const int p = (n >> page_shift) - first_page;
-    return (size_t)(p < PREFILL_PAGE_IDS ? page_ids[p] : table[first_page + p]);
   };
+  load_page_ids();
+  if constexpr (DP > D) {
+    for (int e = tid; e < BN * (DP - D); e += 256) k_tile[(e / (DP - D)) * KS + D + e % (DP - D)] = from_f32<T>(0.f);
+  }
+  auto page_of = [&](int n) -> size_t { return (size_t)page_ids[(n >> page_shift) - first_page]; };
 
-  Operand qf[NQB];
-  {
-    const T* qp = qkv + (size_t)(q_start + tok) * qkv_stride + (size_t)head * D + VEC * g;
+  Operand qf[CT][NQB];
+  float m_i[CT], l_i[CT];
+  float4_t acc_o[CT][NC];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const T* qp = qkv + (size_t)(q_start + tok[ct]) * qkv_stride + (size_t)head[ct] * D + VEC * g;
 #pragma unroll
     for (int cb = 0; cb < NQB; ++cb) {
-      const bool inside = row_ok && (KB * cb + VEC * g < D);
-      qf[cb] = inside ? load_operand<T>(qp + KB * cb) : __builtin_bit_cast(Operand, float4_t{0.f, 0.f, 0.f, 0.f});
+      const bool inside = row_ok[ct] && (KB * cb + VEC * g < D);
+      qf[ct][cb] = inside ? load_operand<T>(qp + KB * cb) : __builtin_bit_cast(Operand, float4_t{0.f, 0.f, 0.f, 0.f});
     }
-  }
-
-  float m_i = -INFINITY, l_i = 0.f;
-  float4_t acc_o[NC];
+    m_i[ct] = -INFINITY;
+    l_i[ct] = 0.f;
 #pragma unroll
-  for (int c = 0; c < NC; ++c) acc_o[c] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < NC; ++c) acc_o[ct][c] = float4_t{0.f, 0.f, 0.f, 0.f};
+  }
   const float scale_eff = scale * Softmax<T>::SCALE;
 
   // ---- staging: global -> registers (issued a tile ahead) -> LDS; what does not change from tile to tile is computed once
@@ -245,7 +259,7 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
   int k_key[ITERS], k_col[ITERS], v_dd[ITERS], v_key[ITERS], v_lds[ITERS];
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
-    const int v = tid + it * 256;
+    const int v = tid + it * 256 < VECS ? tid + it * 256 : VECS - 1;  // (the spare threads of a last pass repeat its last vector)
     k_key[it] = v / VPR;
     k_col[it] = (v % VPR) * VEC;
     const int rn = (v >> run_shift) / D;            // run index within the tile
@@ -258,33 +272,42 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
   }
   float4_t k_regs[ITERS], v_regs[ITERS];
 
+  // Every load is issued without a branch around it (a key beyond the sequence is read from the last valid place and
+  // zeroed when the tile is written to LDS): a branch per load would make each wait for the one before.
   auto fetch = [&](int n0) {
+    const T* k_src[ITERS];
+    const T* v_src[ITERS];
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-      k_regs[it] = float4_t{0.f, 0.f, 0.f, 0.f};
-      v_regs[it] = float4_t{0.f, 0.f, 0.f, 0.f};
-      if (tid + it * 256 >= VECS) continue;
-      const int nk = n0 + k_key[it];
-      if (nk < kv_len)
-        k_regs[it] = *reinterpret_cast<const float4_t*>(
-            k_cache + (((page_of(nk) * nkv + kvh) << page_shift) + (nk & (page_size - 1))) * D + k_col[it]);
-      if (v_by_vectors) {
-        const int nv = n0 + v_key[it];
-        if (nv < kv_len) {
-          Vec16<T> x;
-          x.v = *reinterpret_cast<const float4_t*>(v_cache + (((page_of(nv) * nkv + kvh) * D + v_dd[it]) << page_shift) + (nv & (page_size - 1)));
-          if (nv + VEC > kv_len) mask_tail(x, kv_len - nv);
-          v_regs[it] = x.v;
-        }
-      }
+      int nk = n0 + k_key[it];
+      nk = nk < kv_len ? nk : kv_len - 1;
+      k_src[it] = k_cache + (((page_of(nk) * nkv + kvh) << page_shift) + (nk & (page_size - 1))) * D + k_col[it];
+      int nv = n0 + v_key[it];
+      nv = nv < kv_len ? nv : (kv_len - 1) & ~(VEC - 1);
+      v_src[it] = v_cache + (((page_of(nv) * nkv + kvh) * D + v_dd[it]) << page_shift) + (nv & (page_size - 1));
+    }
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) k_regs[it] = *reinterpret_cast<const float4_t*>(k_src[it]);
+    if (v_by_vectors) {
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) v_regs[it] = *reinterpret_cast<const float4_t*>(v_src[it]);
     }
   };
   auto commit = [&](int n0) {
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-      if (tid + it * 256 >= VECS) continue;
+      if constexpr (VECS % 256 != 0) {
+        if (tid + it * 256 >= VECS) continue;
+      }
+      if (n0 + k_key[it] >= kv_len) k_regs[it] = float4_t{0.f, 0.f, 0.f, 0.f};
       *reinterpret_cast<float4_t*>(k_tile + k_key[it] * KS + k_col[it]) = k_regs[it];
       if (v_by_vectors) {
+        if (n0 + v_key[it] + VEC > kv_len) {
+          Vec16<T> x;
+          x.v = v_regs[it];
+          mask_tail(x, kv_len - n0 - v_key[it]);
+          v_regs[it] = x.v;
+        }
         if constexpr (KB == 32) {
           // keys 8m .. 8m+7 of a 32-key block: the first four belong to lane group (2m) % 4 of S^T tile (2m) / 4, the
           // next four to lane group (2m+1) % 4 of tile (2m+1) / 4; lane group g's column run is 8g + 4 * tile
@@ -325,92 +348,115 @@ __global__ void __launch_bounds__(256) paged_attention_kernel(
     __syncthreads();  // the previous tile has been read by every wave
     commit(n0);
     __syncthreads();
-    if (tile + 1 < tile_hi) fetch(n0 + BN);  // in flight while this tile is computed
+    if (tile + 1 < tile_hi) {
+      if (((n0 + 2 * BN - 1) >> page_shift) - first_page >= PREFILL_PAGE_IDS) {  // the same for every thread
+        first_page = (n0 + BN) >> page_shift;
+        load_page_ids();
+        __syncthreads();
+      }
+      fetch(n0 + BN);  // in flight while this tile is computed
+    }
     if (n0 > wave_last_pos) continue;        // nothing this wave may read; it still took part in the staging
 
     // ---- S^T = K Q^T ----------------------------------------------------------------------
-    float4_t s[NT];
+    float4_t s[CT][NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      s[t] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int cb = 0; cb < NQB; ++cb)
-        s[t] = B::mma(load_operand<T>(k_tile + (16 * t + i) * KS + KB * cb + VEC * g), qf[cb], s[t]);
+      for (int ct = 0; ct < CT; ++ct) s[ct][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int cb = 0; cb < NQB; ++cb) {
+        const Operand kf = load_operand<T>(k_tile + (16 * t + i) * KS + KB * cb + VEC * g);
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) s[ct][t] = B::mma(kf, qf[ct][cb], s[ct][t]);
+      }
     }
     // ---- scale, mask (only where the tile crosses a row's limits), running maximum ----------
     const bool whole = n0 + BN <= kv_len && n0 + BN - 1 <= wave_first_pos && (window <= 0 || n0 > wave_last_pos - window);
-    float mx = -INFINITY;
-    if (whole) {
+    float alpha[CT];
+    Operand pf[CT][NKB];
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
+    for (int ct = 0; ct < CT; ++ct) {
+      float mx = -INFINITY;
+      if (whole) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          s[t][j] *= scale_eff;
-          mx = fmaxf(mx, s[t][j]);
-        }
-    } else {
+        for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
+          for (int j = 0; j < 4; ++j) {
+            s[ct][t][j] *= scale_eff;
+            mx = fmaxf(mx, s[ct][t][j]);
+          }
+      } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int n = n0 + 16 * t + 4 * g + j;
-          const bool keep = row_ok && n < kv_len && n <= pos && (window <= 0 || n > pos - window);
-          s[t][j] = keep ? s[t][j] * scale_eff : -INFINITY;
-          mx = fmaxf(mx, s[t][j]);
-        }
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int n = n0 + 16 * t + 4 * g + j;
+            const bool keep = row_ok[ct] && n < kv_len && n <= pos[ct] && (window <= 0 || n > pos[ct] - window);
+            s[ct][t][j] = keep ? s[ct][t][j] * scale_eff : -INFINITY;
+            mx = fmaxf(mx, s[ct][t][j]);
+          }
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, VELOX_WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, VELOX_WAVE));
+      const float m_new = fmaxf(m_i[ct], mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      alpha[ct] = (m_i[ct] == -INFINITY) ? 0.f : Softmax<T>::exp_of(m_i[ct] - m_safe);
+      float psum = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb) {
+        Vec16<T> packed;
+        T* e = reinterpret_cast<T*>(&packed.v);
+#pragma unroll
+        for (int u = 0; u < TPB; ++u)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float sv = s[ct][kb * TPB + u][j];
+            const float p = (sv == -INFINITY) ? 0.f : Softmax<T>::exp_of(sv - m_safe);
+            psum += p;
+            e[4 * u + j] = from_f32<T>(p);
+          }
+        pf[ct][kb] = __builtin_bit_cast(Operand, packed.v);
+      }
+      l_i[ct] = l_i[ct] * alpha[ct] + psum;  // partial over this lane's keys; the four lane groups are summed at the end
+      m_i[ct] = m_new;
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, VELOX_WAVE));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, VELOX_WAVE));
-    const float m_new = fmaxf(m_i, mx);
-    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = (m_i == -INFINITY) ? 0.f : Softmax<T>::exp_of(m_i - m_safe);
-    float psum = 0.f;
-    Operand pf[NKB];
-#pragma unroll
-    for (int kb = 0; kb < NKB; ++kb) {
-      Vec16<T> packed;
-      T* e = reinterpret_cast<T*>(&packed.v);
-#pragma unroll
-      for (int u = 0; u < TPB; ++u)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float sv = s[kb * TPB + u][j];
-          const float p = (sv == -INFINITY) ? 0.f : Softmax<T>::exp_of(sv - m_safe);
-          psum += p;
-          e[4 * u + j] = from_f32<T>(p);
-        }
-      pf[kb] = __builtin_bit_cast(Operand, packed.v);
-    }
-    l_i = l_i * alpha + psum;  // partial over this lane's keys; the four lane groups are summed at the end
-    m_i = m_new;
     // ---- O^T = O^T * alpha + V^T P^T ------------------------------------------------------
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
-      acc_o[c] = acc_o[c] * alpha;
 #pragma unroll
-      for (int kb = 0; kb < NKB; ++kb)
-        acc_o[c] = B::mma(load_operand<T>(v_tile + (16 * c + i) * VS + KB * kb + VEC * g), pf[kb], acc_o[c]);
+      for (int ct = 0; ct < CT; ++ct) acc_o[ct][c] = acc_o[ct][c] * alpha[ct];
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb) {
+        const Operand vf = load_operand<T>(v_tile + (16 * c + i) * VS + KB * kb + VEC * g);
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) acc_o[ct][c] = B::mma(vf, pf[ct][kb], acc_o[ct][c]);
+      }
     }
   }
 
-  l_i += __shfl_xor(l_i, 16, VELOX_WAVE);
-  l_i += __shfl_xor(l_i, 32, VELOX_WAVE);
-  if (!row_ok) return;
-  const float inv = l_i > 0.f ? 1.f / l_i : 1.f;
-  const size_t token = (size_t)(q_start + tok);
-  if (splits == 1) {
-    T* dst = out + (token * nh + head) * D + 4 * g;
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
+  for (int ct = 0; ct < CT; ++ct) {
+    float l = l_i[ct];
+    l += __shfl_xor(l, 16, VELOX_WAVE);
+    l += __shfl_xor(l, 32, VELOX_WAVE);
+    if (!row_ok[ct]) continue;
+    const float inv = l > 0.f ? 1.f / l : 1.f;
+    const size_t token = (size_t)(q_start + tok[ct]);
+    if (splits == 1) {
+      T* dst = out + (token * nh + head[ct]) * D + 4 * g;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) dst[16 * c + j] = from_f32<T>(acc_o[c][j] * inv);
+      for (int c = 0; c < NC; ++c) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[16 * c + j] = from_f32<T>(acc_o[ct][c][j] * inv);
+      }
+    } else {
+      const size_t slot = ((size_t)split * total_tokens + token) * nh + head[ct];
+      float* dst = part_o + slot * D + 4 * g;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) *reinterpret_cast<float4_t*>(dst + 16 * c) = acc_o[ct][c] * inv;
+      if (g == 0) part_lse[slot] = l > 0.f ? m_i[ct] * Softmax<T>::LN_UNIT + logf(l) : -INFINITY;
     }
-  } else {
-    const size_t slot = ((size_t)split * total_tokens + token) * nh + head;
-    float* dst = part_o + slot * D + 4 * g;
-#pragma unroll
-    for (int c = 0; c < NC; ++c) *reinterpret_cast<float4_t*>(dst + 16 * c) = acc_o[c] * inv;
-    if (g == 0) part_lse[slot] = l_i > 0.f ? m_i * Softmax<T>::LN_UNIT + logf(l_i) : -INFINITY;
   }
 }
 
@@ -656,9 +702,9 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
     merge_splits_kernel<T><<<dim3(total_tokens, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens);
     return (int)hipGetLastError();
   }
-  const int row_tiles = (max_q_len * group + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
-  dim3 grid(row_tiles, nkv, num_seqs * splits);
-  paged_attention_kernel<T, BN><<<grid, 256, 0, stream>>>(
+  // (two row tiles per wave, CT = 2, need more registers than two waves per SIMD leave and measured slower)
+  dim3 grid((max_q_len * group + 63) / 64, nkv, num_seqs * splits);
+  paged_attention_kernel<T, BN, 1><<<grid, 256, 0, stream>>>(
       (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
       part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
   int status = (int)hipGetLastError();
