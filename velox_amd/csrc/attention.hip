@@ -530,38 +530,31 @@ __global__ void __launch_bounds__(256) decode_attention_kernel(
     for (int c = 0; c < NC; ++c) qf[c] = row_ok ? load_frag<T>(qp + 16 * c) : zero_frag<T>();
   }
   __syncthreads();
+  // (the launcher sends a step here only if a split's keys span at most DECODE_PAGE_IDS pages; the clamp keeps a
+  // violated promise from reading outside the array)
   auto page_of = [&](int n) -> size_t {
     const int p = (n >> page_shift) - first_page;
-    return (size_t)(p < DECODE_PAGE_IDS ? page_ids[p] : table[first_page + p]);
+    return (size_t)page_ids[p < DECODE_PAGE_IDS ? p : DECODE_PAGE_IDS - 1];
   };
 
   struct Tile {
     Frag<T> k[NC];
     Frag<T> v[NC];
   };
+  // No branch surrounds a load, so the loads of a tile do not wait for those of the tiles before it: a key beyond the
+  // sequence is read from the last valid place instead; its score is masked and its values are zeroed when the
+  // tile is used.
   auto load_tile = [&](Tile& tile, int t) {
-    const int n_k = n_begin + 16 * t + i;      // the key whose row this lane reads
-    const int n_v = n_begin + 16 * t + 4 * g;  // the first of the four keys whose values this lane reads
-    if (n_k < kv_len) {
-      const T* kp = k_cache + ((page_of(n_k) * nkv + kvh) * page_size + (n_k & (page_size - 1))) * D + 4 * g;
+    int n_k = n_begin + 16 * t + i;      // the key whose row this lane reads
+    int n_v = n_begin + 16 * t + 4 * g;  // the first of the four keys whose values this lane reads
+    n_k = n_k < kv_len ? n_k : kv_len - 1;
+    n_v = n_v < kv_len ? n_v : (kv_len - 1) & ~3;
+    const T* kp = k_cache + ((page_of(n_k) * nkv + kvh) * page_size + (n_k & (page_size - 1))) * D + 4 * g;
+    const T* vp = v_cache + ((page_of(n_v) * nkv + kvh) * D + i) * page_size + (n_v & (page_size - 1));
 #pragma unroll
-      for (int c = 0; c < NC; ++c) tile.k[c] = load_frag<T>(kp + 16 * c);
-    } else {
+    for (int c = 0; c < NC; ++c) tile.k[c] = load_frag<T>(kp + 16 * c);
 #pragma unroll
-      for (int c = 0; c < NC; ++c) tile.k[c] = zero_frag<T>();
-    }
-    if (n_v < kv_len) {
-      const T* vp = v_cache + ((page_of(n_v) * nkv + kvh) * D + i) * page_size + (n_v & (page_size - 1));
-#pragma unroll
-      for (int c = 0; c < NC; ++c) tile.v[c] = load_frag<T>(vp + (size_t)16 * c * page_size);
-      if (n_v + 4 > kv_len) {
-#pragma unroll
-        for (int c = 0; c < NC; ++c) mask_frag(tile.v[c], kv_len - n_v);
-      }
-    } else {
-#pragma unroll
-      for (int c = 0; c < NC; ++c) tile.v[c] = zero_frag<T>();
-    }
+    for (int c = 0; c < NC; ++c) tile.v[c] = load_frag<T>(vp + (size_t)16 * c * page_size);
   };
 
   float m_i = -INFINITY, l_i = 0.f;
@@ -569,7 +562,12 @@ __global__ void __launch_bounds__(256) decode_attention_kernel(
 #pragma unroll
   for (int c = 0; c < NC; ++c) acc_o[c] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  auto compute_tile = [&](const Tile& tile, int t) {
+  auto compute_tile = [&](Tile& tile, int t) {
+    if (n_begin + 16 * t + 16 > kv_len) {  // the sequence ends inside this tile (the same for the whole wave)
+      const int valid = kv_len - (n_begin + 16 * t + 4 * g);
+#pragma unroll
+      for (int c = 0; c < NC; ++c) mask_frag(tile.v[c], valid);
+    }
     float4_t s = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int c = 0; c < NC; ++c) s = mma16(tile.k[c], qf[c], s);
@@ -689,10 +687,13 @@ template <typename T> constexpr int tile_keys() { return (sizeof(T) * D > 512) ?
 template <typename T>
 static int launch(const void* qkv, int qkv_stride, const void* k_cache, const void* v_cache, const int* block_tables, int table_width,
                   const int* cu_q, const int* kv_lens, void* out, float* part_o, float* part_lse, int num_seqs, int total_tokens,
-                  int max_q_len, int nh, int nkv, int page_shift, float scale, int window, int splits, hipStream_t stream) {
+                  int max_q_len, int max_kv_len, int nh, int nkv, int page_shift, float scale, int window, int splits, hipStream_t stream) {
   constexpr int BN = tile_keys<T>();
   const int group = nh / nkv;
-  if (max_q_len == 1 && total_tokens == num_seqs && group <= 16 && page_shift >= 2 && sizeof(T) * D <= 512) {
+  // the streaming kernel keeps the page ids of a split's keys in LDS: they have to fit
+  const int keys_per_split = (((max_kv_len + 15) / 16 + splits - 1) / splits) * 16;
+  const bool ids_fit = (keys_per_split >> page_shift) + 2 <= DECODE_PAGE_IDS;
+  if (max_q_len == 1 && total_tokens == num_seqs && group <= 16 && page_shift >= 2 && sizeof(T) * D <= 512 && ids_fit) {
     // every sequence decodes one token: the streaming kernel
     decode_attention_kernel<T><<<dim3(splits, nkv, num_seqs), 256, 0, stream>>>(
         (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, kv_lens, (T*)out, part_o, part_lse,
@@ -718,13 +719,13 @@ extern "C" int velox_attention_head_dim() { return D; }
 // part_o: float32 [splits, total_tokens, nh, D]; part_lse: float32 [splits, total_tokens, nh]; both unused when splits == 1.
 extern "C" int velox_paged_attention(const void* qkv, int qkv_stride, const void* k_cache, const void* v_cache,
                                      const int* block_tables, int table_width, const int* cu_q, const int* kv_lens, void* out,
-                                     float* part_o, float* part_lse, int num_seqs, int total_tokens, int max_q_len, int nh, int nkv,
-                                     int page_shift, float scale, int window, int splits, int dtype, hipStream_t stream) {
+                                     float* part_o, float* part_lse, int num_seqs, int total_tokens, int max_q_len, int max_kv_len,
+                                     int nh, int nkv, int page_shift, float scale, int window, int splits, int dtype, hipStream_t stream) {
   if (num_seqs <= 0 || total_tokens <= 0) return 0;
-  if (nh % nkv != 0 || splits < 1 || page_shift < 0) return -1;
+  if (nh % nkv != 0 || splits < 1 || page_shift < 0 || max_kv_len < 1) return -1;
   if (dtype == VELOX_BF16)
     return launch<bf16_t>(qkv, qkv_stride, k_cache, v_cache, block_tables, table_width, cu_q, kv_lens, out, part_o, part_lse, num_seqs,
-                          total_tokens, max_q_len, nh, nkv, page_shift, scale, window, splits, stream);
+                          total_tokens, max_q_len, max_kv_len, nh, nkv, page_shift, scale, window, splits, stream);
   return launch<float>(qkv, qkv_stride, k_cache, v_cache, block_tables, table_width, cu_q, kv_lens, out, part_o, part_lse, num_seqs,
-                       total_tokens, max_q_len, nh, nkv, page_shift, scale, window, splits, stream);
+                       total_tokens, max_q_len, max_kv_len, nh, nkv, page_shift, scale, window, splits, stream);
 }

@@ -87,7 +87,7 @@ class HipOps:
         lib = self._attention.get(head_dim)
         if lib is None:
             lib = ctypes.CDLL(build.ensure_attention(head_dim))
-            lib.velox_paged_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P]
+            lib.velox_paged_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P]
             lib.velox_paged_attention.restype = _I
             lib.velox_attention_head_dim.restype = _I
             if lib.velox_attention_head_dim() != head_dim:
@@ -424,7 +424,7 @@ class HipOps:
             part_lse = workspace.get("attention_partial_lse", splits * tokens * num_heads)
         status = lib.velox_paged_attention(
             _ptr(qkv), width, _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), block_tables.shape[1], _ptr(cu_q), _ptr(kv_lens),
-            _ptr(out), _ptr(part_o), _ptr(part_lse), num_seqs, tokens, max_q_len, num_heads, num_kv_heads,
+            _ptr(out), _ptr(part_o), _ptr(part_lse), num_seqs, tokens, max_q_len, int(max_kv_len), num_heads, num_kv_heads,
             block_size.bit_length() - 1, float(scale), int(window or 0), splits, _code(qkv.dtype), self._stream())
         self._launched(status, "paged_attention")
         return out
