@@ -141,6 +141,53 @@ def test_rope_kv_write(ops, ref, dtype, nh, nkv, d, half, page):
     assert not k_cache.any() and not v_cache.any()
 
 
+@pytest.mark.parametrize("m", [1, 5, 16])
+@pytest.mark.parametrize("nh,nkv,d,k,page", [(4, 2, 64, 128, 4), (28, 4, 128, 3584, 16), (3, 1, 32, 192, 1), (2, 2, 96, 64, 8), (5, 5, 160, 320, 32)])
+def test_qkv_projection_with_rotation_and_cache_write_in_one_kernel(ops, ref, m, nh, nkv, d, k, page):
+    """The fused decode kernel against product -> bias -> rotation -> cache write done one after the other in float32,
+    and against the unfused kernels; untouched cache entries stay untouched."""
+    pages = 24
+    width = (nh + 2 * nkv) * d
+    half = d // 2
+    x = rand((m, k), torch.bfloat16, 70)
+    w = rand((width, k), torch.bfloat16, 71, 0.05)
+    bias = rand((width,), torch.float32, 72, 0.3)
+    positions = torch.randint(0, 500, (m,), generator=torch.Generator().manual_seed(73)).to(torch.int32).cuda()
+    slots = (torch.randperm((pages - 1) * page, generator=torch.Generator().manual_seed(74))[:m] + page).to(torch.int32).cuda()
+    angles = torch.outer(torch.arange(512, dtype=torch.float32), 1.0 / (10000.0 ** (torch.arange(half, dtype=torch.float32) / half)))
+    cos, sin = angles.cos().cuda(), angles.sin().cuda()
+    ops.register_weight(w, rotary_heads=(nh, nkv, d))
+    assert ops.packed_weight(w, "rotary") is not None
+    for use_bias in (bias, None):
+        # float32 reference: exact product of the bfloat16 operands, then everything in float32
+        k32 = torch.full((pages, nkv, page, d), 7.0, dtype=torch.float32, device="cuda")
+        v32 = torch.full((pages, nkv, d, page), 7.0, dtype=torch.float32, device="cuda")
+        wide = ref.linear(x, w, None, torch.float32)
+        ref.rope_kv_write(wide, nh, nkv, d, positions, cos, sin, slots, k32, v32, page, write_kv=True, bias=use_bias)
+        results = {}
+        for fused in (True, False):
+            k_cache = torch.full((pages, nkv, page, d), 7.0, dtype=torch.bfloat16, device="cuda")
+            v_cache = torch.full((pages, nkv, d, page), 7.0, dtype=torch.bfloat16, device="cuda")
+            for waves in ((8, 16) if fused else (None,)):
+                q = ops.qkv_rope_write(x, w, use_bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, waves=waves, fused=fused)
+                results[(fused, waves)] = (q[:, : nh * d].float(), k_cache.float(), v_cache.float())
+        scale = float(wide.abs().max())
+        for key, (q, kc, vc) in results.items():
+            fused = key[0]
+            # the unfused route rounds the product to bfloat16 before the rotation: one more rounding
+            bound = dict(rtol=1e-2, atol=(1e-2 if fused else 2e-2) * scale)
+            torch.testing.assert_close(q, wide[:, : nh * d], msg=lambda t: f"{key} q: {t}", **bound)
+            torch.testing.assert_close(kc, k32, msg=lambda t: f"{key} k: {t}", **bound)
+            torch.testing.assert_close(vc, v32, msg=lambda t: f"{key} v: {t}", **bound)
+        torch.testing.assert_close(results[(True, 8)][0], results[(False, None)][0], rtol=2e-2, atol=2e-2 * scale)
+    # a layer that reads another layer's cache writes nothing: not a case for the fused kernel
+    with pytest.raises(Exception):
+        ops.qkv_rope_write(x, w, bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, write_kv=False, fused=True)
+    before = k_cache.clone()
+    ops.qkv_rope_write(x, w, bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, write_kv=False)
+    assert torch.equal(before, k_cache)
+
+
 def _attention_case(dtype, nh, nkv, d, page, seqs, seed, garbage=False):
     """seqs: list of (q_len, kv_len).  Builds a paged cache with shuffled pages and a flat qkv."""
     g = torch.Generator().manual_seed(seed)

@@ -61,8 +61,13 @@ class TorchOps:
     def prepare(self, model, dtype) -> None:
         pass
 
-    def register_weight(self, weight, stacked=1) -> None:
+    def register_weight(self, weight, stacked=1, rotary_heads=None) -> None:
         pass
+
+    def qkv_rope_write(self, x, weight, bias, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size, write_kv=True):
+        qkv = self.linear(x, weight, None, x.dtype)
+        self.rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size, write_kv=write_kv, bias=bias)
+        return qkv
 
     # -- embedding and norms ------------------------------------------------------------
     def embed(self, token_ids, table):

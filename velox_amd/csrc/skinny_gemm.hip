@@ -45,11 +45,12 @@ __device__ __forceinline__ Run16 zero_run() {
 // PACKED = true: W is stored tile by tile in the order the lanes read it, [row tile of 16][block of 64 indices][lane][16
 // elements] (rows padded with zeros to a multiple of 16; for GLU gate and up are padded separately), so that a wave's
 // load is one contiguous kilobyte.
-template <int RT, int CT, int WAVES, typename TO, bool GLU = false, bool PACKED = false>
-__global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
-                                                                 const float* __restrict__ bias, TO* __restrict__ out, int m, int n, int k) {
+// The products of one workgroup: every wave multiplies its share of K and leaves its sums in partial[wave]; after
+// the barrier at the end each tile's sum is partial[0][tile] + partial[1][tile] + ... (to be added in that order).
+template <int RT, int CT, int WAVES, bool GLU, bool PACKED>
+__device__ __forceinline__ void skinny_partial_sums(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, int m, int n, int k,
+                                                    float4_t (&partial)[WAVES][RT * CT][64]) {
   constexpr int UNROLL = 4;  // blocks of 64 indices whose loads are issued together
-  __shared__ float4_t partial[WAVES][RT * CT][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int g = lane >> 4, i = lane & 15;
   constexpr int RTO = GLU ? RT / 2 : RT;  // row tiles that become output columns
@@ -117,12 +118,21 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
         }
   }
 
-  // add the waves' partial sums in wave order; each tile's 64 lanes are then spread over the workgroup
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) partial[wave][rt * CT + ct][lane] = acc[rt][ct];
   __syncthreads();
+}
+
+template <int RT, int CT, int WAVES, typename TO, bool GLU = false, bool PACKED = false>
+__global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
+                                                                 const float* __restrict__ bias, TO* __restrict__ out, int m, int n, int k) {
+  __shared__ float4_t partial[WAVES][RT * CT][64];
+  constexpr int RTO = GLU ? RT / 2 : RT;
+  const int n0 = blockIdx.x * 16 * RTO;
+  skinny_partial_sums<RT, CT, WAVES, GLU, PACKED>(a, w, m, n, k, partial);
+  // add the waves' partial sums in wave order; each tile's 64 lanes are spread over the workgroup
   for (int item = threadIdx.x; item < RTO * CT * 64; item += WAVES * 64) {
     const int tile = item >> 6, l = item & 63;
     float4_t sum = partial[0][tile][l];
@@ -202,6 +212,113 @@ extern "C" int velox_skinny_gemm_bf16(const void* a, const void* w, const float*
   if (waves >= 8) PICK(2, 4, 8);
   PICK(2, 4, 4);
 #undef PICK
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The query/key/value projection of a decode step with everything that follows it before attention: bias, rotation
+// and the write into the paged cache are the epilogue of the product, so the [M, (heads + 2 kv_heads) d] result never
+// goes to memory and one launch is saved.  W is packed (see above) with its rows reordered so that a workgroup's two
+// row tiles are what one rotation needs: for a query or key head the 16 channels c0 .. c0 + 15 of the low half and
+// their partners c0 + d/2 ..; for a value head two consecutive tiles.  Needs d % 32 == 0 and a rotation of the
+// whole head (tables of d / 2 angles per position).
+// ---------------------------------------------------------------------------------------------------------------
+struct RotaryWrite {
+  const float* bias;       // [(heads + 2 kv_heads) * d] in the original row order, or null
+  const int* positions;    // [M]
+  const float* cos_table;  // [positions, d / 2]
+  const float* sin_table;
+  const int* slots;        // [M]: page * page_size + offset of the token's key
+  bf16_t* q_out;           // [M, heads * d]
+  bf16_t* k_cache;         // [pages, kv_heads, page_size, d]
+  bf16_t* v_cache;         // [pages, kv_heads, d, page_size]
+  int heads, kv_heads, d, page_size;
+};
+
+template <int WAVES>
+__global__ void __launch_bounds__(WAVES * 64) skinny_qkv_rotary_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
+                                                                       RotaryWrite args, int m, int n, int k) {
+  __shared__ float4_t partial[WAVES][2][64];
+  skinny_partial_sums<2, 1, WAVES, false, true>(a, w, m, n, k, partial);
+  const int l = threadIdx.x;
+  if (l >= 64) return;
+  const int row = l & 15;  // batch row
+  if (row >= m) return;
+  float4_t first = partial[0][0][l], second = partial[0][1][l];
+#pragma unroll
+  for (int wv = 1; wv < WAVES; ++wv) {
+    first += partial[wv][0][l];
+    second += partial[wv][1][l];
+  }
+  const int d = args.d, half = d / 2;
+  const int pairs_per_head = d / 32;
+  const int head = blockIdx.x / pairs_per_head, j = blockIdx.x % pairs_per_head;
+  const int r4 = 4 * (l >> 4);
+  const int slot = args.slots[row];
+  const size_t page = (size_t)(slot / args.page_size);
+  const int offset = slot % args.page_size;
+  if (head < args.heads + args.kv_heads) {
+    const int c = 16 * j + r4;  // channels c .. c + 3 of the low half and their partners
+    if (args.bias) {
+      const float* b = args.bias + (size_t)head * d + c;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        first[e] += b[e];
+        second[e] += b[half + e];
+      }
+    }
+    const size_t angle = (size_t)args.positions[row] * half + c;
+    const float4_t cs = *reinterpret_cast<const float4_t*>(args.cos_table + angle);
+    const float4_t sn = *reinterpret_cast<const float4_t*>(args.sin_table + angle);
+    __attribute__((aligned(8))) bf16_t lo[4];
+    __attribute__((aligned(8))) bf16_t hi[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      lo[e] = from_f32<bf16_t>(first[e] * cs[e] - second[e] * sn[e]);
+      hi[e] = from_f32<bf16_t>(first[e] * sn[e] + second[e] * cs[e]);
+    }
+    bf16_t* dst = head < args.heads
+                      ? args.q_out + ((size_t)row * args.heads + head) * d + c
+                      : args.k_cache + (((page * args.kv_heads + (head - args.heads)) * args.page_size) + offset) * d + c;
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    *reinterpret_cast<float2_t*>(dst) = *reinterpret_cast<const float2_t*>(lo);
+    *reinterpret_cast<float2_t*>(dst + half) = *reinterpret_cast<const float2_t*>(hi);
+  } else {
+    const int vh = head - args.heads - args.kv_heads;
+    const int c = 32 * j + r4;  // channels c .. c + 3 and c + 16 .. c + 19
+    if (args.bias) {
+      const float* b = args.bias + (size_t)head * d + c;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        first[e] += b[e];
+        second[e] += b[16 + e];
+      }
+    }
+    bf16_t* dst = args.v_cache + ((page * args.kv_heads + vh) * d + c) * args.page_size + offset;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      dst[(size_t)e * args.page_size] = from_f32<bf16_t>(first[e]);
+      dst[(size_t)(16 + e) * args.page_size] = from_f32<bf16_t>(second[e]);
+    }
+  }
+}
+
+// a [M, K] (M <= 16), w: packed rows of [Wq; Wk; Wv] in the rotary order; q_out [M, heads * d]; keys and values go to
+// the cache at slots[M].  waves: 8 or 16.
+extern "C" int velox_skinny_qkv_rotary_bf16(const void* a, const void* w, const float* bias, const int* positions,
+                                            const float* cos_table, const float* sin_table, const int* slots, void* q_out,
+                                            void* k_cache, void* v_cache, int m, int k, int heads, int kv_heads, int d,
+                                            int page_size, int waves, hipStream_t stream) {
+  if (m <= 0) return 0;
+  if (m > 16 || k % 64 != 0 || d % 32 != 0 || heads < 1 || kv_heads < 1 || page_size < 1) return -1;
+  RotaryWrite args{bias, positions, cos_table, sin_table, slots, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
+                   heads, kv_heads, d, page_size};
+  const int n = (heads + 2 * kv_heads) * d;
+  const int blocks = n / 32;
+  if (waves >= 16)
+    skinny_qkv_rotary_kernel<16><<<blocks, 16 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, args, m, n, k);
+  else
+    skinny_qkv_rotary_kernel<8><<<blocks, 8 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, args, m, n, k);
+  return (int)hipGetLastError();
 }
 
 // out[M, n] = silu(A Wgate^T) * (A Wup^T) with W = [Wgate; Wup] of 2n rows, bfloat16 in and out, M <= 32.

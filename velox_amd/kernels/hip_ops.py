@@ -15,7 +15,7 @@ from __future__ import annotations
 import ctypes
 import os
 import tempfile
-from typing import Dict, Optional
+from typing import Tuple, Dict, Optional
 
 import torch
 
@@ -67,6 +67,7 @@ class HipOps:
         c = self._core
         c.velox_embed.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
         c.velox_add_rmsnorm.argtypes = [_P, _P, _P, _P, _P, _I, _I, _F, _I, _I, _I, ctypes.c_longlong, _P]
+        c.velox_skinny_qkv_rotary_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_silu_mul.argtypes = [_P, _P, _I, _I, _I, _P]
         c.velox_rope_kv_write.argtypes = [_P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_gemm_fma.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
@@ -104,11 +105,13 @@ class HipOps:
         for part in model.all_parts():
             part.prepare_kernels(self)
 
-    def register_weight(self, weight: torch.Tensor, stacked: int = 1) -> None:
+    def register_weight(self, weight: torch.Tensor, stacked: int = 1, rotary_heads: Optional[Tuple[int, int, int]] = None) -> None:
         """Keeps a second copy of a bfloat16 ``[N, K]`` weight in the order the skinny kernels' lanes read it (see
-        ``pack_rows``): decode-sized products then stream contiguous kilobytes.  ``stacked`` = 2 marks ``[Wgate; Wup]``.
-        Costs the weight's size again in memory; ``pack_decode_weights = False`` turns it off.  The copy hangs on the
-        tensor object itself, so it lives exactly as long as the weight and is found only through that object."""
+        ``pack_rows``): decode-sized products then stream contiguous kilobytes.  ``stacked`` = 2 marks ``[Wgate; Wup]``;
+        ``rotary_heads = (heads, kv_heads, head_dim)`` marks ``[Wq; Wk; Wv]`` whose product is followed by a rotation of
+        whole heads and gets a further copy for ``qkv_rope_write``.  Each copy costs the weight's size again in memory;
+        ``pack_decode_weights = False`` turns them off.  The copies hang on the tensor object itself, so they live
+        exactly as long as the weight and are found only through that object."""
         if (not self.pack_decode_weights or weight is None or weight.dtype != torch.bfloat16 or weight.dim() != 2
                 or weight.shape[1] % 64 != 0 or weight.shape[0] % stacked != 0 or weight.device != self.device):
             return
@@ -116,15 +119,28 @@ class HipOps:
         if copies is None or copies["version"] != weight._version:
             copies = {"version": weight._version}
             weight._velox_packed = copies
-        if stacked in copies:
-            return
-        per_matrix = weight.shape[0] // stacked
-        whole_tiles = [c for key, c in copies.items() if key != "version"] if per_matrix % 16 == 0 else []
-        # with whole tiles every stacking gives the same bytes
-        copies[stacked] = whole_tiles[0] if whole_tiles else self.pack_rows(weight, stacked)
+        if stacked not in copies:
+            per_matrix = weight.shape[0] // stacked
+            whole_tiles = [c for key, c in copies.items() if key in (1, 2)] if per_matrix % 16 == 0 else []
+            # with whole tiles every stacking gives the same bytes
+            copies[stacked] = whole_tiles[0] if whole_tiles else self.pack_rows(weight, stacked)
+        if rotary_heads is not None and "rotary" not in copies:
+            heads, kv_heads, head_dim = rotary_heads
+            if head_dim % 32 == 0 and weight.shape[0] == (heads + 2 * kv_heads) * head_dim:
+                copies["rotary"] = self.pack_rows(weight[self.rotary_row_order(heads, kv_heads, head_dim, weight.device)])
 
     @staticmethod
-    def packed_weight(weight: torch.Tensor, stacked: int = 1) -> Optional[torch.Tensor]:
+    def rotary_row_order(heads: int, kv_heads: int, head_dim: int, device) -> torch.Tensor:
+        """Row order of ``[Wq; Wk; Wv]`` for ``qkv_rope_write``: inside every query and key head, 16 channels of the low
+        half are followed by their 16 partners of the high half; value heads keep their order."""
+        half = head_dim // 2
+        inside = torch.arange(half, device=device).view(half // 16, 1, 16) + torch.tensor([0, half], device=device).view(1, 2, 1)
+        rotary = (torch.arange(heads + kv_heads, device=device).view(-1, 1) * head_dim + inside.reshape(1, -1)).reshape(-1)
+        values = torch.arange((heads + kv_heads) * head_dim, (heads + 2 * kv_heads) * head_dim, device=device)
+        return torch.cat([rotary, values])
+
+    @staticmethod
+    def packed_weight(weight: torch.Tensor, stacked=1) -> Optional[torch.Tensor]:
         copies = getattr(weight, "_velox_packed", None)
         if copies is None or copies["version"] != weight._version:
             return None
@@ -373,6 +389,45 @@ class HipOps:
             tokens, num_heads, num_kv_heads, head_dim, block_size, 1 if write_kv else 0, _code(qkv.dtype), self._stream())
         self._launched(status, "rope_kv_write")
 
+    def qkv_rope_write(self, x, weight, bias, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache,
+                       block_size, write_kv=True, waves: Optional[int] = None, fused: Optional[bool] = None) -> torch.Tensor:
+        """Projects ``x`` with ``weight = [Wq; Wk; Wv]``, adds ``bias``, rotates queries and keys and writes keys and values
+        into the cache.  Returns a tensor whose first ``num_heads * head_dim`` columns are the rotated queries (it may be
+        wider).  Decode-sized bfloat16 batches run as one kernel when ``register_weight(weight, rotary_heads=...)`` has
+        prepared the weight; everything else is the product followed by ``rope_kv_write``."""
+        m, k = x.shape
+        packed = self.packed_weight(weight, "rotary")
+        can_fuse = (self.use_skinny_gemm and packed is not None and write_kv and x.dtype == torch.bfloat16 and m <= 16 and k % 64 == 0
+                    and cos is not None and 2 * cos.shape[1] == head_dim and head_dim % 32 == 0 and k_cache.dtype == torch.bfloat16)
+        if fused is None:
+            fused = can_fuse
+        elif fused and not can_fuse:
+            raise KernelError("qkv_rope_write: this call cannot run fused")
+        if not fused:
+            qkv = self.linear(x, weight, None, x.dtype)
+            self.rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size,
+                               write_kv=write_kv, bias=bias)
+            return qkv
+        width = (num_heads + 2 * num_kv_heads) * head_dim
+        self._check("x", x, torch.bfloat16, align=16)
+        if weight.shape != (width, k):
+            raise KernelError(f"qkv_rope_write: weight {tuple(weight.shape)} is not [{width}, {k}]")
+        self._check("positions", positions, torch.int32, (m,))
+        self._check("slot_mapping", slot_mapping, torch.int32, (m,))
+        if bias is not None:
+            self._check("bias", bias, torch.float32, (width,))
+        self._check("cos", cos, torch.float32, align=16)
+        self._check("sin", sin, torch.float32, tuple(cos.shape), align=16)
+        pages = k_cache.shape[0]
+        self._check("k_cache", k_cache, torch.bfloat16, (pages, num_kv_heads, block_size, head_dim), align=16)
+        self._check("v_cache", v_cache, torch.bfloat16, (pages, num_kv_heads, head_dim, block_size), align=16)
+        q = torch.empty((m, num_heads * head_dim), dtype=torch.bfloat16, device=self.device)
+        status = self._core.velox_skinny_qkv_rotary_bf16(
+            _ptr(x), _ptr(packed), _ptr(bias), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping), _ptr(q), _ptr(k_cache),
+            _ptr(v_cache), m, k, num_heads, num_kv_heads, head_dim, block_size, int(waves or 8), self._stream())
+        self._launched(status, "skinny_qkv_rotary")
+        return q
+
     # -- attention ------------------------------------------------------------------------------
     def choose_splits(self, num_seqs: int, num_kv_heads: int, row_tiles: int, max_kv_len: int, all_decode: bool) -> int:
         """Splits of the key range for an all-decode step (reference ``src/decode_attention.py:237-252``:
@@ -389,7 +444,9 @@ class HipOps:
     def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens,
                         max_q_len, max_kv_len, scale, window, all_decode, workspace, splits: Optional[int] = None):
         tokens = qkv.shape[0]
-        width = (num_heads + 2 * num_kv_heads) * head_dim
+        width = qkv.shape[1] if qkv.dim() == 2 else -1  # rows may carry keys and values after the queries
+        if width not in (num_heads * head_dim, (num_heads + 2 * num_kv_heads) * head_dim):
+            raise KernelError(f"paged_attention: rows of {width} elements hold neither the queries nor queries, keys and values")
         self._check("qkv", qkv, None, (tokens, width), align=16)
         num_seqs = kv_lens.shape[0]
         self._check("kv_lens", kv_lens, torch.int32, (num_seqs,))

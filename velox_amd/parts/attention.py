@@ -71,26 +71,30 @@ class AttentionMixer(Mixer):
     def cache_need(self):
         return PagedNeed(self.num_kv_heads, self.head_dim, self.window)
 
+    def _rotary_tables(self):
+        tables = self.position.rotary_tables() if self.position is not None else None
+        return tables if tables is not None else (None, None)
+
     def prepare_kernels(self, ops) -> None:
-        ops.register_weight(self.qkv_weight)
+        cos, _ = self._rotary_tables()
+        whole_heads = cos is not None and 2 * cos.shape[1] == self.head_dim
+        ops.register_weight(self.qkv_weight, rotary_heads=(self.num_heads, self.num_kv_heads, self.head_dim) if whole_heads else None)
         ops.register_weight(self.o_weight)
 
     def forward(self, x, ctx, cache, owns_cache: bool = True):
         ops = ctx.ops
-        # the bias is added (in float32) by the kernel that rotates and stores, which reads qkv anyway
-        qkv = ops.linear(x, self.qkv_weight, None, ctx.dtype)
-        tables = self.position.rotary_tables() if self.position is not None else None
-        cos, sin = tables if tables is not None else (None, None)
+        cos, sin = self._rotary_tables()
         meta = cache.batch
-        ops.rope_kv_write(
-            qkv, self.num_heads, self.num_kv_heads, self.head_dim,
+        # product, bias (added in float32), rotation and the write into the cache: one kernel for decode-sized batches
+        q = ops.qkv_rope_write(
+            x, self.qkv_weight, self.qkv_bias_vec if self.qkv_bias else None,
+            self.num_heads, self.num_kv_heads, self.head_dim,
             ctx.positions, cos, sin,
             meta.slot_mapping, cache.k, cache.v, cache.block_size,
             write_kv=owns_cache,
-            bias=self.qkv_bias_vec if self.qkv_bias else None,
         )
         attn = ops.paged_attention(
-            qkv, self.num_heads, self.num_kv_heads, self.head_dim,
+            q, self.num_heads, self.num_kv_heads, self.head_dim,
             cache.k, cache.v, cache.block_size,
             meta.block_tables, ctx.cu_q, meta.kv_lens,
             ctx.max_q_len, meta.max_kv_len, self.scale, self.window,
