@@ -25,6 +25,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from ..parts.base import PagedNeed, StateNeed
@@ -38,6 +39,17 @@ class SequenceCache:
     slot: int
     tables: List[List[int]]
     released: List[int]  # per group: number of leading table entries already given back
+    version: int = 0  # counts the changes of ``tables``: whoever changes a table in place adds one
+
+    def table_arrays(self) -> List[np.ndarray]:
+        """The block tables as int32 arrays, converted again only after a change (see ``version``)."""
+        if self._arrays_version != self.version or self._arrays is None:
+            self._arrays = [np.asarray(table, dtype=np.int32) for table in self.tables]
+            self._arrays_version = self.version
+        return self._arrays
+
+    _arrays: Optional[List[np.ndarray]] = field(default=None, repr=False, compare=False)
+    _arrays_version: int = field(default=-1, repr=False, compare=False)
 
 
 class PageGroup:
@@ -221,7 +233,9 @@ class CacheManager:
             if n > group.allocator.num_free or len(table) + n > self.max_pages_per_seq:
                 return False
         for n, group, table in zip(extra, self.groups, seq.tables):
-            table.extend(group.allocator.allocate_many(n))
+            if n:
+                table.extend(group.allocator.allocate_many(n))
+                seq.version += 1
         return True
 
     def release_behind_window(self, seq: SequenceCache, num_computed: int) -> int:
@@ -234,6 +248,7 @@ class CacheManager:
                 if table[position] != NULL_PAGE:
                     group.allocator.free(table[position])
                     table[position] = NULL_PAGE
+                    seq.version += 1
                     given_back += 1
             seq.released[index] = max(seq.released[index], first)
         return given_back
@@ -245,6 +260,7 @@ class CacheManager:
                     group.allocator.free(page)
             seq.tables[index] = []
             seq.released[index] = 0
+        seq.version += 1
 
     def free_sequence(self, seq: SequenceCache) -> None:
         self.free_pages(seq)

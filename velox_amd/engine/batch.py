@@ -122,14 +122,18 @@ class BatchBuilder:
         slots = np.full(b, cache.state.pad_slot, dtype=np.int32)
         rows: List[int] = []
         for i, e in enumerate(entries):
-            lo, hi = cu[i], cu[i + 1]
-            ids[lo:hi] = np.asarray(e.token_ids, dtype=np.int32)
-            positions[lo:hi] = np.arange(e.start, e.start + q_lens[i], dtype=np.int32)
+            lo, n = int(cu[i]), q_lens[i]
+            if n == 1:  # a decoded token: plain integers are quicker than arrays of one
+                ids[lo] = e.token_ids[0]
+                positions[lo] = e.start
+            else:
+                ids[lo:lo + n] = np.asarray(e.token_ids, dtype=np.int32)
+                positions[lo:lo + n] = np.arange(e.start, e.start + n, dtype=np.int32)
             slots[i] = e.seq.slot
             for w in e.want:
-                if not 0 <= w < q_lens[i]:
-                    raise ValueError(f"want index {w} outside the entry's {q_lens[i]} tokens")
-                rows.append(int(lo) + int(w))
+                if not 0 <= w < n:
+                    raise ValueError(f"want index {w} outside the entry's {n} tokens")
+                rows.append(lo + int(w))
         if pad_to is not None:
             rows.extend(range(int(cu[b_real]), t))  # padded rows ask for their own logits: fixed layout
         r = len(rows)
@@ -170,14 +174,18 @@ class BatchBuilder:
             slot_map = np.zeros(t, dtype=np.int32)
             tables = np.zeros((b, width), dtype=np.int32)
             for i, e in enumerate(entries):
-                table = np.asarray(e.seq.tables[g], dtype=np.int64)
-                end = e.start + q_lens[i]
+                table = e.seq.table_arrays()[g]
+                n = q_lens[i]
+                end = e.start + n
                 if len(table) * page < end:
                     raise ValueError(f"entry {i}: its block table covers {len(table) * page} tokens but the step reaches {end}")
                 tables[i, : len(table)] = table
                 kv[i] = end
-                pos = np.arange(e.start, end, dtype=np.int64)
-                slot_map[cu[i]:cu[i + 1]] = table[pos // page] * page + pos % page
+                if n == 1:
+                    slot_map[cu[i]] = int(table[e.start // page]) * page + e.start % page
+                else:
+                    pos = np.arange(e.start, end, dtype=np.int64)
+                    slot_map[cu[i]:cu[i + 1]] = table[pos // page].astype(np.int64) * page + pos % page
             put(f"kv{g}", kv, b)
             put(f"slot{g}", slot_map, t)
             put(f"bt{g}", tables, b * width)

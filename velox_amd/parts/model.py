@@ -159,17 +159,28 @@ class DecoderModel(Part):
         return needs
 
     # -- arithmetic ---------------------------------------------------------------------
-    def forward(self, token_ids: torch.Tensor, ctx):
-        """Runs every block; returns ``(residual float32 [T, H], pending [T, H])``."""
+    def embed(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
+        """The residual stream before the first block: float32 ``[T, H]``."""
         residual = self.embedding.forward(token_ids, ctx)
         if self.spec.embedding_position is not None:
             residual = self.positions[self.spec.embedding_position].on_embeddings(residual, ctx)
-        pending = None
-        for index, entry in enumerate(self.schedule):
+        return residual
+
+    def run_schedule(self, residual: torch.Tensor, pending, ctx, first: int = 0, last: Optional[int] = None):
+        """Runs schedule entries ``first .. last - 1`` on ``residual`` (updated in place); takes and returns ``pending``,
+        the sub-layer output that the next norm still has to add."""
+        last = len(self.schedule) if last is None else last
+        for index in range(first, last):
+            entry = self.schedule[index]
             owner = index if entry.cache_from is None else entry.cache_from
             cache = ctx.cache_view(owner)
             pending = self.blocks[entry.layer].forward(residual, pending, ctx, cache, entry.cache_from is None)
-        return residual, pending
+        return pending
+
+    def forward(self, token_ids: torch.Tensor, ctx):
+        """Runs every block; returns ``(residual float32 [T, H], pending [T, H])``."""
+        residual = self.embed(token_ids, ctx)
+        return residual, self.run_schedule(residual, None, ctx)
 
     def logits(self, residual: torch.Tensor, pending, rows: torch.Tensor, ctx) -> torch.Tensor:
         """Final norm and output head on ``rows`` (int32 [R]) only: float32 [R, vocab]."""
