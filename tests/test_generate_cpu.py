@@ -96,3 +96,58 @@ def test_seeded_sampling_is_independent_of_the_batch(tmp_path):
     mixed = engine.generate([sampled(7, prompts[0]), greedy([prompts[1]], 6, prefix="g-mixed")[0], sampled(8, prompts[3])])
     assert mixed[1].output_token_ids == greedy_alone.output_token_ids
     assert len({tuple(r.output_token_ids) for r in together}) > 1
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_launching_the_next_step_early_changes_no_token(tmp_path, name):
+    """decode_lookahead launches a decode step before the tokens of the step before it have been read: same tokens,
+    same finish reasons, also when a request stops on a token that was still in flight, and every page comes back."""
+    folder = make_folder(tmp_path, name)
+    config, weights = read_model_folder(folder)
+    prompts = [random_tokens(config["vocab_size"], n, seed=90 + n) for n in (4, 11, 19)]
+    expected = [plain_greedy(config, weights, p, 10) for p in prompts]
+    stop_at = expected[1][4]  # request 1 stops in the middle of the others' decoding
+
+    def requests(prefix):
+        out = greedy(prompts, 10, prefix=prefix)
+        out[1] = Request(f"{prefix}stop", prompts[1], SamplingParams(temperature=0.0, max_tokens=10, stop_token_ids=[stop_at]))
+        out[2] = Request(f"{prefix}short", prompts[2], SamplingParams(temperature=0.0, max_tokens=3, ignore_eos=True))
+        return out
+
+    results = {}
+    for lookahead in (True, False):
+        engine = engine_for(folder, name, decode_lookahead=lookahead)
+        launches = []
+        inner = engine.runner.step
+        engine.runner.step = lambda entries, ids_on_device=None: (launches.append(ids_on_device is not None), inner(entries, ids_on_device=ids_on_device))[1]
+        done = engine.generate(requests("on-" if lookahead else "off-"))
+        results[lookahead] = [(r.output_token_ids, r.finish_reason) for r in done]
+        assert any(launches) == lookahead
+        assert engine.cache.num_used_pages() == 0
+        engine.cache.assert_consistent([])
+        assert engine._ahead is None or not any(engine._alive(r) for r in engine._ahead.sampled)
+    assert results[True] == results[False]
+    cut = expected[1].index(stop_at) + 1
+    assert results[True][0] == (expected[0], FinishReason.LENGTH)
+    assert results[True][1] == (expected[1][:cut], FinishReason.STOP)
+    assert results[True][2] == (expected[2][:3], FinishReason.LENGTH)
+
+
+def test_abort_while_a_step_is_in_flight(tmp_path):
+    folder = make_folder(tmp_path, "A")
+    config, weights = read_model_folder(folder)
+    prompts = [random_tokens(config["vocab_size"], n, seed=95 + n) for n in (6, 9)]
+    engine = engine_for(folder, "A")
+    keep, drop = greedy(prompts, 12)
+    engine.add_request(keep)
+    engine.add_request(drop)
+    while len(keep.output_token_ids) < 4:
+        engine.step()
+    assert engine._ahead is not None  # a decode step is in flight
+    engine.abort_request(drop.request_id)
+    while engine.has_work():
+        engine.step()
+    assert keep.output_token_ids == plain_greedy(config, weights, prompts[0], 12)
+    assert drop.finish_reason is FinishReason.ABORT and len(drop.output_token_ids) < 12
+    assert engine.cache.num_used_pages() == 0
+    engine.cache.assert_consistent([])

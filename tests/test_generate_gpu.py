@@ -71,6 +71,43 @@ def test_graph_decode_equals_eager_decode_and_preemption_keeps_tokens(tmp_path):
     assert tight_engine.cache.num_used_pages() == 0
 
 
+@pytest.mark.parametrize("graphs", [False, True])
+def test_launching_the_next_step_early_changes_no_token(tmp_path, graphs):
+    """decode_lookahead on the GPU, eager and through graphs: the next decode step is queued, with its token ids taken
+    on the device from the sampler's output, before the host reads the tokens.  Same tokens and finish reasons as with
+    one step at a time, also for a request that stops on a token that was still in flight."""
+    folder = make_folder(tmp_path, "B", "float32")
+    config, weights = read_model_folder(folder)
+    prompts = [random_tokens(config["vocab_size"], n, seed=60 + n) for n in (7, 15, 22, 3)]
+    expected = [plain_greedy(config, weights, p, 14) for p in prompts]
+    stop_at = expected[1][5]
+
+    def requests(prefix):
+        out = greedy(prompts, 14, prefix=prefix)
+        out[1] = Request(f"{prefix}stop", prompts[1], SamplingParams(temperature=0.0, max_tokens=14, stop_token_ids=[stop_at]))
+        out[2] = Request(f"{prefix}short", prompts[2], SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))
+        out[3] = Request(f"{prefix}drawn", prompts[3], SamplingParams(temperature=0.9, max_tokens=14, seed=5, ignore_eos=True))
+        return out
+
+    results = {}
+    for lookahead in (True, False):
+        engine = engine_for(folder, "B", "float32", enable_cuda_graphs=graphs, decode_lookahead=lookahead)
+        launches = []
+        inner = engine.runner.step
+        engine.runner.step = lambda entries, ids_on_device=None: (launches.append(ids_on_device is not None), inner(entries, ids_on_device=ids_on_device))[1]
+        done = engine.generate(requests("on-" if lookahead else "off-"))
+        results[lookahead] = [(r.output_token_ids, r.finish_reason) for r in done]
+        assert any(launches) == lookahead
+        assert engine.cache.num_used_pages() == 0
+        engine.cache.assert_consistent([])
+    assert results[True] == results[False]
+    cut = expected[1].index(stop_at) + 1
+    assert results[True][0][0] == expected[0]
+    assert results[True][1][0] == expected[1][:cut]
+    assert results[True][2][0] == expected[2][:4]
+    assert len(results[True][3][0]) == 14
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_graph_replay_gives_the_eager_logits(tmp_path, name, dtype):

@@ -217,3 +217,63 @@ def test_a_victim_leaves_the_step_it_was_already_given_a_token_in():
     while s.has_work():
         run_step(s, s.schedule())
     assert len(a.output_token_ids) == 2 and len(b.output_token_ids) == 9
+
+
+def decoding(s, lengths, max_tokens=8):
+    """Requests read in whole and given their first token: all decoding."""
+    requests = [request(f"d{i}", n, max_tokens) for i, n in enumerate(lengths)]
+    for r in requests:
+        s.add_request(r)
+    while any(r.status is not RequestStatus.RUNNING_DECODE for r in requests):
+        run_step(s, s.schedule())
+    return requests
+
+
+def test_the_next_decode_step_can_be_fixed_while_one_is_in_flight():
+    s = make(pages=33, page=4, budget=16)
+    requests = decoding(s, [3, 4, 7])
+    out = s.schedule()  # a decode-only step: "in flight" until run_step books it
+    assert out.decode_batch == requests and not out.prefill_batch
+    pages_before = [len(r.cache.tables[0]) for r in requests]
+    ahead = s.schedule_ahead(out.decode_batch)
+    assert ahead == requests
+    # every table now covers the position after the one in flight
+    for r, before in zip(requests, pages_before):
+        assert len(r.cache.tables[0]) * 4 >= r.num_computed_tokens + 2 and len(r.cache.tables[0]) - before in (0, 1)
+    run_step(s, out)
+    # the step fixed ahead runs next, without schedule(): its pages are there
+    for r in ahead:
+        assert len(r.cache.tables[0]) * 4 >= r.num_computed_tokens + 1
+        s.advance(r, 1)
+        r.append_token(7)
+    s.cache.assert_consistent([r.cache for r in requests])
+
+
+def test_nothing_is_fixed_ahead_when_the_next_step_could_look_different():
+    # somebody waits
+    s = make(pages=33, page=4, seqs=2, budget=16)
+    requests = decoding(s, [3, 4])
+    s.add_request(request("late", 5))
+    out = s.schedule()  # both slots are taken: the late request waits
+    assert not out.prefill_batch and len(s.waiting) == 1
+    assert s.schedule_ahead(out.decode_batch) is None
+    # a request reaches its length limit with the token in flight
+    s = make(pages=33, page=4, budget=16)
+    requests = decoding(s, [3, 4], max_tokens=2)  # one token each so far
+    out = s.schedule()
+    assert s.schedule_ahead(out.decode_batch) is None
+    # not every running request is in the step
+    s = make(pages=33, page=4, budget=16)
+    requests = decoding(s, [3, 4, 5])
+    out = s.schedule()
+    assert s.schedule_ahead(out.decode_batch[:2]) is None
+    # pages are short: both requests sit at the end of a page and one page is free; nothing may be taken
+    s = make(pages=4, page=4, budget=16, watermark=0.01)  # 3 usable pages
+    requests = decoding(s, [3, 3])  # 4 tokens each after the first sampled one: position 4 needs a second page
+    out = s.schedule()
+    assert len(out.decode_batch) == 2
+    if True:
+        free_before = s.cache.groups[0].allocator.num_free
+        tables = [list(r.cache.tables[0]) for r in requests]
+        assert s.schedule_ahead(out.decode_batch) is None
+        assert s.cache.groups[0].allocator.num_free == free_before and [list(r.cache.tables[0]) for r in requests] == tables

@@ -56,6 +56,8 @@ class EngineConfig:
     # a second copy of every bfloat16 weight in the order the decode kernels read it: faster decoding for the
     # weights' size again in memory (not a reference option)
     pack_decode_weights: bool = True
+    # launch a decode step's successor before reading the step's tokens (not a reference option)
+    decode_lookahead: bool = True
     watermark: float = 0.01
 
     seed: Optional[int] = None

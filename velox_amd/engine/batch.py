@@ -97,12 +97,17 @@ class BatchBuilder:
 
     def section_total(self, t: int, b: int, r: int, w: int) -> int:
         n_groups = len(self.cache.groups)
-        return _align(t) * 2 + _align(b + 1) + _align(b) + _align(r) + n_groups * (_align(b) + _align(t) + _align(b * w))
+        return _align(t) * 2 + _align(b + 1) + _align(b) * 2 + _align(r) + n_groups * (_align(b) + _align(t) + _align(b * w))
 
-    def build(self, entries: Sequence[StepEntry], ops, dtype, workspace: Workspace, device_buffer: Optional[torch.Tensor] = None, pad_to: Optional[int] = None, width: Optional[int] = None) -> StepContext:
+    def build(self, entries: Sequence[StepEntry], ops, dtype, workspace: Workspace, device_buffer: Optional[torch.Tensor] = None, pad_to: Optional[int] = None, width: Optional[int] = None,
+              ids_on_device: Optional[tuple] = None) -> StepContext:
         """Lays the step out.  ``pad_to``/``width``/``device_buffer`` are for captured decode steps:
         the batch is padded to ``pad_to`` one-token rows that read and write the null page, the
-        block table has the fixed ``width``, and the sections land in the caller's buffer."""
+        block table has the fixed ``width``, and the sections land in the caller's buffer.
+
+        ``ids_on_device = (tokens int32 [R] on the device, rows)``: every entry has one token and entry ``i``'s is
+        ``tokens[rows[i]]``, which the host may not know yet; it is copied into place on the device, after the
+        staging copy, in stream order."""
         cache = self.cache
         page = cache.page_size
         b_real = len(entries)
@@ -168,6 +173,12 @@ class BatchBuilder:
         put("cu", cu, b + 1)
         put("slots", slots, b)
         put("rows", np.asarray(rows, dtype=np.int32), r)
+        source = np.zeros(b, dtype=np.int32)  # always laid out: a captured step reads its sections at fixed places
+        if ids_on_device is not None:
+            if t != b or len(ids_on_device[1]) != b_real:
+                raise ValueError("token ids on the device need one token per entry and one source row per entry")
+            source[:b_real] = np.asarray(ids_on_device[1], dtype=np.int32)
+        put("source", source, b)
         max_kv: List[int] = []
         for g, group in enumerate(cache.groups):
             kv = np.ones(b, dtype=np.int32)
@@ -199,6 +210,12 @@ class BatchBuilder:
         def view(name: str) -> torch.Tensor:
             lo, n = sections[name]
             return device[lo:lo + n]
+
+        if ids_on_device is not None:
+            tokens = ids_on_device[0]
+            if tokens.dtype != torch.int32 or tokens.dim() != 1 or int(max(ids_on_device[1])) >= tokens.shape[0] or min(ids_on_device[1]) < 0:
+                raise ValueError("token ids on the device must be int32 [R] and every source row inside it")
+            torch.index_select(tokens, 0, view("source")[:b_real], out=view("ids")[:b_real])
 
         groups = [
             GroupBatch(

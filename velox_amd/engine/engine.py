@@ -11,6 +11,7 @@ step function.  The one host wait per step is the read of the sampled tokens
 from __future__ import annotations
 
 import time
+from dataclasses import dataclass
 from typing import Dict, FrozenSet, Iterable, List, Optional, Sequence
 
 import torch
@@ -27,6 +28,17 @@ from .batch import StepEntry
 from .request import FinishReason, Request
 from .runner import ModelRunner
 from .scheduler import Scheduler, SchedulerConfig
+
+@dataclass
+class _Flight:
+    """A step that has been queued on the device."""
+
+    decode: List[Request]
+    prefill: List[Request]
+    sampled: List[Request]  # the requests whose rows were sampled, in row order
+    tokens: Optional[torch.Tensor]  # int32 [len(sampled)] on the device
+    landing: Optional[tuple] = None  # (pinned host tensor the tokens are copied to, event recorded behind the copy)
+
 
 _STAGES = ("scheduler_ms", "prepare_ms", "forward_ms", "sampling_ms", "cpu_sync_wait_ms", "step_ms")
 
@@ -66,6 +78,12 @@ class Engine:
         self.sampler = Sampler(ops, self.device, seed=config.seed)
         self.stats: Dict[str, List[float]] = {name: [] for name in _STAGES}
         self.num_steps = 0
+        self._ahead: Optional[_Flight] = None
+        self._landings = []
+        self._next_landing = 0
+        if self.device.type == "cuda":
+            rows = max(config.max_num_seqs, 1)
+            self._landings = [(torch.zeros(rows, dtype=torch.int32, pin_memory=True), torch.cuda.Event()) for _ in range(3)]
 
     # -- construction -------------------------------------------------------------------
     @classmethod
@@ -155,20 +173,50 @@ class Engine:
     # -- one step -----------------------------------------------------------------------
     @torch.no_grad()
     def step(self) -> None:
+        """One step of every scheduled request.  When it returns, each of them holds its new token.  With
+        ``decode_lookahead`` the NEXT step may already be running by then: while the device works on a decode-only
+        step, the host fixes that step's successor (``Scheduler.schedule_ahead``), lays it out and launches it with
+        the token ids taken on the device from this step's sampler output, and only then waits for this step's
+        tokens.  The device so never waits for the host between decode steps.  A request that stops on a token that
+        was still in flight has a row in the successor that nobody reads."""
         step_start = time.perf_counter()
-        scheduled = self.scheduler.schedule()
-        self.stats["scheduler_ms"].append((time.perf_counter() - step_start) * 1000)
-        if scheduled.is_empty():
-            return
+        flight, self._ahead = self._ahead, None
+        if flight is not None and not any(self._alive(r) for r in flight.sampled):
+            flight = None  # launched for requests that have all stopped or been aborted since
+        if flight is None:
+            scheduled = self.scheduler.schedule()
+            self.stats["scheduler_ms"].append((time.perf_counter() - step_start) * 1000)
+            if scheduled.is_empty():
+                return
+            flight = self._launch(scheduled.decode_batch, scheduled.prefill_batch)
+        if self.config.decode_lookahead and flight.tokens is not None and not flight.prefill:
+            alive = [(row, r) for row, r in enumerate(flight.sampled) if self._alive(r)]
+            if alive and not any(r.sampling_params.has_penalties for _, r in alive):
+                ahead = self.scheduler.schedule_ahead([r for _, r in alive])
+                if ahead is not None:
+                    self._ahead = self._launch(ahead, [], ids_on_device=(flight.tokens, [row for row, _ in alive]))
+        self._finish_step(flight)
+        self.num_steps += 1
+        self.stats["step_ms"].append((time.perf_counter() - step_start) * 1000)
 
+    @staticmethod
+    def _alive(request: Request) -> bool:
+        return not request.finished and request.cache is not None
+
+    def _launch(self, decode: List[Request], prefill: List[Request], ids_on_device=None) -> "_Flight":
+        """Queues one step on the device: the forward over the batch and the sampler.  With ``ids_on_device`` the step
+        before this one has not been finished on the host yet: every request is one position and one generated token
+        further than its fields say."""
+        ahead = 1 if ids_on_device is not None else 0
         entries: List[StepEntry] = []
         sampled: List[Request] = []
         # decode rows first, then prompt portions; only rows that complete their tokens are sampled
-        for request in scheduled.decode_batch:
-            token = request.all_token_ids[request.num_computed_tokens]
-            entries.append(StepEntry(request.cache, [token], request.num_computed_tokens, [0]))
+        for request in decode:
+            start = request.num_computed_tokens + ahead
+            token = 0 if ahead else request.all_token_ids[start]
+            entries.append(StepEntry(request.cache, [token], start, [0]))
             sampled.append(request)
-        for request in scheduled.prefill_batch:
+        for request in prefill:
             start = request.num_computed_tokens
             chunk = request.current_chunk_size
             tokens = request.all_token_ids[start:start + chunk]
@@ -178,10 +226,10 @@ class Engine:
                 sampled.append(request)
 
         t0 = time.perf_counter()
-        logits = self.runner.step(entries)
+        logits = self.runner.step(entries, ids_on_device=ids_on_device)
         self.stats["forward_ms"].append((time.perf_counter() - t0) * 1000)
 
-        tokens: List[int] = []
+        tokens_gpu = None
         if sampled:
             t0 = time.perf_counter()
             needs_history = any(r.sampling_params.has_penalties for r in sampled)
@@ -189,29 +237,48 @@ class Engine:
                 logits,
                 [r.sampling_params for r in sampled],
                 [r.request_id for r in sampled],
-                [len(r.output_token_ids) for r in sampled],
+                [len(r.output_token_ids) + ahead for r in sampled],
                 histories=[r.all_token_ids for r in sampled] if needs_history else None,
             )
-            sync_start = time.perf_counter()
-            tokens = tokens_gpu.tolist()  # the one place per step where the host waits for the device
-            self.stats["cpu_sync_wait_ms"].append((time.perf_counter() - sync_start) * 1000)
             self.stats["sampling_ms"].append((time.perf_counter() - t0) * 1000)
+        # the copy of the tokens to the host is queued right behind the sampler, before a later step can be queued
+        # behind it: waiting for it then waits for this step only
+        landing = None
+        if tokens_gpu is not None and self.device.type == "cuda":
+            landing = self._landings[self._next_landing]
+            self._next_landing = (self._next_landing + 1) % len(self._landings)
+            landing[0][: len(sampled)].copy_(tokens_gpu, non_blocking=True)
+            landing[1].record()
+        return _Flight(list(decode), list(prefill), sampled, tokens_gpu, landing)
 
-        for request in scheduled.decode_batch:
-            self.scheduler.advance(request, 1)
-        for request in scheduled.prefill_batch:
-            self.scheduler.advance(request, request.current_chunk_size)
-            request.refresh_status()
-        for request, token in zip(sampled, tokens):
+    def _finish_step(self, flight: "_Flight") -> None:
+        """Waits for the step's tokens and books them: positions computed, tokens appended, stops."""
+        tokens: List[int] = []
+        if flight.tokens is not None:
+            sync_start = time.perf_counter()
+            # the one place per step where the host waits for the device
+            if flight.landing is not None:
+                flight.landing[1].synchronize()
+                tokens = flight.landing[0][: len(flight.sampled)].tolist()
+            else:
+                tokens = flight.tokens.tolist()
+            self.stats["cpu_sync_wait_ms"].append((time.perf_counter() - sync_start) * 1000)
+        for request in flight.decode:
+            if self._alive(request):
+                self.scheduler.advance(request, 1)
+        for request in flight.prefill:
+            if self._alive(request):
+                self.scheduler.advance(request, request.current_chunk_size)
+                request.refresh_status()
+        for request, token in zip(flight.sampled, tokens):
+            if not self._alive(request):
+                continue  # stopped or aborted while this step was in flight
             request.append_token(int(token))
             request.refresh_status()
             reason = request.should_stop(int(token), self.eos_token_ids)
             if reason is not None:
                 request.finish(reason)
                 self.sampler.release(request.request_id)
-
-        self.num_steps += 1
-        self.stats["step_ms"].append((time.perf_counter() - step_start) * 1000)
 
     @torch.no_grad()
     def generate(self, requests: Sequence[Request], max_steps: Optional[int] = None) -> List[Request]:

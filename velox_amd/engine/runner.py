@@ -64,15 +64,16 @@ class ModelRunner:
 
     # -- the step -----------------------------------------------------------------------
     @torch.no_grad()
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], ids_on_device: Optional[tuple] = None) -> Optional[torch.Tensor]:
         """Runs the entries' tokens as one batch; returns float32 logits ``[wanted, vocab]``
-        in the order of the entries and of their ``want`` (None when nothing is wanted)."""
+        in the order of the entries and of their ``want`` (None when nothing is wanted).
+        ``ids_on_device``: see ``BatchBuilder.build`` (the entries' own ``token_ids`` are placeholders then)."""
         if self.enable_graphs and all(len(e.token_ids) == 1 for e in entries):
             if all(list(e.want) == [0] for e in entries):
                 bucket = self._bucket_for(len(entries))
                 if bucket is not None:
-                    return self._replay(bucket, entries)
-        ctx = self.builder.build(entries, self.ops, self.dtype, self.workspace)
+                    return self._replay(bucket, entries, ids_on_device)
+        ctx = self.builder.build(entries, self.ops, self.dtype, self.workspace, ids_on_device=ids_on_device)
         return self._forward(ctx)
 
     def _forward(self, ctx: StepContext) -> Optional[torch.Tensor]:
@@ -88,12 +89,12 @@ class ModelRunner:
                 return bucket
         return None
 
-    def _padded_entries_context(self, bucket: int, entries: Sequence[StepEntry]) -> StepContext:
+    def _padded_entries_context(self, bucket: int, entries: Sequence[StepEntry], ids_on_device: Optional[tuple] = None) -> StepContext:
         buffer = self._graph_buffers[bucket]
         padded = [StepEntry(e.seq, e.token_ids, e.start, [0]) for e in entries]
         ctx = self.builder.build(
             padded, self.ops, self.dtype, self.workspace,
-            device_buffer=buffer, pad_to=bucket, width=self.builder.width,
+            device_buffer=buffer, pad_to=bucket, width=self.builder.width, ids_on_device=ids_on_device,
         )
         return ctx
 
@@ -138,9 +139,9 @@ class ModelRunner:
         ctx.rows = ctx.rows[:bucket]
         return ctx
 
-    def _replay(self, bucket: int, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def _replay(self, bucket: int, entries: Sequence[StepEntry], ids_on_device: Optional[tuple] = None) -> torch.Tensor:
         graph, logits, _ = self._graphs[bucket]
-        self._padded_entries_context(bucket, entries)  # refreshes the bucket's buffer in place
+        self._padded_entries_context(bucket, entries, ids_on_device)  # refreshes the bucket's buffer in place
         graph.replay()
         self.num_graph_replays += 1
         return logits[: len(entries)]
