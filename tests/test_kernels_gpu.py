@@ -242,6 +242,28 @@ def test_paged_attention_mixed_batch(ops, ref, dtype, nh, nkv, d, page):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,page", [(28, 4, 128, 16), (32, 16, 64, 64), (16, 8, 32, 8), (24, 12, 48, 4)])
+@pytest.mark.parametrize("window", [None, 300])
+def test_paged_attention_long_portions(ops, ref, dtype, nh, nkv, d, page, window):
+    """Steps with thousands of rows take the 128-row workgroups in bfloat16: long whole prompts, a long portion behind
+    a longer context, and short entries beside them.  A row's result is the same bits as in a small step."""
+    seqs = [(1100, 1100), (700, 1300), (1, 97), (300, 300), (2, 40)]
+    case = _attention_case(dtype, nh, nkv, d, page, seqs, seed=d + nh + 1)
+    got = _run_attention(ops, case, nh, nkv, d, page, window=window)
+    want = _run_attention(ref, case, nh, nkv, d, page, window=window)
+    torch.testing.assert_close(got, want, **(dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)))
+    # the 300-token prompt again, in a step of its own (64-row workgroups): its rows must not have changed
+    first = sum(q for q, _ in seqs[:3])
+    alone = dict(case)
+    alone["qkv"] = case["qkv"][first:first + 300].contiguous()
+    alone["tables"] = case["tables"][3:4].contiguous()
+    alone["cu"] = torch.tensor([0, 300], dtype=torch.int32, device="cuda")
+    alone["kv"] = case["kv"][3:4].contiguous()
+    alone["max_q"], alone["max_kv"] = 300, 300
+    torch.testing.assert_close(_run_attention(ops, alone, nh, nkv, d, page, window=window), got[first:first + 300], rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 4), (28, 4, 128, 16), (3, 1, 32, 8)])
 def test_paged_attention_garbage_in_unused_slots_and_null_page(ops, ref, dtype, nh, nkv, d, page):
     seqs = [(5, 37), (1, 64), (9, 9)]

@@ -127,11 +127,14 @@ template <> struct Softmax<bf16_t> {
 };
 
 constexpr int PREFILL_PAGE_IDS = 2048;
+// two waves per SIMD hide each other's waits; up to head size 128 the registers allow it without spilling, and the
+// compiler is held to it (left alone it takes more registers than one wave per SIMD's worth buys back)
+constexpr int GENERAL_MIN_WAVES = D <= 128 ? 2 : 1;
 
 // CT = 16-row tiles per wave: a workgroup owns 64 * CT rows.  With CT = 2 every K and V^T operand read from LDS feeds
 // two matrix instructions, which is what long portions of prompts need; a row's arithmetic is the same for every CT.
 template <typename T, int BN, int CT>
-__global__ void __launch_bounds__(256) paged_attention_kernel(
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(GENERAL_MIN_WAVES, 2))) paged_attention_kernel(
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
     T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
@@ -682,6 +685,17 @@ __global__ void merge_splits_kernel(const float* __restrict__ part_o, const floa
   }
 }
 
+static int compute_units() {
+  static int cached = 0;  // (the same value whichever thread gets here first)
+  if (cached == 0) {
+    int device = 0, count = 0;
+    if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0)
+      count = 256;
+    cached = count;
+  }
+  return cached;
+}
+
 template <typename T> constexpr int tile_keys() { return (sizeof(T) * D > 512) ? 32 : 64; }
 
 template <typename T>
@@ -703,11 +717,21 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
     merge_splits_kernel<T><<<dim3(total_tokens, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens);
     return (int)hipGetLastError();
   }
-  // (two row tiles per wave, CT = 2, need more registers than two waves per SIMD leave and measured slower)
-  dim3 grid((max_q_len * group + 63) / 64, nkv, num_seqs * splits);
-  paged_attention_kernel<T, BN, 1><<<grid, 256, 0, stream>>>(
-      (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-      part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
+  // 128 rows per workgroup (two row tiles per wave) when bfloat16 portions are long enough to fill them
+  // and the step brings enough rows that the larger workgroups still fill the GPU
+  constexpr int WIDE = (sizeof(T) == 2 && D <= 128) ? 2 : 1;
+  const int rows = max_q_len * group;
+  if (WIDE == 2 && rows > 64 && (long long)total_tokens * group / 128 * nkv >= compute_units()) {
+    dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
+    paged_attention_kernel<T, BN, WIDE><<<grid, 256, 0, stream>>>(
+        (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
+  } else {
+    dim3 grid((rows + 63) / 64, nkv, num_seqs * splits);
+    paged_attention_kernel<T, BN, 1><<<grid, 256, 0, stream>>>(
+        (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
+  }
   int status = (int)hipGetLastError();
   if (status != 0 || splits == 1) return status;
   merge_splits_kernel<T><<<dim3(total_tokens, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens);
