@@ -138,7 +138,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(GENERA
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
     T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
-    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens) {
+    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens, int slots) {
   typedef Block<T> B;
   typedef typename B::Operand Operand;
   constexpr int KB = B::KB;
@@ -161,7 +161,6 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(GENERA
   const int lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 4, i = lane & 15;
   const int group = nh / nkv;
-  const int kvh = blockIdx.y;
   const int b = blockIdx.z / splits, split = blockIdx.z % splits;
   const int page_size = 1 << page_shift;
 
@@ -170,9 +169,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(GENERA
   const int kv_len = kv_lens[b];
   const int ctx = kv_len - q_len;
   const int rows_total = q_len * group;
-  // late rows read the most keys: they go first, so that the long workgroups do not start last
-  const int r0 = (gridDim.x - 1 - blockIdx.x) * ROWS_PER_BLOCK;
-  if (r0 >= rows_total) return;
+  // Which (row block, KV head) this workgroup takes.  Late rows read the most keys.  Workgroups are handed to the
+  // compute units in launch order, `slots` at a time: the first round takes the longest units, the second the
+  // shortest (so that a compute unit's second workgroup makes up for its first), the third the next longest, ...
+  const int blocks_here = (rows_total + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
+  const int units = blocks_here * nkv;
+  const int launch_index = blockIdx.x + gridDim.x * blockIdx.y;
+  if (launch_index >= units) return;
+  const int round = launch_index / slots, within = launch_index % slots;
+  const int rank = (round & 1) ? units - 1 - ((round >> 1) * slots + within) : (round >> 1) * slots + within;  // 0 = longest
+  const int kvh = rank % nkv;
+  const int r0 = (blocks_here - 1 - rank / nkv) * ROWS_PER_BLOCK;
 
   bool row_ok[CT];
   int tok[CT], head[CT], pos[CT];
@@ -380,15 +387,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(GENERA
     Operand pf[CT][NKB];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
+      // the scale (positive) is applied inside the exponent's argument: the maximum is taken over the raw scores
       float mx = -INFINITY;
       if (whole) {
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            s[ct][t][j] *= scale_eff;
-            mx = fmaxf(mx, s[ct][t][j]);
-          }
+          for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[ct][t][j]);
       } else {
 #pragma unroll
         for (int t = 0; t < NT; ++t)
@@ -396,13 +401,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(GENERA
           for (int j = 0; j < 4; ++j) {
             const int n = n0 + 16 * t + 4 * g + j;
             const bool keep = row_ok[ct] && n < kv_len && n <= pos[ct] && (window <= 0 || n > pos[ct] - window);
-            s[ct][t][j] = keep ? s[ct][t][j] * scale_eff : -INFINITY;
+            s[ct][t][j] = keep ? s[ct][t][j] : -INFINITY;
             mx = fmaxf(mx, s[ct][t][j]);
           }
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16, VELOX_WAVE));
       mx = fmaxf(mx, __shfl_xor(mx, 32, VELOX_WAVE));
-      const float m_new = fmaxf(m_i[ct], mx);
+      const float m_new = fmaxf(m_i[ct], mx * scale_eff);
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
       alpha[ct] = (m_i[ct] == -INFINITY) ? 0.f : Softmax<T>::exp_of(m_i[ct] - m_safe);
       float psum = 0.f;
@@ -414,8 +419,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(GENERA
         for (int u = 0; u < TPB; ++u)
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const float sv = s[ct][kb * TPB + u][j];
-            const float p = (sv == -INFINITY) ? 0.f : Softmax<T>::exp_of(sv - m_safe);
+            // a masked score is -inf and gives exp(-inf) = 0; m_safe is finite
+            const float p = Softmax<T>::exp_of(fmaf(s[ct][kb * TPB + u][j], scale_eff, -m_safe));
             psum += p;
             e[4 * u + j] = from_f32<T>(p);
           }
@@ -725,12 +730,12 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
     dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
     paged_attention_kernel<T, BN, WIDE><<<grid, 256, 0, stream>>>(
         (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
+        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
   } else {
     dim3 grid((rows + 63) / 64, nkv, num_seqs * splits);
     paged_attention_kernel<T, BN, 1><<<grid, 256, 0, stream>>>(
         (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
+        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
   }
   int status = (int)hipGetLastError();
   if (status != 0 || splits == 1) return status;

@@ -463,6 +463,8 @@ class HipOps:
         self._check("v_cache", v_cache, qkv.dtype, (pages, num_kv_heads, head_dim, block_size), align=16)
         if num_heads % num_kv_heads != 0:
             raise KernelError("num_heads must be a multiple of num_kv_heads")
+        if not scale > 0:
+            raise KernelError(f"paged_attention: the scale must be positive, got {scale}")
         if max_q_len < 1 or max_q_len > tokens:
             raise KernelError(f"max_q_len={max_q_len} outside [1, {tokens}]")
         lib = self.attention_library(head_dim)
