@@ -246,7 +246,8 @@ def test_paged_attention_mixed_batch(ops, ref, dtype, nh, nkv, d, page):
 @pytest.mark.parametrize("window", [None, 300])
 def test_paged_attention_long_portions(ops, ref, dtype, nh, nkv, d, page, window):
     """Steps with thousands of rows take the 128-row workgroups in bfloat16: long whole prompts, a long portion behind
-    a longer context, and short entries beside them.  A row's result is the same bits as in a small step."""
+    a longer context, and short entries beside them.  A row's result is the same as in a small step, to rounding (the
+    large workgroups add a row's keys in another order) and to the bit in float32, which has one kind of workgroup."""
     seqs = [(1100, 1100), (700, 1300), (1, 97), (300, 300), (2, 40)]
     case = _attention_case(dtype, nh, nkv, d, page, seqs, seed=d + nh + 1)
     got = _run_attention(ops, case, nh, nkv, d, page, window=window)
@@ -260,7 +261,8 @@ def test_paged_attention_long_portions(ops, ref, dtype, nh, nkv, d, page, window
     alone["cu"] = torch.tensor([0, 300], dtype=torch.int32, device="cuda")
     alone["kv"] = case["kv"][3:4].contiguous()
     alone["max_q"], alone["max_kv"] = 300, 300
-    torch.testing.assert_close(_run_attention(ops, alone, nh, nkv, d, page, window=window), got[first:first + 300], rtol=0, atol=0)
+    same = dict(rtol=0, atol=0) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(_run_attention(ops, alone, nh, nkv, d, page, window=window), got[first:first + 300], **same)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

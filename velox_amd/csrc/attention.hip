@@ -133,8 +133,11 @@ constexpr int GENERAL_MIN_WAVES = D <= 128 ? 2 : 1;
 
 // CT = 16-row tiles per wave: a workgroup owns 64 * CT rows.  With CT = 2 every K and V^T operand read from LDS feeds
 // two matrix instructions, which is what long portions of prompts need; a row's arithmetic is the same for every CT.
-template <typename T, int BN, int CT>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(GENERAL_MIN_WAVES, 2))) paged_attention_kernel(
+// KSPLIT = 2: the workgroup has two sets of 4 waves that own the same rows and take the key tiles alternately, each
+// set staging its own tiles; at the end the second set hands its running (maximum, sum, output) to the first
+// through LDS.  The longest workgroups of a causal step, which decide how long the step takes, finish in half the time.
+template <typename T, int BN, int CT, int KSPLIT>
+__global__ void __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(GENERAL_MIN_WAVES, 2))) paged_attention_kernel(
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
     T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
@@ -153,11 +156,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(GENERA
   constexpr int TPB = KB / 16;                  // S^T tiles per key block
   constexpr int NC = D / 16;                    // 16-channel tiles of the output
   constexpr int ROWS_PER_BLOCK = 64 * CT;
-  __shared__ __attribute__((aligned(16))) T k_tile[BN * KS];
-  __shared__ __attribute__((aligned(16))) T v_tile[D * VS];
+  constexpr int TILE_ELEMS = BN * KS + D * VS;                      // one set's K tile and V^T tile
+  constexpr int MERGE_FLOATS = KSPLIT > 1 ? 256 * CT * (4 * NC + 2) : 0;  // what the second set hands over at the end
+  constexpr int TILE_BYTES = KSPLIT * TILE_ELEMS * (int)sizeof(T);
+  constexpr int SMEM_BYTES = TILE_BYTES > 4 * MERGE_FLOATS ? TILE_BYTES : 4 * MERGE_FLOATS;
+  __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
   __shared__ int page_ids[PREFILL_PAGE_IDS];
 
-  const int tid = threadIdx.x;
+  const int set = KSPLIT > 1 ? threadIdx.x / 256 : 0;  // which set of 4 waves
+  const int tid = KSPLIT > 1 ? threadIdx.x % 256 : threadIdx.x;  // thread within the set
+  T* const k_tile = reinterpret_cast<T*>(smem) + set * TILE_ELEMS;
+  T* const v_tile = k_tile + BN * KS;
   const int lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 4, i = lane & 15;
   const int group = nh / nkv;
@@ -233,7 +242,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(GENERA
   int first_page = (n_begin + tile_lo * BN) >> page_shift;  // first page of the window
   auto load_page_ids = [&]() {
     const int num_pages = last_page - first_page + 1;
-    for (int p = tid; p < num_pages && p < PREFILL_PAGE_IDS; p += 256) page_ids[p] = table[first_page + p];
+    for (int p = threadIdx.x; p < num_pages && p < PREFILL_PAGE_IDS; p += 256 * KSPLIT) page_ids[p] = table[first_page + p];
   };
   load_page_ids();
   if constexpr (DP > D) {
@@ -352,21 +361,26 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(GENERA
   };
 
   __syncthreads();  // page ids are in place
-  if (tile_lo < tile_hi) fetch(n_begin + tile_lo * BN);
-  for (int tile = tile_lo; tile < tile_hi; ++tile) {
+  // iteration `it` covers tiles tile_lo + it * KSPLIT .. + KSPLIT - 1, one per set (the last iteration may leave a set without one)
+  const int iterations = tile_hi > tile_lo ? (tile_hi - tile_lo + KSPLIT - 1) / KSPLIT : 0;
+  if (tile_lo + set < tile_hi) fetch(n_begin + (tile_lo + set) * BN);
+  for (int it = 0; it < iterations; ++it) {
+    const int tile = tile_lo + it * KSPLIT + set;
+    const bool have_tile = KSPLIT == 1 || tile < tile_hi;
     const int n0 = n_begin + tile * BN;
     __syncthreads();  // the previous tile has been read by every wave
-    commit(n0);
+    if (have_tile) commit(n0);
     __syncthreads();
-    if (tile + 1 < tile_hi) {
-      if (((n0 + 2 * BN - 1) >> page_shift) - first_page >= PREFILL_PAGE_IDS) {  // the same for every thread
-        first_page = (n0 + BN) >> page_shift;
+    if (it + 1 < iterations) {
+      const int next_first = n_begin + (tile_lo + (it + 1) * KSPLIT) * BN;  // first key of the next iteration's tiles
+      if (((next_first + KSPLIT * BN - 1) >> page_shift) - first_page >= PREFILL_PAGE_IDS) {  // the same for every thread
+        first_page = next_first >> page_shift;
         load_page_ids();
         __syncthreads();
       }
-      fetch(n0 + BN);  // in flight while this tile is computed
+      if (tile + KSPLIT < tile_hi) fetch(n0 + KSPLIT * BN);  // in flight while this tile is computed
     }
-    if (n0 > wave_last_pos) continue;        // nothing this wave may read; it still took part in the staging
+    if (!have_tile || n0 > wave_last_pos) continue;  // nothing this wave may read; it still took part in the staging
 
     // ---- S^T = K Q^T ----------------------------------------------------------------------
     float4_t s[CT][NT];
@@ -440,6 +454,36 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(GENERA
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) acc_o[ct][c] = B::mma(vf, pf[ct][kb], acc_o[ct][c]);
       }
+    }
+  }
+
+  if constexpr (KSPLIT > 1) {
+    // the second set's state goes through LDS (the tiles are no longer needed) and is folded into the first set's
+    __syncthreads();
+    float4_t* const hand_acc = reinterpret_cast<float4_t*>(smem);
+    float* const hand_ml = reinterpret_cast<float*>(smem) + 256 * CT * NC * 4;
+    if (set == 1) {
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) hand_acc[(ct * NC + c) * 256 + tid] = acc_o[ct][c];
+        hand_ml[ct * 256 + tid] = m_i[ct];
+        hand_ml[(CT + ct) * 256 + tid] = l_i[ct];
+      }
+    }
+    __syncthreads();
+    if (set == 1) return;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      const float m_other = hand_ml[ct * 256 + tid], l_other = hand_ml[(CT + ct) * 256 + tid];
+      const float m_new = fmaxf(m_i[ct], m_other);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float mine = (m_i[ct] == -INFINITY) ? 0.f : Softmax<T>::exp_of(m_i[ct] - m_safe);
+      const float theirs = (m_other == -INFINITY) ? 0.f : Softmax<T>::exp_of(m_other - m_safe);
+      l_i[ct] = l_i[ct] * mine + l_other * theirs;
+      m_i[ct] = m_new;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) acc_o[ct][c] = acc_o[ct][c] * mine + hand_acc[(ct * NC + c) * 256 + tid] * theirs;
     }
   }
 
@@ -728,12 +772,18 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
   const int rows = max_q_len * group;
   if (WIDE == 2 && rows > 64 && (long long)total_tokens * group / 128 * nkv >= compute_units()) {
     dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
-    paged_attention_kernel<T, BN, WIDE><<<grid, 256, 0, stream>>>(
+    paged_attention_kernel<T, BN, WIDE, 1><<<grid, 256, 0, stream>>>(
+        (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+  } else if (WIDE == 2 && (long long)((rows + 63) / 64) * nkv * num_seqs * splits < 2 * compute_units() && max_kv_len >= 8 * BN) {
+    // too few workgroups to fill the GPU and many keys each: two sets of waves share a workgroup's keys
+    dim3 grid((rows + 63) / 64, nkv, num_seqs * splits);
+    paged_attention_kernel<T, BN, 1, WIDE><<<grid, 256 * WIDE, 0, stream>>>(
         (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
         part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
   } else {
     dim3 grid((rows + 63) / 64, nkv, num_seqs * splits);
-    paged_attention_kernel<T, BN, 1><<<grid, 256, 0, stream>>>(
+    paged_attention_kernel<T, BN, 1, 1><<<grid, 256, 0, stream>>>(
         (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
         part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
   }
