@@ -266,6 +266,19 @@ def test_paged_attention_long_portions(ops, ref, dtype, nh, nkv, d, page, window
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,page", [(28, 4, 128, 16), (4, 2, 16, 4), (6, 2, 96, 8), (8, 8, 64, 1)])
+@pytest.mark.parametrize("window", [None, 200])
+def test_paged_attention_few_rows_many_keys(ops, ref, dtype, nh, nkv, d, page, window):
+    """Short portions behind long contexts: few workgroups, each with many key tiles (in bfloat16 two sets of waves
+    then share a workgroup's tiles, an odd number of tiles included)."""
+    seqs = [(40, 900), (3, 705), (1, 520), (17, 64 * 9 + 17)]
+    case = _attention_case(dtype, nh, nkv, d, page, seqs, seed=d + nh + 2)
+    got = _run_attention(ops, case, nh, nkv, d, page, window=window)
+    want = _run_attention(ref, case, nh, nkv, d, page, window=window)
+    torch.testing.assert_close(got, want, **(dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 4), (28, 4, 128, 16), (3, 1, 32, 8)])
 def test_paged_attention_garbage_in_unused_slots_and_null_page(ops, ref, dtype, nh, nkv, d, page):
     seqs = [(5, 37), (1, 64), (9, 9)]
