@@ -344,6 +344,21 @@ def test_far_key_among_hundreds_is_found(ops):
     torch.testing.assert_close(out, want, rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("rows,vocab", [(1, 152064), (8, 151936), (64, 32003), (3, 5000), (300, 4099), (2, 2047)])
+def test_argmax_over_chunks_of_the_vocabulary(ops, ref, rows, vocab):
+    logits = rand((rows, vocab), torch.float32, 31, 3.0)
+    torch.testing.assert_close(ops.argmax(logits), ref.argmax(logits))
+    # ties across chunks: the first index wins; a maximum in the last, shorter chunk is found
+    logits[0, vocab // 3] = logits[0, vocab - 5] = 60.0
+    logits[rows - 1, vocab - 1] = 70.0
+    got = ops.argmax(logits)
+    assert int(got[rows - 1]) == vocab - 1 and (rows == 1 or int(got[0]) == vocab // 3)
+    # an unaligned row start (a slice of a wider tensor)
+    wide = rand((rows, vocab + 3), torch.float32, 32, 3.0)
+    if (vocab + 3) % 4 == 0:
+        torch.testing.assert_close(ops.argmax(wide[:, :vocab].contiguous()), ref.argmax(wide[:, :vocab]))
+
+
 def test_argmax_and_sampling(ops, ref):
     vocab = 1003
     logits = rand((6, vocab), torch.float32, 30, 3.0)

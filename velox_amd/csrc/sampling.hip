@@ -44,29 +44,61 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
   return total;
 }
 
-__global__ void __launch_bounds__(SAMPLE_THREADS) argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int vocab) {
-  __shared__ Best scratch[16];
-  const float* row = logits + (size_t)blockIdx.x * vocab;
+// the best of row[lo .. hi), indices counted from the start of the row
+__device__ __forceinline__ Best best_of_range(const float* __restrict__ row, int lo, int hi, Best* scratch) {
   Best best{-INFINITY, 0x7fffffff};
-  // 16-byte loads over the aligned middle of the row, single elements at its ends
-  const int head = (int)((16 - ((uintptr_t)row & 15)) & 15) / 4;
-  const int first = head < vocab ? head : vocab;
-  const int quads = (vocab - first) / 4;
-  for (int i = threadIdx.x; i < first; i += blockDim.x) best = better(best, Best{row[i], i});
-  const float4_t* body = reinterpret_cast<const float4_t*>(row + first);
+  // 16-byte loads over the aligned middle of the range, single elements at its ends
+  const float* start = row + lo;
+  const int count = hi - lo;
+  const int head = (int)((16 - ((uintptr_t)start & 15)) & 15) / 4;
+  const int first = head < count ? head : count;
+  const int quads = (count - first) / 4;
+  for (int i = threadIdx.x; i < first; i += blockDim.x) best = better(best, Best{start[i], lo + i});
+  const float4_t* body = reinterpret_cast<const float4_t*>(start + first);
   for (int q = threadIdx.x; q < quads; q += blockDim.x) {
     const float4_t v = body[q];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) best = better(best, Best{v[j], first + 4 * q + j});
+    for (int j = 0; j < 4; ++j) best = better(best, Best{v[j], lo + first + 4 * q + j});
   }
-  for (int i = first + 4 * quads + threadIdx.x; i < vocab; i += blockDim.x) best = better(best, Best{row[i], i});
-  best = block_best(best, scratch);
+  for (int i = first + 4 * quads + threadIdx.x; i < count; i += blockDim.x) best = better(best, Best{start[i], lo + i});
+  return block_best(best, scratch);
+}
+
+// One workgroup per (row, chunk of the vocabulary).  With one chunk the index goes straight to `out`; with several, each
+// chunk's best goes to `partial[row][chunk]` and argmax_merge_kernel picks among them (few rows alone would leave most
+// of the GPU idle while 600 KB per row are read).
+__global__ void __launch_bounds__(SAMPLE_THREADS) argmax_kernel(const float* __restrict__ logits, int* __restrict__ out,
+                                                               Best* __restrict__ partial, int vocab, int chunk) {
+  __shared__ Best scratch[16];
+  const float* row = logits + (size_t)blockIdx.x * vocab;
+  const int lo = blockIdx.y * chunk;
+  const int hi = lo + chunk < vocab ? lo + chunk : vocab;
+  const Best best = best_of_range(row, lo, hi, scratch);
+  if (threadIdx.x != 0) return;
+  if (gridDim.y == 1) out[blockIdx.x] = best.index;
+  else partial[blockIdx.x * gridDim.y + blockIdx.y] = best;
+}
+
+__global__ void __launch_bounds__(64) argmax_merge_kernel(const Best* __restrict__ partial, int* __restrict__ out, int chunks) {
+  Best best{-INFINITY, 0x7fffffff};
+  for (int c = threadIdx.x; c < chunks; c += 64) best = better(best, partial[blockIdx.x * chunks + c]);
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) {
+    Best other;
+    other.value = __shfl_xor(best.value, offset, VELOX_WAVE);
+    other.index = __shfl_xor(best.index, offset, VELOX_WAVE);
+    best = better(best, other);
+  }
   if (threadIdx.x == 0) out[blockIdx.x] = best.index;
 }
 
-extern "C" int velox_argmax(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
+// partial: room for rows * chunks (value, index) pairs of 8 bytes, used when chunks > 1.
+extern "C" int velox_argmax(const float* logits, int* out, void* partial, int rows, int vocab, int chunks, hipStream_t stream) {
   if (rows <= 0) return 0;
-  argmax_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, out, vocab);
+  if (chunks < 1 || (chunks > 1 && partial == nullptr)) return -1;
+  const int chunk = (vocab + chunks - 1) / chunks;
+  argmax_kernel<<<dim3(rows, chunks), SAMPLE_THREADS, 0, stream>>>(logits, out, (Best*)partial, vocab, chunk);
+  if (chunks > 1) argmax_merge_kernel<<<rows, 64, 0, stream>>>((const Best*)partial, out, chunks);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 

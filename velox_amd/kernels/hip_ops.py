@@ -77,7 +77,7 @@ class HipOps:
         c.velox_skinny_gemm_glu_bf16.restype = _I
         c.velox_skinny_gemm_splitk_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
         c.velox_skinny_gemm_splitk_bf16.restype = _I
-        c.velox_argmax.argtypes = [_P, _P, _I, _I, _P]
+        c.velox_argmax.argtypes = [_P, _P, _P, _I, _I, _I, _P]
         c.velox_sample.argtypes = [_P, _P, _P, _I, _I, _P]
         c.velox_apply_penalties.argtypes = [_P, _P, _P, _P, _I, _I, _I, _P]
         for fn in (c.velox_embed, c.velox_add_rmsnorm, c.velox_silu_mul, c.velox_rope_kv_write, c.velox_gemm_fma,
@@ -493,7 +493,10 @@ class HipOps:
         self._check("logits", logits, torch.float32)
         rows, vocab = logits.shape
         out = torch.empty(rows, dtype=torch.int32, device=self.device)
-        self._launched(self._core.velox_argmax(_ptr(logits), _ptr(out), rows, vocab, self._stream()), "argmax")
+        # few rows alone would leave most of the GPU idle: the vocabulary is cut into chunks of at least 2048 entries
+        chunks = max(1, min(2 * self.num_cus // rows, vocab // 2048, 256))
+        partial = torch.empty((rows, chunks, 2), dtype=torch.int32, device=self.device) if chunks > 1 else None
+        self._launched(self._core.velox_argmax(_ptr(logits), _ptr(out), _ptr(partial), rows, vocab, chunks, self._stream()), "argmax")
         return out
 
     def sample(self, logits: torch.Tensor, options: torch.Tensor) -> torch.Tensor:
