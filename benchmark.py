@@ -47,8 +47,12 @@ def rule(title: str = "") -> None:
     print("\n" + "=" * 78 + f"\n  {title}\n" + "=" * 78 if title else "-" * 78)
 
 
-def build_prompts(workload: str, count: int, vocab: int, limit: int, fixed_len: Optional[int], seed: int) -> List[List[int]]:
+SHARED_PREFIX_TOKENS = 96  # stands in for the reference's shared system prompt (``benchmark.py:42-47``, about 90 tokens)
+
+
+def build_prompts(workload: str, count: int, vocab: int, limit: int, fixed_len: Optional[int], seed: int, shared_prefix: bool = False) -> List[List[int]]:
     rng = random.Random(seed)
+    prefix = [rng.randrange(vocab) for _ in range(min(SHARED_PREFIX_TOKENS, max(0, limit - 1)))] if shared_prefix else []
     prompts = []
     for index in range(count):
         if fixed_len:
@@ -57,8 +61,8 @@ def build_prompts(workload: str, count: int, vocab: int, limit: int, fixed_len: 
             kind = workload if workload != "mixed" else ("short", "long")[index % 2]
             lo, hi = WORKLOAD_LENGTHS[kind]
             length = rng.randint(lo, hi)
-        length = max(1, min(length, limit))
-        prompts.append([rng.randrange(vocab) for _ in range(length)])
+        length = max(1, min(length, limit - len(prefix)))
+        prompts.append(prefix + [rng.randrange(vocab) for _ in range(length)])
     return prompts
 
 
@@ -150,7 +154,9 @@ def parse_args(argv=None) -> argparse.Namespace:
     parser.add_argument("--block-size", type=int, default=16)
     parser.add_argument("--num-gpu-blocks", type=int, default=None)
     parser.add_argument("--gpu-memory-utilization", type=float, default=0.85)
+    parser.add_argument("--no-prefix-caching", action="store_true", help="accepted for the reference's command lines; there is no prefix cache to turn off")
     parser.add_argument("--no-cuda-graphs", "--no-hip-graphs", dest="no_graphs", action="store_true")
+    parser.add_argument("--shared-system-prompt", action="store_true", help="every prompt starts with the same %d tokens" % SHARED_PREFIX_TOKENS)
     parser.add_argument("--sweep-batch-size", default=None, help="comma-separated max_num_seqs values to sweep")
     parser.add_argument("--rounds", type=int, default=1, help="replay the workload N times")
     parser.add_argument("--show-outputs", action="store_true")
@@ -193,7 +199,7 @@ def main(argv=None) -> int:
         limit = engine.max_model_len - args.max_tokens - 1
         if limit < 1:
             raise SystemExit("--max-tokens leaves no room for a prompt under --max-model-len")
-        prompts = build_prompts(args.workload, args.num_requests, vocab, limit, args.prompt_len, args.seed)
+        prompts = build_prompts(args.workload, args.num_requests, vocab, limit, args.prompt_len, args.seed, args.shared_system_prompt)
         rule("ENGINE BENCHMARK")
         print(f"  Model            : {args.model or args.shape + ' (random weights)'}")
         print(f"  PyTorch / HIP    : {torch.__version__} / {torch.version.hip}")
