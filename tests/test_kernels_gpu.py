@@ -188,6 +188,67 @@ def test_qkv_projection_with_rotation_and_cache_write_in_one_kernel(ops, ref, m,
     assert torch.equal(before, k_cache)
 
 
+@pytest.mark.parametrize("m", [1, 7, 16])
+@pytest.mark.parametrize("hidden,inner", [(64, 128), (3584, 3584), (200, 320), (96, 18944)])
+def test_residual_add_and_norm_split_between_two_products(ops, ref, m, hidden, inner):
+    """The decode fusion: a product adds itself to the residual and applies the norm weight (DeferredNorm); the next
+    product (plain, gate/up + SiLU, or q/k/v with rotation) scales its rows.  Against residual add -> RMSNorm -> product
+    done one after the other."""
+    from velox_amd.parts.base import DeferredNorm, ResidualSink
+    from velox_amd.parts.norms import RMSNorm
+
+    x = rand((m, inner), torch.bfloat16, 80)
+    w_out = rand((hidden, inner), torch.bfloat16, 81, 0.05)
+    residual0 = rand((m, hidden), torch.float32, 82, 2.0)
+    norm = RMSNorm("", hidden, 1e-5)
+    norm.weight = (1.0 + rand((hidden,), torch.float32, 83, 0.1))
+    ops.register_weight(w_out)
+    if hidden % 64 != 0:
+        # the next product cannot stream this width: it gets the materialised rows
+        pass
+    # reference: product in float32 from the bfloat16 operands, add, norm
+    delta = ref.linear(x, w_out, None, torch.float32)
+    want_residual = residual0 + delta
+    want_normed = ref.add_rmsnorm(residual0.clone(), delta, norm.weight, norm.eps, torch.float32)
+    residual = residual0.clone()
+    deferred = ops.linear(x, w_out, None, torch.bfloat16, partials_ok=True, residual_norm=ResidualSink(residual, norm))
+    assert isinstance(deferred, DeferredNorm) and deferred.norm is norm
+    torch.testing.assert_close(residual, want_residual, rtol=1e-5, atol=1e-4 * float(want_residual.abs().max()))
+    torch.testing.assert_close(ops.materialize(deferred).float(), want_normed, rtol=2e-2, atol=2e-2)
+    assert norm.forward(residual, deferred, None) is deferred
+    with pytest.raises(ValueError):
+        RMSNorm("", hidden, 1e-5).forward(residual, deferred, None)
+    if hidden % 64 != 0:
+        return
+    # consumers
+    normed_bf16 = want_normed.to(torch.bfloat16)
+    w_next = rand((320, hidden), torch.bfloat16, 84, 0.05)
+    bias = rand((320,), torch.float32, 85)
+    scale = float(ref.linear(normed_bf16, w_next, None, torch.float32).abs().max())
+    tol = dict(rtol=2e-2, atol=2e-2 * scale)
+    torch.testing.assert_close(ops.linear(deferred, w_next, bias, torch.float32), ref.linear(normed_bf16, w_next, bias, torch.float32), **tol)  # unregistered: materialised
+    ops.register_weight(w_next)
+    torch.testing.assert_close(ops.linear(deferred, w_next, bias, torch.float32), ref.linear(normed_bf16, w_next, bias, torch.float32), **tol)
+    ops.register_weight(w_next, stacked=2)
+    want_glu = ref.linear_silu_mul(normed_bf16, w_next, torch.bfloat16).float()
+    torch.testing.assert_close(ops.linear_silu_mul(deferred, w_next, torch.bfloat16).float(), want_glu, rtol=3e-2, atol=3e-2 * float(want_glu.abs().max()))
+    # q/k/v with rotation: 2 heads, 1 kv head, head size 80 -> 320 rows
+    nh, nkv, d, page, pages = 2, 1, 80, 8, 12
+    ops.register_weight(w_next, rotary_heads=(nh, nkv, d))
+    positions = torch.randint(0, 300, (m,), generator=torch.Generator().manual_seed(86)).to(torch.int32).cuda()
+    slots = (torch.randperm((pages - 1) * page, generator=torch.Generator().manual_seed(87))[:m] + page).to(torch.int32).cuda()
+    angles = torch.outer(torch.arange(512, dtype=torch.float32), 1.0 / (10000.0 ** (torch.arange(d // 2, dtype=torch.float32) / (d // 2))))
+    cos, sin = angles.cos().cuda(), angles.sin().cuda()
+    outs = []
+    for source in (deferred, normed_bf16):
+        k_cache = torch.zeros((pages, nkv, page, d), dtype=torch.bfloat16, device="cuda")
+        v_cache = torch.zeros((pages, nkv, d, page), dtype=torch.bfloat16, device="cuda")
+        q = ops.qkv_rope_write(source, w_next, bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page)
+        outs.append((q[:, : nh * d].float(), k_cache.float(), v_cache.float()))
+    for got, want in zip(*outs):
+        torch.testing.assert_close(got, want, rtol=3e-2, atol=3e-2 * max(1.0, float(want.abs().max())))
+
+
 def _attention_case(dtype, nh, nkv, d, page, seqs, seed, garbage=False):
     """seqs: list of (q_len, kv_len).  Builds a paged cache with shuffled pages and a flat qkv."""
     g = torch.Generator().manual_seed(seed)

@@ -64,6 +64,9 @@ class TorchOps:
     def register_weight(self, weight, stacked=1, rotary_heads=None) -> None:
         pass
 
+    def materialize(self, x):
+        return x
+
     def qkv_rope_write(self, x, weight, bias, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size, write_kv=True):
         qkv = self.linear(x, weight, None, x.dtype)
         self.rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size, write_kv=write_kv, bias=bias)
@@ -91,7 +94,7 @@ class TorchOps:
         return (x * torch.rsqrt(var + eps) * weight.float()).to(out_dtype)
 
     # -- matrix products ----------------------------------------------------------------
-    def linear(self, x, weight, bias, out_dtype, partials_ok=False):
+    def linear(self, x, weight, bias, out_dtype, partials_ok=False, residual_norm=None):
         out = x.float() @ weight.float().T
         if bias is not None:
             out = out + bias.float()

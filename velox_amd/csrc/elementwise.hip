@@ -365,3 +365,27 @@ extern "C" int velox_rope_kv_write(void* qkv, const float* bias, const int* posi
                                                            (float*)k_cache, (float*)v_cache, nh, nkv, d, page_size, write_kv);
   VELOX_RETURN_LAUNCH_STATUS();
 }
+
+
+// out[m, :] = x[m, :] * rsqrt(sum_b sums[m][b] / width + eps): the second half of a norm whose first half (the weight)
+// a product's epilogue has applied already; for consumers that cannot scale their own result rows.  m <= 16 rows.
+__global__ void row_scale_apply_kernel(const bf16_t* __restrict__ x, const float* __restrict__ sums, int blocks, float inv_width,
+                                       float eps, bf16_t* __restrict__ out, int n) {
+  __shared__ float scale;
+  const int row = blockIdx.x;
+  if (threadIdx.x == 0) {
+    float total = 0.f;
+    for (int b = 0; b < blocks; ++b) total += sums[(size_t)row * blocks + b];
+    scale = rsqrtf(total * inv_width + eps);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += blockDim.x) out[(size_t)row * n + i] = from_f32<bf16_t>(to_f32(x[(size_t)row * n + i]) * scale);
+}
+
+extern "C" int velox_row_scale_apply(const void* x, const float* sums, int blocks, float inv_width, float eps, void* out, int m, int n,
+                                     hipStream_t stream) {
+  if (m <= 0 || n <= 0) return 0;
+  if (m > 16) return -1;
+  row_scale_apply_kernel<<<m, 256, 0, stream>>>((const bf16_t*)x, sums, blocks, inv_width, eps, (bf16_t*)out, n);
+  VELOX_RETURN_LAUNCH_STATUS();
+}

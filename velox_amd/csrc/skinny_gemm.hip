@@ -125,12 +125,54 @@ __device__ __forceinline__ void skinny_partial_sums(const bf16_t* __restrict__ a
   __syncthreads();
 }
 
+// Rows of A that still have to be normalised: A holds x * norm_weight in bfloat16 and the producer (the kernel
+// below that adds a product to the residual stream) left sums of squares of x, one per workgroup and row; a product with
+// such an A is scaled row by row with rstd[m] = rsqrt(sum_b partial[b][m] / width + eps) in its epilogue, which is the
+// same as normalising A first.  The sums are added in a fixed order.  Only for M <= 16.
+struct RowScale {
+  const float* partial;  // [16][blocks] (row m's sums are contiguous), or null: rows are used as they are
+  int blocks;
+  float inv_width, eps;
+};
+
+// The table of sums is copied into LDS by loads that write LDS directly: issued before the main loop, they fly while
+// the weights stream and hold no registers meanwhile.  After the main loop's barrier row_scale_of adds a row's entries.
+constexpr int ROW_SCALE_BLOCKS = 512;  // room in LDS: residual widths up to 16 * 512
+
+template <int WAVES>
+__device__ __forceinline__ void row_scale_copy(const RowScale& rs, int m, float (&table)[ROW_SCALE_BLOCKS * 16]) {
+  if (rs.partial == nullptr) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int count = rs.blocks * m;  // the rows in use come first
+  for (int first = wave * 64; first < count; first += WAVES * 64) {
+    const int at = first + lane < count ? first + lane : count - 1;  // (the spare lanes of a last pass repeat the last entry)
+    // lane's 4 bytes land at table[first + lane]
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(rs.partial + at),
+                                     (__attribute__((address_space(3))) void*)(table + first), 4, 0, 0);
+  }
+}
+
+// after the barrier that follows the main loop; every lane of the wave has to call it (l = its lane)
+__device__ __forceinline__ float row_scale_of(const RowScale& rs, int m, const float (&table)[ROW_SCALE_BLOCKS * 16], int l) {
+  if (rs.partial == nullptr) return 1.f;
+  const int row = l & 15, grp = l >> 4;
+  float total = 0.f;
+  if (row < m)
+    for (int b = grp; b < rs.blocks; b += 4) total += table[row * rs.blocks + b];
+  total += __shfl_xor(total, 16, VELOX_WAVE);  // the four lane groups took every fourth block: a fixed order
+  total += __shfl_xor(total, 32, VELOX_WAVE);
+  return rsqrtf(total * rs.inv_width + rs.eps);
+}
+
 template <int RT, int CT, int WAVES, typename TO, bool GLU = false, bool PACKED = false>
 __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
-                                                                 const float* __restrict__ bias, TO* __restrict__ out, int m, int n, int k) {
+                                                                 const float* __restrict__ bias, TO* __restrict__ out, int m, int n, int k,
+                                                                 RowScale rs) {
   __shared__ float4_t partial[WAVES][RT * CT][64];
+  __shared__ float scale_table[ROW_SCALE_BLOCKS * 16];
   constexpr int RTO = GLU ? RT / 2 : RT;
   const int n0 = blockIdx.x * 16 * RTO;
+  row_scale_copy<WAVES>(rs, m, scale_table);
   skinny_partial_sums<RT, CT, WAVES, GLU, PACKED>(a, w, m, n, k, partial);
   // add the waves' partial sums in wave order; each tile's 64 lanes are spread over the workgroup
   for (int item = threadIdx.x; item < RTO * CT * 64; item += WAVES * 64) {
@@ -138,10 +180,13 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
     float4_t sum = partial[0][tile][l];
 #pragma unroll
     for (int wv = 1; wv < WAVES; ++wv) sum += partial[wv][tile][l];
+    const float row_scale = row_scale_of(rs, m, scale_table, l);  // (1 unless the rows of A wait for their norm)
+    sum = sum * row_scale;
     if constexpr (GLU) {
       float4_t up = partial[0][tile + RTO * CT][l];
 #pragma unroll
       for (int wv = 1; wv < WAVES; ++wv) up += partial[wv][tile + RTO * CT][l];
+      up = up * row_scale;
 #pragma unroll
       for (int j = 0; j < 4; ++j) sum[j] = sum[j] / (1.f + expf(-sum[j])) * up[j];
     }
@@ -160,29 +205,29 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
 }
 
 template <int RT, int CT, int WAVES>
-static int launch_skinny_glu(const void* a, const void* w, void* out, int m, int n, int k, bool packed, hipStream_t stream) {
+static int launch_skinny_glu(const void* a, const void* w, void* out, int m, int n, int k, bool packed, RowScale rs, hipStream_t stream) {
   const int blocks = (n + 8 * RT - 1) / (8 * RT);
   if (packed)
-    skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k);
+    skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k, rs);
   else
-    skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k);
+    skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k, rs);
   return (int)hipGetLastError();
 }
 
 template <int RT, int CT, int WAVES>
-static int launch_skinny(const void* a, const void* w, const float* bias, void* out, int m, int n, int k, int out_dtype, bool packed, hipStream_t stream) {
+static int launch_skinny(const void* a, const void* w, const float* bias, void* out, int m, int n, int k, int out_dtype, bool packed, RowScale rs, hipStream_t stream) {
   const int blocks = (n + 16 * RT - 1) / (16 * RT);
   if (packed) {
     if (out_dtype == VELOX_BF16)
-      skinny_gemm_kernel<RT, CT, WAVES, bf16_t, false, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (bf16_t*)out, m, n, k);
+      skinny_gemm_kernel<RT, CT, WAVES, bf16_t, false, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (bf16_t*)out, m, n, k, rs);
     else
-      skinny_gemm_kernel<RT, CT, WAVES, float, false, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (float*)out, m, n, k);
+      skinny_gemm_kernel<RT, CT, WAVES, float, false, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (float*)out, m, n, k, rs);
     return (int)hipGetLastError();
   }
   if (out_dtype == VELOX_BF16)
-    skinny_gemm_kernel<RT, CT, WAVES, bf16_t><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (bf16_t*)out, m, n, k);
+    skinny_gemm_kernel<RT, CT, WAVES, bf16_t><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (bf16_t*)out, m, n, k, rs);
   else
-    skinny_gemm_kernel<RT, CT, WAVES, float><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (float*)out, m, n, k);
+    skinny_gemm_kernel<RT, CT, WAVES, float><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (float*)out, m, n, k, rs);
   return (int)hipGetLastError();
 }
 
@@ -190,11 +235,14 @@ static int launch_skinny(const void* a, const void* w, const float* bias, void* 
 // caller picks it so that the launch fills the GPU.
 // row_tiles: 16-row tiles of W per wave for M <= 16 (1 or 4).  With 4 a wave reuses each activation fragment for 64 rows
 // of W, which quarters the traffic of the activations; worth it when N is large enough that N / 64 workgroups still fill the GPU.
+// scale_partial (or null), scale_blocks, inv_width, eps: see RowScale; only with M <= 16.
 extern "C" int velox_skinny_gemm_bf16(const void* a, const void* w, const float* bias, void* out, int m, int n, int k, int out_dtype,
-                                      int waves, int row_tiles, int packed, hipStream_t stream) {
+                                      int waves, int row_tiles, int packed, const float* scale_partial, int scale_blocks,
+                                      float inv_width, float eps, hipStream_t stream) {
   if (m <= 0 || n <= 0) return 0;
-  if (k % 64 != 0 || m > 64) return -1;
-#define PICK(RT, CT, W) return launch_skinny<RT, CT, W>(a, w, bias, out, m, n, k, out_dtype, packed != 0, stream)
+  if (k % 64 != 0 || m > 64 || (scale_partial != nullptr && (m > 16 || scale_blocks > ROW_SCALE_BLOCKS))) return -1;
+  const RowScale rs{scale_partial, scale_blocks, inv_width, eps};
+#define PICK(RT, CT, W) return launch_skinny<RT, CT, W>(a, w, bias, out, m, n, k, out_dtype, packed != 0, rs, stream)
   if (m <= 16 && row_tiles >= 4) {
     if (waves >= 8) PICK(4, 1, 8);
     PICK(4, 1, 4);
@@ -236,11 +284,14 @@ struct RotaryWrite {
 
 template <int WAVES>
 __global__ void __launch_bounds__(WAVES * 64) skinny_qkv_rotary_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
-                                                                       RotaryWrite args, int m, int n, int k) {
+                                                                       RotaryWrite args, int m, int n, int k, RowScale rs) {
   __shared__ float4_t partial[WAVES][2][64];
+  __shared__ float scale_table[ROW_SCALE_BLOCKS * 16];
+  row_scale_copy<WAVES>(rs, m, scale_table);
   skinny_partial_sums<2, 1, WAVES, false, true>(a, w, m, n, k, partial);
   const int l = threadIdx.x;
   if (l >= 64) return;
+  const float row_scale = row_scale_of(rs, m, scale_table, l);
   const int row = l & 15;  // batch row
   if (row >= m) return;
   float4_t first = partial[0][0][l], second = partial[0][1][l];
@@ -249,6 +300,8 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_qkv_rotary_kernel(const bf1
     first += partial[wv][0][l];
     second += partial[wv][1][l];
   }
+  first = first * row_scale;
+  second = second * row_scale;
   const int d = args.d, half = d / 2;
   const int pairs_per_head = d / 32;
   const int head = blockIdx.x / pairs_per_head, j = blockIdx.x % pairs_per_head;
@@ -303,39 +356,102 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_qkv_rotary_kernel(const bf1
 }
 
 // a [M, K] (M <= 16), w: packed rows of [Wq; Wk; Wv] in the rotary order; q_out [M, heads * d]; keys and values go to
-// the cache at slots[M].  waves: 8 or 16.
+// the cache at slots[M].  waves: kept for the call's shape; 8 are used.
 extern "C" int velox_skinny_qkv_rotary_bf16(const void* a, const void* w, const float* bias, const int* positions,
                                             const float* cos_table, const float* sin_table, const int* slots, void* q_out,
                                             void* k_cache, void* v_cache, int m, int k, int heads, int kv_heads, int d,
-                                            int page_size, int waves, hipStream_t stream) {
+                                            int page_size, int waves, const float* scale_partial, int scale_blocks, float inv_width,
+                                            float eps, hipStream_t stream) {
   if (m <= 0) return 0;
   if (m > 16 || k % 64 != 0 || d % 32 != 0 || heads < 1 || kv_heads < 1 || page_size < 1) return -1;
+  if (scale_partial != nullptr && scale_blocks > ROW_SCALE_BLOCKS) return -1;
   RotaryWrite args{bias, positions, cos_table, sin_table, slots, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
                    heads, kv_heads, d, page_size};
+  const RowScale rs{scale_partial, scale_blocks, inv_width, eps};
   const int n = (heads + 2 * kv_heads) * d;
   const int blocks = n / 32;
+  (void)waves;  // (16 waves leave 128 registers per lane, which this kernel does not fit without spilling, and measured no faster)
+  skinny_qkv_rotary_kernel<8><<<blocks, 8 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, args, m, n, k, rs);
+  return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The last product of a sub-layer at decode size, with the residual add and the first half of the next norm as its
+// epilogue: residual[M, N] += A W^T (float32, in place; every element belongs to one workgroup), next[M, N] =
+// bfloat16(residual * norm_weight), and sums[m][block] = the sum of squares of the block's 16 new residual values of
+// row m.  Whoever multiplies `next` scales its rows with the sums (RowScale above): the norm costs no kernel.
+// ---------------------------------------------------------------------------------------------------------------
+template <int WAVES>
+__global__ void __launch_bounds__(WAVES * 64) skinny_residual_norm_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
+                                                                          float* __restrict__ residual, const float* __restrict__ norm_weight,
+                                                                          bf16_t* __restrict__ next, float* __restrict__ sums, int m, int n, int k) {
+  __shared__ float4_t partial[WAVES][1][64];
+  // what the epilogue reads is fetched before the main loop (by the 64 threads that will need it)
+  const int l = threadIdx.x;
+  const int row = l & 15;
+  const int col = blockIdx.x * 16 + 4 * (l >> 4);  // first of this lane's four columns
+  float old_residual[4], weight[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const bool inside = l < 64 && row < m && col + j < n;
+    old_residual[j] = inside ? residual[(size_t)row * n + col + j] : 0.f;
+    weight[j] = inside ? norm_weight[col + j] : 0.f;
+  }
+  skinny_partial_sums<1, 1, WAVES, false, true>(a, w, m, n, k, partial);
+  if (l >= 64) return;
+  float4_t sum = partial[0][0][l];
+#pragma unroll
+  for (int wv = 1; wv < WAVES; ++wv) sum += partial[wv][0][l];
+  float squares = 0.f;
+  if (row < m) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (col + j >= n) break;
+      const size_t at = (size_t)row * n + col + j;
+      const float r = old_residual[j] + sum[j];
+      residual[at] = r;
+      next[at] = from_f32<bf16_t>(r * weight[j]);
+      squares += r * r;
+    }
+  }
+  // the four lane groups hold four columns each of the same rows: added in a fixed order
+  squares += __shfl_xor(squares, 16, VELOX_WAVE);
+  squares += __shfl_xor(squares, 32, VELOX_WAVE);
+  if (l < 16) sums[(size_t)l * gridDim.x + blockIdx.x] = squares;
+}
+
+// a [M, K] bfloat16 (M <= 16), w packed [N, K]; sums: float32 [16][ceil(N / 16)].  waves: 4, 8 or 16.
+extern "C" int velox_skinny_residual_norm_bf16(const void* a, const void* w, float* residual, const float* norm_weight, void* next,
+                                               float* sums, int m, int n, int k, int waves, hipStream_t stream) {
+  if (m <= 0 || n <= 0) return 0;
+  if (m > 16 || k % 64 != 0) return -1;
+  const int blocks = (n + 15) / 16;
   if (waves >= 16)
-    skinny_qkv_rotary_kernel<16><<<blocks, 16 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, args, m, n, k);
+    skinny_residual_norm_kernel<16><<<blocks, 16 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, residual, norm_weight, (bf16_t*)next, sums, m, n, k);
+  else if (waves >= 8)
+    skinny_residual_norm_kernel<8><<<blocks, 8 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, residual, norm_weight, (bf16_t*)next, sums, m, n, k);
   else
-    skinny_qkv_rotary_kernel<8><<<blocks, 8 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, args, m, n, k);
+    skinny_residual_norm_kernel<4><<<blocks, 4 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, residual, norm_weight, (bf16_t*)next, sums, m, n, k);
   return (int)hipGetLastError();
 }
 
 // out[M, n] = silu(A Wgate^T) * (A Wup^T) with W = [Wgate; Wup] of 2n rows, bfloat16 in and out, M <= 32.
 // pairs: gate/up tile pairs per wave (1 or 2).
-extern "C" int velox_skinny_gemm_glu_bf16(const void* a, const void* w, void* out, int m, int n, int k, int waves, int pairs, int packed, hipStream_t stream) {
+extern "C" int velox_skinny_gemm_glu_bf16(const void* a, const void* w, void* out, int m, int n, int k, int waves, int pairs, int packed,
+                                          const float* scale_partial, int scale_blocks, float inv_width, float eps, hipStream_t stream) {
   if (m <= 0 || n <= 0) return 0;
-  if (k % 64 != 0 || m > 32) return -1;
+  if (k % 64 != 0 || m > 32 || (scale_partial != nullptr && (m > 16 || scale_blocks > ROW_SCALE_BLOCKS))) return -1;
+  const RowScale rs{scale_partial, scale_blocks, inv_width, eps};
   if (m <= 16) {
     if (pairs >= 2) {
-      if (waves >= 8) return launch_skinny_glu<4, 1, 8>(a, w, out, m, n, k, packed != 0, stream);
-      return launch_skinny_glu<4, 1, 4>(a, w, out, m, n, k, packed != 0, stream);
+      if (waves >= 8) return launch_skinny_glu<4, 1, 8>(a, w, out, m, n, k, packed != 0, rs, stream);
+      return launch_skinny_glu<4, 1, 4>(a, w, out, m, n, k, packed != 0, rs, stream);
     }
-    if (waves >= 8) return launch_skinny_glu<2, 1, 8>(a, w, out, m, n, k, packed != 0, stream);
-    return launch_skinny_glu<2, 1, 4>(a, w, out, m, n, k, packed != 0, stream);
+    if (waves >= 8) return launch_skinny_glu<2, 1, 8>(a, w, out, m, n, k, packed != 0, rs, stream);
+    return launch_skinny_glu<2, 1, 4>(a, w, out, m, n, k, packed != 0, rs, stream);
   }
-  if (waves >= 8) return launch_skinny_glu<2, 2, 8>(a, w, out, m, n, k, packed != 0, stream);
-  return launch_skinny_glu<2, 2, 4>(a, w, out, m, n, k, packed != 0, stream);
+  if (waves >= 8) return launch_skinny_glu<2, 2, 8>(a, w, out, m, n, k, packed != 0, rs, stream);
+  return launch_skinny_glu<2, 2, 4>(a, w, out, m, n, k, packed != 0, rs, stream);
 }
 
 // ---------------------------------------------------------------------------------------------------------------

@@ -19,6 +19,7 @@ from typing import Tuple, Dict, Optional
 
 import torch
 
+from ..parts.base import DeferredNorm, ResidualSink
 from . import build
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
@@ -60,6 +61,7 @@ class HipOps:
         self.use_library_gemm = True
         self.use_skinny_gemm = True
         self.pack_decode_weights = True
+        self.fuse_residual_norm = True
         self._mm_out_dtype_ok: Optional[bool] = None
 
     # -- loading --------------------------------------------------------------------------------
@@ -67,13 +69,15 @@ class HipOps:
         c = self._core
         c.velox_embed.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
         c.velox_add_rmsnorm.argtypes = [_P, _P, _P, _P, _P, _I, _I, _F, _I, _I, _I, ctypes.c_longlong, _P]
-        c.velox_skinny_qkv_rotary_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_skinny_qkv_rotary_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _P]
         c.velox_silu_mul.argtypes = [_P, _P, _I, _I, _I, _P]
         c.velox_rope_kv_write.argtypes = [_P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_gemm_fma.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
-        c.velox_skinny_gemm_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_skinny_gemm_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _P]
+        c.velox_skinny_residual_norm_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]
+        c.velox_row_scale_apply.argtypes = [_P, _P, _I, _F, _F, _P, _I, _I, _P]
         c.velox_skinny_gemm_bf16.restype = _I
-        c.velox_skinny_gemm_glu_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_skinny_gemm_glu_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _P]
         c.velox_skinny_gemm_glu_bf16.restype = _I
         c.velox_skinny_gemm_splitk_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
         c.velox_skinny_gemm_splitk_bf16.restype = _I
@@ -234,9 +238,36 @@ class HipOps:
         return self._norm(residual, delta, rows, weight, eps, out_dtype)
 
     # -- matrix products --------------------------------------------------------------------------
-    def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype, partials_ok: bool = False) -> torch.Tensor:
+    @staticmethod
+    def _scale_args(deferred: Optional[DeferredNorm]):
+        """The four arguments by which a skinny product learns how to scale its result rows."""
+        if deferred is None:
+            return _P(0), 0, 0.0, 0.0
+        return _ptr(deferred.sums), int(deferred.sums.shape[1]), 1.0 / deferred.width, float(deferred.eps)
+
+    def materialize(self, x):
+        """A ``DeferredNorm`` as the plain normalised tensor (one small kernel); anything else is returned as it is."""
+        if not isinstance(x, DeferredNorm):
+            return x
+        m, n = x.x.shape
+        out = torch.empty_like(x.x)
+        sums, blocks, inv_width, eps = self._scale_args(x)
+        self._launched(self._core.velox_row_scale_apply(_ptr(x.x), sums, blocks, inv_width, eps, _ptr(out), m, n, self._stream()), "row_scale_apply")
+        return out
+
+    def linear(self, x, weight: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype, partials_ok: bool = False,
+               residual_norm: Optional[ResidualSink] = None):
         """``x @ weight^T (+ bias)`` as ``[M, N]`` in ``out_dtype``.  With ``partials_ok`` the result may instead come back as
-        float32 partial sums ``[S, M, N]`` that the consumer adds (``add_rmsnorm`` does)."""
+        float32 partial sums ``[S, M, N]`` that the consumer adds (``add_rmsnorm`` does).  With ``residual_norm`` it may
+        come back as a ``DeferredNorm``: the product has then been added to ``residual_norm.residual`` and multiplied
+        with the weight of ``residual_norm.norm`` (decode-sized bfloat16 products whose weight is registered).  ``x`` may
+        be a ``DeferredNorm``."""
+        deferred = x if isinstance(x, DeferredNorm) else None
+        if deferred is not None:
+            x = deferred.x
+            packed = self.packed_weight(weight)
+            if not (self.use_skinny_gemm and packed is not None and x.shape[0] <= 16 and x.shape[1] % 64 == 0 and weight.dtype == torch.bfloat16):
+                x, deferred = self.materialize(deferred), None
         self._check("x", x, align=16)
         self._check("weight", weight, align=16)
         if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
@@ -245,6 +276,12 @@ class HipOps:
         n = weight.shape[0]
         if bias is not None:
             self._check("bias", bias, torch.float32, (n,))
+        if deferred is not None:
+            return self.skinny_gemm(x, weight, bias, out_dtype, packed=self.packed_weight(weight), row_scale=deferred)
+        if residual_norm is not None and bias is None:
+            fused = self._linear_into_residual(x, weight, residual_norm)
+            if fused is not None:
+                return fused
         if (partials_ok and bias is None and self.use_skinny_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
                 and 16 < m <= 64 and k % 64 == 0 and n <= 8192 and n % 4 == 0):
             return self.skinny_gemm_splitk(x, weight)
@@ -263,6 +300,28 @@ class HipOps:
                     self._mm_out_dtype_ok = False
         return self.gemm_fma(x, weight, bias, out_dtype)
 
+    def _linear_into_residual(self, x: torch.Tensor, weight: torch.Tensor, sink: ResidualSink, waves: Optional[int] = None) -> Optional[DeferredNorm]:
+        """``sink.residual += x @ weight^T`` with the first half of ``sink.norm`` in the same kernel, if this product
+        qualifies (bfloat16, at most 16 rows, registered weight, a norm that can be split); None otherwise."""
+        form = sink.norm.deferred_form()
+        packed = self.packed_weight(weight)
+        m, k = x.shape
+        n = weight.shape[0]
+        residual = sink.residual
+        if (not self.use_skinny_gemm or not self.fuse_residual_norm or form is None or packed is None or m > 16 or k % 64 != 0 or n > 16 * 512
+                or x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16):
+            return None
+        norm_weight, eps = form
+        self._check("residual", residual, torch.float32, (m, n), align=16)
+        self._check("norm weight", norm_weight, torch.float32, (n,))
+        blocks = (n + 15) // 16
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=self.device)
+        sums = torch.empty((16, blocks), dtype=torch.float32, device=self.device)
+        status = self._core.velox_skinny_residual_norm_bf16(_ptr(x), _ptr(packed), _ptr(residual), _ptr(norm_weight), _ptr(out), _ptr(sums),
+                                                            m, n, k, int(waves or 8), self._stream())
+        self._launched(status, "skinny_residual_norm")
+        return DeferredNorm(out, sums, n, float(eps), sink.norm)
+
     @staticmethod
     def pack_rows(weight: torch.Tensor, matrices: int = 1) -> torch.Tensor:
         """``weight`` [N, K] bfloat16 (``matrices`` stacked matrices of N / matrices rows each) in the order the skinny
@@ -276,9 +335,11 @@ class HipOps:
         # [matrix, tile, row i, block, group g, 16] -> [matrix, tile, block, g, i, 16]
         return padded.view(matrices, tiles, 16, k // 64, 4, 16).permute(0, 1, 3, 4, 2, 5).contiguous().view(-1)
 
-    def skinny_gemm(self, x, weight, bias, out_dtype, waves: Optional[int] = None, row_tiles: Optional[int] = None, packed: Optional[torch.Tensor] = None, n: Optional[int] = None):
+    def skinny_gemm(self, x, weight, bias, out_dtype, waves: Optional[int] = None, row_tiles: Optional[int] = None, packed: Optional[torch.Tensor] = None, n: Optional[int] = None,
+                    row_scale: Optional[DeferredNorm] = None):
         """Few rows (M <= 64) times a bfloat16 weight: the weight-streaming kernel of the decode step.  ``packed`` is
-        ``pack_rows(weight)``, used instead of ``weight`` when given (``n`` = rows of the weight)."""
+        ``pack_rows(weight)``, used instead of ``weight`` when given (``n`` = rows of the weight).  ``row_scale``: ``x`` is
+        its ``.x`` and the result rows are scaled as it says (M <= 16)."""
         m, k = x.shape
         n = weight.shape[0] if weight is not None else n
         if packed is not None:
@@ -300,19 +361,25 @@ class HipOps:
             wanted = (8 * self.num_cus + blocks - 1) // blocks  # about eight waves per SIMD lane group across the GPU
             waves = 16 if wanted > 8 else 8 if wanted > 4 else 4
         out = torch.empty((m, n), dtype=out_dtype, device=self.device)
-        status = self._core.velox_skinny_gemm_bf16(_ptr(x), _ptr(weight_arg), _ptr(bias), _ptr(out), m, n, k, _code(out_dtype), int(waves), int(row_tiles), 1 if packed is not None else 0, self._stream())
+        if row_scale is not None and m > 16:
+            raise KernelError("skinny_gemm: rows are scaled only for M <= 16")
+        status = self._core.velox_skinny_gemm_bf16(_ptr(x), _ptr(weight_arg), _ptr(bias), _ptr(out), m, n, k, _code(out_dtype), int(waves), int(row_tiles),
+                                                   1 if packed is not None else 0, *self._scale_args(row_scale), self._stream())
         self._launched(status, "skinny_gemm")
         return out
 
     def linear_silu_mul(self, x: torch.Tensor, gate_up_weight: torch.Tensor, out_dtype: torch.dtype, waves: Optional[int] = None, pairs: Optional[int] = None, packed: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``silu(x Wgate^T) * (x Wup^T)`` for ``W = [Wgate; Wup]``.  Decode-sized bfloat16 batches run as one kernel that
         never writes the [M, 2I] product; everything else is the product followed by the SiLU kernel."""
+        deferred = x if isinstance(x, DeferredNorm) else None
+        if deferred is not None:
+            x = deferred.x
         m, k = x.shape
         two_n = gate_up_weight.shape[0]
         fused = (self.use_skinny_gemm and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16 and out_dtype == torch.bfloat16
                  and m <= 16 and k % 64 == 0 and two_n % 2 == 0 and x.dim() == 2 and gate_up_weight.shape[1] == k)
         if not fused:
-            return self.silu_mul(self.linear(x, gate_up_weight, None, out_dtype))
+            return self.silu_mul(self.linear(deferred if deferred is not None else x, gate_up_weight, None, out_dtype))
         if packed is None:
             packed = self.packed_weight(gate_up_weight, 2)
         self._check("x", x, align=16)
@@ -323,7 +390,8 @@ class HipOps:
         if waves is None:
             waves = 8
         out = torch.empty((m, n), dtype=out_dtype, device=self.device)
-        status = self._core.velox_skinny_gemm_glu_bf16(_ptr(x), _ptr(packed if packed is not None else gate_up_weight), _ptr(out), m, n, k, int(waves), int(pairs), 1 if packed is not None else 0, self._stream())
+        status = self._core.velox_skinny_gemm_glu_bf16(_ptr(x), _ptr(packed if packed is not None else gate_up_weight), _ptr(out), m, n, k, int(waves), int(pairs),
+                                                       1 if packed is not None else 0, *self._scale_args(deferred), self._stream())
         self._launched(status, "skinny_gemm_glu")
         return out
 
@@ -395,6 +463,9 @@ class HipOps:
         into the cache.  Returns a tensor whose first ``num_heads * head_dim`` columns are the rotated queries (it may be
         wider).  Decode-sized bfloat16 batches run as one kernel when ``register_weight(weight, rotary_heads=...)`` has
         prepared the weight; everything else is the product followed by ``rope_kv_write``."""
+        deferred = x if isinstance(x, DeferredNorm) else None
+        if deferred is not None:
+            x = deferred.x
         m, k = x.shape
         packed = self.packed_weight(weight, "rotary")
         can_fuse = (self.use_skinny_gemm and packed is not None and write_kv and x.dtype == torch.bfloat16 and m <= 16 and k % 64 == 0
@@ -404,7 +475,7 @@ class HipOps:
         elif fused and not can_fuse:
             raise KernelError("qkv_rope_write: this call cannot run fused")
         if not fused:
-            qkv = self.linear(x, weight, None, x.dtype)
+            qkv = self.linear(deferred if deferred is not None else x, weight, None, x.dtype)
             self.rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size,
                                write_kv=write_kv, bias=bias)
             return qkv
@@ -424,7 +495,7 @@ class HipOps:
         q = torch.empty((m, num_heads * head_dim), dtype=torch.bfloat16, device=self.device)
         status = self._core.velox_skinny_qkv_rotary_bf16(
             _ptr(x), _ptr(packed), _ptr(bias), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping), _ptr(q), _ptr(k_cache),
-            _ptr(v_cache), m, k, num_heads, num_kv_heads, head_dim, block_size, int(waves or 8), self._stream())
+            _ptr(v_cache), m, k, num_heads, num_kv_heads, head_dim, block_size, int(waves or 8), *self._scale_args(deferred), self._stream())
         self._launched(status, "skinny_qkv_rotary")
         return q
 

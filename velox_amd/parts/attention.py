@@ -81,7 +81,10 @@ class AttentionMixer(Mixer):
         ops.register_weight(self.qkv_weight, rotary_heads=(self.num_heads, self.num_kv_heads, self.head_dim) if whole_heads else None)
         ops.register_weight(self.o_weight)
 
-    def forward(self, x, ctx, cache, owns_cache: bool = True):
+    accepts_sink = True  # its last product may add itself to the residual (ResidualSink)
+    accepts_deferred = True  # its first product can read a DeferredNorm
+
+    def forward(self, x, ctx, cache, owns_cache: bool = True, sink=None):
         ops = ctx.ops
         cos, sin = self._rotary_tables()
         meta = cache.batch
@@ -100,7 +103,7 @@ class AttentionMixer(Mixer):
             ctx.max_q_len, meta.max_kv_len, self.scale, self.window,
             ctx.all_decode, ctx.workspace,
         )
-        return ops.linear(attn, self.o_weight, None, ctx.dtype, partials_ok=True)
+        return ops.linear(attn, self.o_weight, None, ctx.dtype, partials_ok=True, residual_norm=sink)
 
 
 register_part("mixer", "attention", AttentionMixer)

@@ -105,6 +105,41 @@ class StateNeed:
     tensors: Tuple[Tuple[str, Tuple[int, ...], Optional[torch.dtype]], ...]
 
 
+@dataclass
+class ResidualSink:
+    """Where a sub-layer's last product may put its result itself: ``residual`` (float32 [T, H]) is what the output is
+    to be added to and ``norm`` the norm that reads the sum next.  A mixer or feed-forward that sets
+    ``accepts_sink = True`` takes ``sink=`` in ``forward`` and hands it to its last ``ops.linear(...,
+    residual_norm=sink)`` (one that sets ``accepts_deferred = True`` is in turn ready to be given a ``DeferredNorm``
+    as its input; others get a plain tensor); what comes back is either the product as always, or, when the kernels could fuse the add and
+    the norm's first half into the product, a ``DeferredNorm`` (the residual is then already updated)."""
+
+    residual: torch.Tensor
+    norm: "Norm"
+
+
+@dataclass
+class DeferredNorm:
+    """Normalised activations that have not been computed as such: ``x`` holds ``residual * weight`` in the run dtype and
+    ``sums`` what is needed for each row's ``rsqrt(mean(residual^2) + eps)``; the products that read them
+    (``ops.linear``, ``ops.linear_silu_mul``, ``ops.qkv_rope_write``) scale their result rows, which is the same thing.
+    ``ops.materialize`` turns it into a plain tensor for anything else."""
+
+    x: torch.Tensor  # [T, H]
+    sums: torch.Tensor  # float32 [16, blocks]: sums of squares of the residual, per row and block of columns
+    width: int
+    eps: float
+    norm: "Norm"  # the norm whose weight is already applied
+
+    @property
+    def shape(self):
+        return self.x.shape
+
+    @property
+    def dtype(self):
+        return self.x.dtype
+
+
 class Mixer(Part):
     def cache_need(self):
         """``PagedNeed``, ``StateNeed`` or None."""
@@ -127,10 +162,16 @@ class FeedForward(Part):
 
 
 class Norm(Part):
+    def deferred_form(self):
+        """``(weight float32 [H], eps)`` if this norm is ``x * rsqrt(mean(x^2) + eps) * weight`` and may therefore be split
+        into a product's epilogue (weight) and the next product's row scale; None otherwise."""
+        return None
+
     def forward(self, residual: torch.Tensor, delta: Optional[torch.Tensor], ctx, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``residual`` [T, H] float32.
 
-        ``delta`` is [T, H] or float32 partial sums [S, T, H], which are added first to last.
+        ``delta`` is [T, H] or float32 partial sums [S, T, H], which are added first to last, or a ``DeferredNorm`` made
+        for this very norm (then the residual is up to date and the ``DeferredNorm`` itself is what comes back).
         With ``rows`` None: ``residual += delta`` in place (delta may be None) and the
         normalised residual comes back in the run dtype, [T, H].  With ``rows`` (int32
         [R]): nothing is changed and ``normalise(residual[rows] + delta[rows])`` comes back.

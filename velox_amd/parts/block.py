@@ -11,7 +11,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from .base import FeedForward, Mixer, Norm, Part
+from .base import FeedForward, Mixer, Norm, Part, ResidualSink
 
 
 class PreNormBlock(Part):
@@ -25,10 +25,21 @@ class PreNormBlock(Part):
     def children(self) -> Tuple[Part, ...]:
         return (self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward)
 
-    def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor], ctx, cache, owns_cache: bool) -> torch.Tensor:
+    def forward(self, residual: torch.Tensor, pending, ctx, cache, owns_cache: bool, next_norm: Optional[Norm] = None):
+        """``next_norm``: the norm that will read this block's output (the next block's first norm), if the caller
+        allows the feed-forward to add its output to the residual itself (see ``ResidualSink``)."""
         normed = self.mixer_norm.forward(residual, pending, ctx)
-        mixed = self.mixer.forward(normed, ctx, cache, owns_cache)
+        if not getattr(self.mixer, "accepts_deferred", False):
+            normed = ctx.ops.materialize(normed)  # (a DeferredNorm becomes a tensor; a tensor stays)
+        if getattr(self.mixer, "accepts_sink", False):
+            mixed = self.mixer.forward(normed, ctx, cache, owns_cache, sink=ResidualSink(residual, self.ff_norm))
+        else:
+            mixed = self.mixer.forward(normed, ctx, cache, owns_cache)
         normed = self.ff_norm.forward(residual, mixed, ctx)
+        if not getattr(self.feed_forward, "accepts_deferred", False):
+            normed = ctx.ops.materialize(normed)
+        if next_norm is not None and getattr(self.feed_forward, "accepts_sink", False):
+            return self.feed_forward.forward(normed, ctx, sink=ResidualSink(residual, next_norm))
         return self.feed_forward.forward(normed, ctx)
 
 

@@ -174,7 +174,10 @@ class DecoderModel(Part):
             entry = self.schedule[index]
             owner = index if entry.cache_from is None else entry.cache_from
             cache = ctx.cache_view(owner)
-            pending = self.blocks[entry.layer].forward(residual, pending, ctx, cache, entry.cache_from is None)
+            # the norm that reads this block's output: the next entry's first norm (the final norm works on chosen rows
+            # and takes its input as it is)
+            following = self.blocks[self.schedule[index + 1].layer].mixer_norm if index + 1 < len(self.schedule) else None
+            pending = self.blocks[entry.layer].forward(residual, pending, ctx, cache, entry.cache_from is None, next_norm=following)
         return pending
 
     def forward(self, token_ids: torch.Tensor, ctx):

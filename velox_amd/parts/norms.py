@@ -12,7 +12,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import Norm, Param, register_part, single
+from .base import DeferredNorm, Norm, Param, register_part, single
 
 
 class RMSNorm(Norm):
@@ -25,7 +25,16 @@ class RMSNorm(Norm):
     def params(self) -> Dict[str, Param]:
         return {"weight": single("weight", (self.hidden_size,), role="vector", init="one_plus_normal")}
 
+    def deferred_form(self):
+        return self.weight, self.eps
+
     def forward(self, residual, delta, ctx, rows=None):
+        if isinstance(delta, DeferredNorm):
+            # the product before this norm has added itself to the residual and applied the weight; the rest of the
+            # norm is a row scale in whatever multiplies next
+            if delta.norm is not self or rows is not None:
+                raise ValueError("a DeferredNorm can only go to the norm it was made for, on all rows")
+            return delta
         if rows is None:
             return ctx.ops.add_rmsnorm(residual, delta, self.weight, self.eps, ctx.dtype)
         return ctx.ops.add_rmsnorm_rows(residual, delta, rows, self.weight, self.eps, ctx.dtype)
