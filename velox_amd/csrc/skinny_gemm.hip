@@ -140,7 +140,7 @@ struct RowScale {
 constexpr int ROW_SCALE_BLOCKS = 512;  // room in LDS: residual widths up to 16 * 512
 
 template <int WAVES>
-__device__ __forceinline__ void row_scale_copy(const RowScale& rs, int m, float (&table)[ROW_SCALE_BLOCKS * 16]) {
+__device__ __forceinline__ void row_scale_copy(const RowScale& rs, int m, float* table) {
   if (rs.partial == nullptr) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int count = rs.blocks * m;  // the rows in use come first
@@ -153,7 +153,7 @@ __device__ __forceinline__ void row_scale_copy(const RowScale& rs, int m, float 
 }
 
 // after the barrier that follows the main loop; every lane of the wave has to call it (l = its lane)
-__device__ __forceinline__ float row_scale_of(const RowScale& rs, int m, const float (&table)[ROW_SCALE_BLOCKS * 16], int l) {
+__device__ __forceinline__ float row_scale_of(const RowScale& rs, int m, const float* table, int l) {
   if (rs.partial == nullptr) return 1.f;
   const int row = l & 15, grp = l >> 4;
   float total = 0.f;
@@ -164,15 +164,16 @@ __device__ __forceinline__ float row_scale_of(const RowScale& rs, int m, const f
   return rsqrtf(total * rs.inv_width + rs.eps);
 }
 
-template <int RT, int CT, int WAVES, typename TO, bool GLU = false, bool PACKED = false>
+// SCALED = true: the instantiation that can scale its rows (it carries the table in LDS); rs.partial is set then.
+template <int RT, int CT, int WAVES, typename TO, bool GLU = false, bool PACKED = false, bool SCALED = false>
 __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
                                                                  const float* __restrict__ bias, TO* __restrict__ out, int m, int n, int k,
                                                                  RowScale rs) {
   __shared__ float4_t partial[WAVES][RT * CT][64];
-  __shared__ float scale_table[ROW_SCALE_BLOCKS * 16];
+  __shared__ float scale_table[SCALED ? ROW_SCALE_BLOCKS * 16 : 1];
   constexpr int RTO = GLU ? RT / 2 : RT;
   const int n0 = blockIdx.x * 16 * RTO;
-  row_scale_copy<WAVES>(rs, m, scale_table);
+  if constexpr (SCALED) row_scale_copy<WAVES>(rs, m, scale_table);
   skinny_partial_sums<RT, CT, WAVES, GLU, PACKED>(a, w, m, n, k, partial);
   // add the waves' partial sums in wave order; each tile's 64 lanes are spread over the workgroup
   for (int item = threadIdx.x; item < RTO * CT * 64; item += WAVES * 64) {
@@ -180,13 +181,16 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
     float4_t sum = partial[0][tile][l];
 #pragma unroll
     for (int wv = 1; wv < WAVES; ++wv) sum += partial[wv][tile][l];
-    const float row_scale = row_scale_of(rs, m, scale_table, l);  // (1 unless the rows of A wait for their norm)
-    sum = sum * row_scale;
+    float row_scale = 1.f;  // (unless the rows of A wait for their norm)
+    if constexpr (SCALED) {
+      row_scale = row_scale_of(rs, m, scale_table, l);
+      sum = sum * row_scale;
+    }
     if constexpr (GLU) {
       float4_t up = partial[0][tile + RTO * CT][l];
 #pragma unroll
       for (int wv = 1; wv < WAVES; ++wv) up += partial[wv][tile + RTO * CT][l];
-      up = up * row_scale;
+      if constexpr (SCALED) up = up * row_scale;
 #pragma unroll
       for (int j = 0; j < 4; ++j) sum[j] = sum[j] / (1.f + expf(-sum[j])) * up[j];
     }
@@ -207,7 +211,14 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
 template <int RT, int CT, int WAVES>
 static int launch_skinny_glu(const void* a, const void* w, void* out, int m, int n, int k, bool packed, RowScale rs, hipStream_t stream) {
   const int blocks = (n + 8 * RT - 1) / (8 * RT);
-  if (packed)
+  if (packed && rs.partial != nullptr) {
+    if constexpr (CT == 1)  // (rows are scaled only for M <= 16)
+      skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true, true, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k, rs);
+    else
+      return -1;
+  } else if (rs.partial != nullptr) {
+    return -1;  // (only the packed weight's kernels scale rows)
+  } else if (packed)
     skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k, rs);
   else
     skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k, rs);
@@ -217,6 +228,17 @@ static int launch_skinny_glu(const void* a, const void* w, void* out, int m, int
 template <int RT, int CT, int WAVES>
 static int launch_skinny(const void* a, const void* w, const float* bias, void* out, int m, int n, int k, int out_dtype, bool packed, RowScale rs, hipStream_t stream) {
   const int blocks = (n + 16 * RT - 1) / (16 * RT);
+  if (rs.partial != nullptr) {
+    if constexpr (CT == 1) {  // (rows are scaled only for M <= 16, and only by the packed weight's kernels)
+      if (!packed) return -1;
+      if (out_dtype == VELOX_BF16)
+        skinny_gemm_kernel<RT, CT, WAVES, bf16_t, false, true, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (bf16_t*)out, m, n, k, rs);
+      else
+        skinny_gemm_kernel<RT, CT, WAVES, float, false, true, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (float*)out, m, n, k, rs);
+      return (int)hipGetLastError();
+    }
+    return -1;
+  }
   if (packed) {
     if (out_dtype == VELOX_BF16)
       skinny_gemm_kernel<RT, CT, WAVES, bf16_t, false, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (bf16_t*)out, m, n, k, rs);

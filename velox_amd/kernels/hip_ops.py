@@ -382,6 +382,8 @@ class HipOps:
             return self.silu_mul(self.linear(deferred if deferred is not None else x, gate_up_weight, None, out_dtype))
         if packed is None:
             packed = self.packed_weight(gate_up_weight, 2)
+        if deferred is not None and packed is None:  # only the kernels of a registered weight scale rows
+            x, deferred = self.materialize(deferred), None
         self._check("x", x, align=16)
         self._check("gate_up_weight", gate_up_weight, align=16)
         n = two_n // 2
