@@ -163,9 +163,10 @@ class HipOps:
         done = 0
         try:
             for n, k in sorted(set(shapes)):
-                weight = torch.zeros((n, k), dtype=torch.bfloat16, device=self.device)
+                # (operands like the real ones: a kernel's time and its clocks depend on the bits it moves)
+                weight = torch.randn((n, k), dtype=torch.float32, device=self.device).mul_(0.02).to(torch.bfloat16)
                 for m in sorted(set(token_counts)):
-                    x = torch.zeros((m, k), dtype=torch.bfloat16, device=self.device)
+                    x = torch.randn((m, k), dtype=torch.float32, device=self.device).to(torch.bfloat16)
                     torch.nn.functional.linear(x, weight)
                     done += 1
                 del weight
