@@ -141,6 +141,39 @@ def test_rope_kv_write(ops, ref, dtype, nh, nkv, d, half, page):
     assert not k_cache.any() and not v_cache.any()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,page", [(28, 4, 128, 16), (4, 2, 16, 8), (3, 1, 32, 32), (6, 2, 48, 4)])
+def test_rope_kv_write_for_consecutive_tokens_of_prompts(ops, ref, dtype, nh, nkv, d, page):
+    """Prompt portions: consecutive tokens in consecutive slots (runs of eight are written as whole vectors), starting
+    anywhere in a page, pages in any order, a single decoded token between two portions."""
+    half = d // 2
+    width = (nh + 2 * nkv) * d
+    pages = 40
+    order = (torch.randperm(pages - 1, generator=torch.Generator().manual_seed(15)) + 1).tolist()
+    slots, positions = [], []
+    for start, count in ((5, 37), (0, 1), (16, 70), (3, 9)):  # (first position, tokens) of each sequence's portion
+        table = [order.pop() for _ in range((start + count + page - 1) // page)]
+        for p in range(start, start + count):
+            slots.append(table[p // page] * page + p % page)
+            positions.append(p)
+    tokens = len(slots)
+    qkv = rand((tokens, width), dtype, 16)
+    bias = rand((width,), torch.float32, 17, 0.1)
+    slots = torch.tensor(slots, dtype=torch.int32).cuda()
+    positions = torch.tensor(positions, dtype=torch.int32).cuda()
+    angles = torch.outer(torch.arange(512, dtype=torch.float32), 1.0 / (10000.0 ** (torch.arange(half, dtype=torch.float32) / half)))
+    cos, sin = angles.cos().cuda(), angles.sin().cuda()
+    results = []
+    for impl in (ops, ref):
+        k_cache = torch.full((pages, nkv, page, d), 3.0, dtype=dtype, device="cuda")
+        v_cache = torch.full((pages, nkv, d, page), 3.0, dtype=dtype, device="cuda")
+        buf = qkv.clone()
+        impl.rope_kv_write(buf, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, write_kv=True, bias=bias)
+        results.append((buf[:, : nh * d].float(), k_cache.float(), v_cache.float()))
+    for got, want in zip(*results):
+        torch.testing.assert_close(got, want, **tol(dtype))
+
+
 @pytest.mark.parametrize("m", [1, 5, 16])
 @pytest.mark.parametrize("nh,nkv,d,k,page", [(4, 2, 64, 128, 4), (28, 4, 128, 3584, 16), (3, 1, 32, 192, 1), (2, 2, 96, 64, 8), (5, 5, 160, 320, 32)])
 def test_qkv_projection_with_rotation_and_cache_write_in_one_kernel(ops, ref, m, nh, nkv, d, k, page):

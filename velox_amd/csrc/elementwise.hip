@@ -311,15 +311,23 @@ __global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, const float* __res
     float4_t hi_v = *reinterpret_cast<const float4_t*>(row + base + half + c0);
     T* lo = reinterpret_cast<T*>(&lo_v);
     T* hi = reinterpret_cast<T*>(&hi_v);
+    // bias and angles of the run, as 16-byte loads (c0 and half are multiples of N, the tables' rows of half)
+    __attribute__((aligned(16))) float b_lo[N], b_hi[N], cos_run[N], sin_run[N];
+#pragma unroll
+    for (int piece = 0; piece < N / 4; ++piece) {
+      const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+      reinterpret_cast<float4_t*>(b_lo)[piece] = bias ? reinterpret_cast<const float4_t*>(bias + base + c0)[piece] : zero;
+      reinterpret_cast<float4_t*>(b_hi)[piece] = bias ? reinterpret_cast<const float4_t*>(bias + base + half + c0)[piece] : zero;
+      reinterpret_cast<float4_t*>(cos_run)[piece] = cs ? reinterpret_cast<const float4_t*>(cs + c0)[piece] : zero;
+      reinterpret_cast<float4_t*>(sin_run)[piece] = sn ? reinterpret_cast<const float4_t*>(sn + c0)[piece] : zero;
+    }
 #pragma unroll
     for (int j = 0; j < N; ++j) {
-      float x0 = to_f32(lo[j]), x1 = to_f32(hi[j]);
-      if (bias) { x0 += bias[base + c0 + j]; x1 += bias[base + half + c0 + j]; }
+      const float x0 = to_f32(lo[j]) + b_lo[j], x1 = to_f32(hi[j]) + b_hi[j];
       float y0 = x0, y1 = x1;
       if (cs) {
-        const float c = cs[c0 + j], s = sn[c0 + j];
-        y0 = x0 * c - x1 * s;
-        y1 = x0 * s + x1 * c;
+        y0 = x0 * cos_run[j] - x1 * sin_run[j];
+        y1 = x0 * sin_run[j] + x1 * cos_run[j];
       }
       lo[j] = from_f32<T>(y0);
       hi[j] = from_f32<T>(y1);
@@ -329,14 +337,39 @@ __global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, const float* __res
     *reinterpret_cast<float4_t*>(dst + half + c0) = hi_v;
   }
   if (write_kv) {
-    // values go to [channel][offset]: neighbouring lanes take neighbouring channels, so that a store instruction
-    // touches as few cache lines as the layout allows
+    // Values go to [channel][offset].  Eight consecutive tokens of a prompt fill eight consecutive offsets of a page:
+    // where this token sits in such a run (slots s .. s + 7 with s a multiple of 8, held by tokens t' .. t' + 7), the
+    // run's first token writes all eight as whole 16- or 32-byte pieces and the other seven write nothing; every
+    // token's workgroup finds the same answer from the slots alone.  (Single 2-byte stores from eight workgroups, on
+    // different parts of the GPU, to one cache line are what made this kernel slow for prompts.)
+    constexpr int RUN = 8;
     const int v_base = (nh + nkv) * d;
-    for (int item = threadIdx.x; item < nkv * d; item += blockDim.x) {
-      const int head = item / d, c = item % d;
-      float x = to_f32(row[v_base + item]);
-      if (bias) x += bias[v_base + item];
-      v_cache[((page * nkv + head) * d + c) * page_size + offset] = from_f32<T>(x);
+    const int lead = t - offset % RUN;  // the token that would hold the run's first slot
+    bool in_run = page_size >= RUN && lead >= 0 && lead + RUN <= (int)gridDim.x;
+    if (in_run) {
+      const int first_slot = slot - offset % RUN;
+      for (int j = 0; j < RUN; ++j) in_run = in_run && slots[lead + j] == first_slot + j;
+    }
+    if (!in_run) {
+      // neighbouring lanes take neighbouring channels, so that a store instruction touches as few cache lines as the layout allows
+      for (int item = threadIdx.x; item < nkv * d; item += blockDim.x) {
+        const int head = item / d, c = item % d;
+        float x = to_f32(row[v_base + item]);
+        if (bias) x += bias[v_base + item];
+        v_cache[((page * nkv + head) * d + c) * page_size + offset] = from_f32<T>(x);
+      }
+    } else if (lead == t) {
+      for (int item = threadIdx.x; item < nkv * d; item += blockDim.x) {
+        const int head = item / d, c = item % d;
+        const float b = bias ? bias[v_base + item] : 0.f;
+        __attribute__((aligned(16))) T run[RUN];
+#pragma unroll
+        for (int j = 0; j < RUN; ++j) run[j] = from_f32<T>(to_f32(qkv[(size_t)(t + j) * width + v_base + item]) + b);
+        T* dst = v_cache + ((page * nkv + head) * d + c) * page_size + offset;
+#pragma unroll
+        for (int piece = 0; piece < (int)(RUN * sizeof(T) / 16); ++piece)
+          reinterpret_cast<float4_t*>(dst)[piece] = reinterpret_cast<const float4_t*>(run)[piece];
+      }
     }
   }
 }
@@ -347,7 +380,7 @@ extern "C" int velox_rope_kv_write(void* qkv, const float* bias, const int* posi
   if (tokens <= 0) return 0;
   const int per = dtype == VELOX_BF16 ? 8 : 4;
   const bool whole_head = (cos_table == nullptr || 2 * half == d) && (d / 2) % per == 0;
-  const bool aligned = (((uintptr_t)qkv | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0;
+  const bool aligned = (((uintptr_t)qkv | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)bias | (uintptr_t)cos_table | (uintptr_t)sin_table) & 15) == 0;
   if (whole_head && aligned) {
     if (dtype == VELOX_BF16)
       rope_kv_write_vec_kernel<bf16_t><<<tokens, 256, 0, stream>>>((bf16_t*)qkv, bias, positions, cos_table, sin_table, slots,
