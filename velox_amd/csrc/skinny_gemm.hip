@@ -509,16 +509,21 @@ __global__ void __launch_bounds__(256) skinny_gemm_splitk_kernel(const bf16_t* _
 
   Run16 w_next[CHUNK];
   float4_t a_next[A_ITERS];
+  // No load sits behind a branch (the compiler would make each wait for the ones before): a block beyond the slice
+  // is read from the slice's last block and its activations are zeroed on their way to LDS; rows beyond N or M are
+  // read from row 0 and their results never stored.
   auto fetch = [&](int kb) {
 #pragma unroll
-    for (int u = 0; u < CHUNK; ++u) w_next[u] = (w_ok && kb + u < kb_hi) ? load_run(w_ptr + (size_t)(kb + u) * 64) : zero_run();
+    for (int u = 0; u < CHUNK; ++u) {
+      const int block = kb + u < kb_hi ? kb + u : kb_hi - 1;
+      w_next[u] = load_run(w_ptr + (size_t)block * 64);
+    }
 #pragma unroll
     for (int it = 0; it < A_ITERS; ++it) {
-      const int v = tid + it * 256;           // vector index: (block u, row r, 16-byte piece p)
+      const int v = tid + it * 256 < A_VECS ? tid + it * 256 : A_VECS - 1;  // vector index: (block u, row r, 16-byte piece p)
       const int u = v / (ROWS * 8), r = (v / 8) % ROWS, p = v % 8;
-      a_next[it] = float4_t{0.f, 0.f, 0.f, 0.f};
-      if (v < A_VECS && r < m && kb + u < kb_hi)
-        a_next[it] = *reinterpret_cast<const float4_t*>(a + (size_t)r * k + (size_t)(kb + u) * 64 + p * 8);
+      const int block = kb + u < kb_hi ? kb + u : kb_hi - 1;
+      a_next[it] = *reinterpret_cast<const float4_t*>(a + (size_t)(r < m ? r : 0) * k + (size_t)block * 64 + p * 8);
     }
   };
 
@@ -530,6 +535,7 @@ __global__ void __launch_bounds__(256) skinny_gemm_splitk_kernel(const bf16_t* _
       const int v = tid + it * 256;
       if (v < A_VECS) {
         const int u = v / (ROWS * 8), r = (v / 8) % ROWS, p = v % 8;
+        if (kb + u >= kb_hi) a_next[it] = float4_t{0.f, 0.f, 0.f, 0.f};  // (only in a slice's last chunk)
         *reinterpret_cast<float4_t*>(a_tile + (u * ROWS + r) * AS + p * 8) = a_next[it];
       }
     }
