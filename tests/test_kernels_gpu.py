@@ -575,7 +575,7 @@ def test_skinny_gemm_with_silu_epilogue(ops, ref, m, inter, k):
     torch.testing.assert_close(ops.linear_silu_mul(big, w, torch.bfloat16).float(), ref.linear_silu_mul(big, w, torch.bfloat16).float(), rtol=3e-2, atol=3e-2 * scale)
 
 
-@pytest.mark.parametrize("m,n,k", [(17, 3584, 18944), (64, 3584, 3584), (33, 100, 640), (64, 4608, 3584), (40, 260, 128)])
+@pytest.mark.parametrize("m,n,k", [(17, 3584, 18944), (64, 3584, 3584), (33, 100, 640), (64, 4608, 3584), (40, 260, 128), (64, 72, 1600)])
 def test_skinny_gemm_splitk_and_norm_that_adds_the_partials(ops, ref, m, n, k):
     x = rand((m, k), torch.bfloat16, 60)
     w = rand((n, k), torch.bfloat16, 61, 0.05)
@@ -585,6 +585,8 @@ def test_skinny_gemm_splitk_and_norm_that_adds_the_partials(ops, ref, m, n, k):
         part = ops.skinny_gemm_splitk(x, w, splits=splits)
         assert part.dim() == 3 and part.shape[1:] == (m, n) and part.dtype == torch.float32
         torch.testing.assert_close(part.sum(0), want, rtol=1e-4, atol=1e-4 * scale)
+        # the weight in the order the lanes read it: the same products in the same order
+        torch.testing.assert_close(ops.skinny_gemm_splitk(x, w, splits=splits, packed=ops.pack_rows(w)), part, rtol=0, atol=0)
     part = ops.skinny_gemm_splitk(x, w)
     if n % 4 == 0:
         residual = rand((m, n), torch.float32, 62)

@@ -480,24 +480,29 @@ extern "C" int velox_skinny_gemm_glu_bf16(const void* a, const void* w, void* ou
 // Split-K variant for 17 .. 64 rows and matrices with few rows of W but a long K (the output and down projections):
 // partial[s, M, N] = A[:, K_s] * W[:, K_s]^T in float32 for each of S slices K_s of K; whoever consumes the result adds the
 // S partial sums (the residual-add + norm kernel does, in a fixed order).  A workgroup owns 64 rows of W (one 16-row
-// tile per wave) and one slice of K.  W streams through registers a chunk (4 blocks of 64 indices) ahead; the
-// activations of a chunk (up to 64 rows x 256 indices) are staged in LDS once per workgroup and read by all four waves.
+// tile per wave) and one slice of K.  W streams through a ring of three register sets, two chunks (of 4 blocks of 64
+// indices) ahead of the arithmetic; the activations of a chunk (up to 64 rows x 256 indices) are asked for one chunk
+// ahead, staged in LDS once per workgroup and read by all four waves.  It runs best with one workgroup per compute
+// unit (the caller picks the number of slices for that).
 // ---------------------------------------------------------------------------------------------------------------
-template <int CT>
+template <int CT, bool PACKED>
 __global__ void __launch_bounds__(256) skinny_gemm_splitk_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
                                                                 float* __restrict__ partial, int m, int n, int k, int blocks_per_split) {
   constexpr int CHUNK = 4;                 // blocks of 64 indices per staging step
   constexpr int ROWS = 16 * CT;            // activation rows held in LDS
   constexpr int AS = 64 + 8;               // row stride of one block of activations, in elements
   constexpr int A_VECS = ROWS * CHUNK * 8; // 16-byte vectors per chunk of activations
-  constexpr int A_ITERS = (A_VECS + 255) / 256;
+  constexpr int A_ITERS = A_VECS / 256;
+  static_assert(A_VECS % 256 == 0, "every thread stages the same number of vectors");
   __shared__ __attribute__((aligned(16))) bf16_t a_tile[CHUNK * ROWS * AS];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 4, i = lane & 15;
   const int row = blockIdx.x * 64 + 16 * wave + i;
-  const bool w_ok = row < n;
-  const bf16_t* w_ptr = w + (size_t)(w_ok ? row : 0) * k + 16 * g;
+  // (rows beyond N: row 0 stands in and nothing is stored; the packed layout pads its last tile with zeros)
+  const bf16_t* w_ptr = PACKED ? w + (size_t)(16 * (blockIdx.x * 4 + wave) < n ? blockIdx.x * 4 + wave : 0) * (k / 64) * 1024 + lane * 16
+                               : w + (size_t)(row < n ? row : 0) * k + 16 * g;
+  constexpr int W_BLOCK = PACKED ? 1024 : 64;  // elements from one block of 64 indices to the next
   const int blocks_total = k / 64;
   const int kb_lo = blockIdx.y * blocks_per_split;
   int kb_hi = kb_lo + blocks_per_split;
@@ -507,43 +512,42 @@ __global__ void __launch_bounds__(256) skinny_gemm_splitk_kernel(const bf16_t* _
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) acc[ct] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  Run16 w_next[CHUNK];
+  // W streams through a ring of three register sets: while a chunk is multiplied the loads of the next two are in
+  // flight.  No load sits behind a branch (the compiler would make each wait for the ones before): a block beyond the
+  // slice is read from the slice's last block and its activations are zeroed on their way to LDS; rows beyond N or M
+  // are read from row 0 and their results never stored.
+  Run16 w_ring[3][CHUNK];
   float4_t a_next[A_ITERS];
-  // No load sits behind a branch (the compiler would make each wait for the ones before): a block beyond the slice
-  // is read from the slice's last block and its activations are zeroed on their way to LDS; rows beyond N or M are
-  // read from row 0 and their results never stored.
-  auto fetch = [&](int kb) {
+  auto fetch_w = [&](int kb, Run16 (&set)[CHUNK]) {
 #pragma unroll
     for (int u = 0; u < CHUNK; ++u) {
       const int block = kb + u < kb_hi ? kb + u : kb_hi - 1;
-      w_next[u] = load_run(w_ptr + (size_t)block * 64);
+      set[u] = load_run(w_ptr + (size_t)block * W_BLOCK);
     }
+  };
+  auto fetch_a = [&](int kb) {
 #pragma unroll
     for (int it = 0; it < A_ITERS; ++it) {
-      const int v = tid + it * 256 < A_VECS ? tid + it * 256 : A_VECS - 1;  // vector index: (block u, row r, 16-byte piece p)
+      const int v = tid + it * 256;  // vector index: (block u, row r, 16-byte piece p)
       const int u = v / (ROWS * 8), r = (v / 8) % ROWS, p = v % 8;
       const int block = kb + u < kb_hi ? kb + u : kb_hi - 1;
       a_next[it] = *reinterpret_cast<const float4_t*>(a + (size_t)(r < m ? r : 0) * k + (size_t)block * 64 + p * 8);
     }
   };
-
-  if (kb_lo < kb_hi) fetch(kb_lo);
-  for (int kb = kb_lo; kb < kb_hi; kb += CHUNK) {
+  // one chunk: its activations go to LDS, the next chunk's activations and the weights two chunks on are asked for
+  // (the activations first: loads come back in order, and they are needed first), then the chunk is multiplied
+  auto step = [&](int kb, Run16 (&w_cur)[CHUNK], Run16 (&w_far)[CHUNK]) {
     __syncthreads();  // the previous chunk has been read by every wave
 #pragma unroll
     for (int it = 0; it < A_ITERS; ++it) {
       const int v = tid + it * 256;
-      if (v < A_VECS) {
-        const int u = v / (ROWS * 8), r = (v / 8) % ROWS, p = v % 8;
-        if (kb + u >= kb_hi) a_next[it] = float4_t{0.f, 0.f, 0.f, 0.f};  // (only in a slice's last chunk)
-        *reinterpret_cast<float4_t*>(a_tile + (u * ROWS + r) * AS + p * 8) = a_next[it];
-      }
+      const int u = v / (ROWS * 8), r = (v / 8) % ROWS, p = v % 8;
+      if (kb + u >= kb_hi) a_next[it] = float4_t{0.f, 0.f, 0.f, 0.f};  // (only in a slice's last chunk)
+      *reinterpret_cast<float4_t*>(a_tile + (u * ROWS + r) * AS + p * 8) = a_next[it];
     }
-    Run16 w_cur[CHUNK];
-#pragma unroll
-    for (int u = 0; u < CHUNK; ++u) w_cur[u] = w_next[u];
     __syncthreads();
-    if (kb + CHUNK < kb_hi) fetch(kb + CHUNK);  // in flight while this chunk is multiplied
+    fetch_a(kb + CHUNK);
+    fetch_w(kb + 2 * CHUNK, w_far);
 #pragma unroll
     for (int u = 0; u < CHUNK; ++u)
 #pragma unroll
@@ -554,6 +558,33 @@ __global__ void __launch_bounds__(256) skinny_gemm_splitk_kernel(const bf16_t* _
         acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[u].lo, lo, acc[ct], 0, 0, 0);
         acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[u].hi, hi, acc[ct], 0, 0, 0);
       }
+  };
+
+  if (kb_lo < kb_hi) {
+    fetch_a(kb_lo);
+    fetch_w(kb_lo, w_ring[0]);
+    fetch_w(kb_lo + CHUNK, w_ring[1]);
+  }
+  for (int kb = kb_lo; kb < kb_hi;) {  // (unrolled by the ring's length: register sets are named at compile time)
+    step(kb, w_ring[0], w_ring[2]);
+    if ((kb += CHUNK) >= kb_hi) break;
+    step(kb, w_ring[1], w_ring[0]);
+    if ((kb += CHUNK) >= kb_hi) break;
+    step(kb, w_ring[2], w_ring[1]);
+    kb += CHUNK;
+  }
+  // Never true.  It keeps what was asked for ahead alive on the way out of the loop: otherwise the compiler moves those
+  // loads behind the loop's exit tests, to the place of their use, where nothing hides their latency any more.
+  if (blocks_per_split < 0) {
+    float4_t keep = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int it = 0; it < A_ITERS; ++it) keep += a_next[it];
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+      for (int u = 0; u < CHUNK; ++u)
+        keep += __builtin_bit_cast(float4_t, w_ring[r][u].lo) + __builtin_bit_cast(float4_t, w_ring[r][u].hi);
+    acc[0] += keep;
   }
   float* dst = partial + (size_t)blockIdx.y * m * n;
   const int col_n = blockIdx.x * 64 + 16 * wave + 4 * g;
@@ -568,15 +599,20 @@ __global__ void __launch_bounds__(256) skinny_gemm_splitk_kernel(const bf16_t* _
 }
 
 // partial: float32 [splits, M, N].  blocks_per_split * splits must cover K / 64.
-extern "C" int velox_skinny_gemm_splitk_bf16(const void* a, const void* w, float* partial, int m, int n, int k, int splits, hipStream_t stream) {
+// packed != 0: w is in the packed layout (see skinny_partial_sums).
+extern "C" int velox_skinny_gemm_splitk_bf16(const void* a, const void* w, float* partial, int m, int n, int k, int splits, int packed, hipStream_t stream) {
   if (m <= 0 || n <= 0) return 0;
   if (k % 64 != 0 || m > 64 || splits < 1) return -1;
   const int blocks_total = k / 64;
   const int per_split = (blocks_total + splits - 1) / splits;
   dim3 grid((n + 63) / 64, splits);
-  if (m <= 32)
-    skinny_gemm_splitk_kernel<2><<<grid, 256, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, partial, m, n, k, per_split);
+  if (m <= 32 && packed)
+    skinny_gemm_splitk_kernel<2, true><<<grid, 256, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, partial, m, n, k, per_split);
+  else if (m <= 32)
+    skinny_gemm_splitk_kernel<2, false><<<grid, 256, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, partial, m, n, k, per_split);
+  else if (packed)
+    skinny_gemm_splitk_kernel<4, true><<<grid, 256, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, partial, m, n, k, per_split);
   else
-    skinny_gemm_splitk_kernel<4><<<grid, 256, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, partial, m, n, k, per_split);
+    skinny_gemm_splitk_kernel<4, false><<<grid, 256, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, partial, m, n, k, per_split);
   return (int)hipGetLastError();
 }

@@ -79,7 +79,7 @@ class HipOps:
         c.velox_skinny_gemm_bf16.restype = _I
         c.velox_skinny_gemm_glu_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _P]
         c.velox_skinny_gemm_glu_bf16.restype = _I
-        c.velox_skinny_gemm_splitk_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
+        c.velox_skinny_gemm_splitk_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P]
         c.velox_skinny_gemm_splitk_bf16.restype = _I
         c.velox_argmax.argtypes = [_P, _P, _P, _I, _I, _I, _P]
         c.velox_sample.argtypes = [_P, _P, _P, _I, _I, _P]
@@ -285,7 +285,7 @@ class HipOps:
                 return fused
         if (partials_ok and bias is None and self.use_skinny_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
                 and 16 < m <= 64 and k % 64 == 0 and n <= 8192 and n % 4 == 0):
-            return self.skinny_gemm_splitk(x, weight)
+            return self.skinny_gemm_splitk(x, weight, packed=self.packed_weight(weight))
         skinny_rows = 16 if n > 8192 else 32  # measured on MI355X: beyond this the library's kernels stream faster
         if self.use_skinny_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and m <= skinny_rows and k % 64 == 0:
             return self.skinny_gemm(x, weight, bias, out_dtype, packed=self.packed_weight(weight))
@@ -398,8 +398,9 @@ class HipOps:
         self._launched(status, "skinny_gemm_glu")
         return out
 
-    def skinny_gemm_splitk(self, x, weight, splits: Optional[int] = None) -> torch.Tensor:
-        """17 .. 64 rows times a bfloat16 weight with few rows and a long K: float32 partial sums ``[S, M, N]``."""
+    def skinny_gemm_splitk(self, x, weight, splits: Optional[int] = None, packed: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """17 .. 64 rows times a bfloat16 weight with few rows and a long K: float32 partial sums ``[S, M, N]``.
+        ``packed``: ``pack_rows(weight)``, read instead of ``weight`` when given."""
         m, k = x.shape
         n = weight.shape[0]
         if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or m > 64 or k % 64 != 0:
@@ -407,12 +408,16 @@ class HipOps:
         self._check("x", x, align=16)
         self._check("weight", weight, align=16)
         if splits is None:
+            # one workgroup per compute unit (measured on MI355X: a unit that gets a second one holds the others up)
             blocks = (n + 63) // 64
-            splits = max(1, min((2 * self.num_cus + blocks - 1) // blocks, k // 512, 16))
+            splits = max(1, min(self.num_cus // blocks, k // 256, 16))
         per_split = (k // 64 + splits - 1) // splits
         splits = (k // 64 + per_split - 1) // per_split  # no empty slice
         out = torch.empty((splits, m, n), dtype=torch.float32, device=self.device)
-        status = self._core.velox_skinny_gemm_splitk_bf16(_ptr(x), _ptr(weight), _ptr(out), m, n, k, splits, self._stream())
+        if packed is not None and (packed.dtype != torch.bfloat16 or packed.numel() != ((n + 15) // 16) * 16 * k):
+            raise KernelError("skinny_gemm_splitk: the packed weight does not match N and K")
+        status = self._core.velox_skinny_gemm_splitk_bf16(_ptr(x), _ptr(weight if packed is None else packed), _ptr(out), m, n, k, splits,
+                                                          int(packed is not None), self._stream())
         self._launched(status, "skinny_gemm_splitk")
         return out
 
