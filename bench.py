@@ -162,7 +162,10 @@ def main() -> int:
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
 
     engine = make_engine(model_config, args.dtype, max(batches), args.context, args.prefill_tokens, graphs)
-    tuned = 0 if args.no_tune else engine.tune_matrix_products([args.prefill_tokens])
+    from velox_amd.engine.runner import decode_buckets
+
+    # the library picks its kernels for the prefill's rows and for the decode batches it serves (graph buckets above 16 rows)
+    tuned = 0 if args.no_tune else engine.tune_matrix_products([args.prefill_tokens] + [b for b in decode_buckets(max(batches)) if b > 16])
     step_s, contexts = {}, {}
     for batch in batches:
         steps = args.steps if batch == args.batch else max(8, args.steps // 2)

@@ -146,6 +146,30 @@ def test_graph_replay_gives_the_eager_logits(tmp_path, name, dtype):
             h.live[rid][1] += 1
 
 
+def test_library_tuning_recaptures_the_decode_graphs_and_keeps_the_logits(tmp_path):
+    """bfloat16: after the matrix library has picked kernels for a decode batch size, the captured steps are captured
+    again (they hold the library's kernels) and generation still agrees with the plain model to rounding."""
+    folder = make_folder(tmp_path, "A", "bfloat16")
+    config, weights = read_model_folder(folder)
+    engine = engine_for(folder, "A", "bfloat16", enable_cuda_graphs=True, max_num_seqs=32, max_num_batched_tokens=64)
+    assert engine.ops.library_serves(128, 64, 64) and not engine.ops.library_serves(8, 1 << 16, 1 << 12)
+    assert not engine.ops.library_serves(32, 256, 64)  # too small for the library's timing to mean anything
+    before = dict(engine.runner._graphs)
+    assert engine.tune_matrix_products([128]) > 0
+    assert all(engine.runner._graphs[b] is before[b] for b in before)  # no captured step has 128 rows
+    engine.ops.library_serves = lambda m, n, k: m > 16  # (tiny weights: pretend they are worth timing)
+    assert engine.tune_matrix_products([32]) > 0
+    assert sorted(engine.runner._graphs) == sorted(before) and all(engine.runner._graphs[b] is not before[b] for b in before)
+    prompts = [random_tokens(config["vocab_size"], 6 + i, seed=70 + i) for i in range(20)]
+    replays = engine.runner.num_graph_replays
+    done = engine.generate(greedy(prompts, 3))
+    assert engine.runner.num_graph_replays > replays
+    for request, prompt in zip(done[:4], prompts):
+        logits = qwen2_logits(config, weights, prompt + request.output_token_ids[:-1])[len(prompt) - 1:]
+        for step, token in enumerate(request.output_token_ids):
+            assert logits[step][token] >= logits[step].max() - 0.05  # the chosen token is the best one up to rounding
+
+
 def test_sampling_through_the_engine(tmp_path):
     folder = make_folder(tmp_path, "B")
     config, _ = read_model_folder(folder)

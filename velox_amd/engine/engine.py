@@ -143,9 +143,11 @@ class Engine:
 
     def tune_matrix_products(self, token_counts: Sequence[int]) -> int:
         """Optional, bfloat16 only: has the matrix library time its candidate kernels for this model's weight shapes at
-        the given numbers of tokens per step (typically the prefill chunk size) and keep the fastest.  Takes seconds
-        per shape; steps with other token counts are unaffected."""
-        if self.dtype != torch.bfloat16 or self.device.type != "cuda":
+        the given numbers of tokens per step (typically the prefill chunk size and the larger decode batch sizes) and
+        keep the fastest.  Takes seconds per shape; steps with other token counts are unaffected.  Only products that
+        the engine hands to the library are timed (``ops.library_serves``); captured decode steps are captured again
+        if one of them holds such a product."""
+        if self.dtype != torch.bfloat16 or self.device.type != "cuda" or not hasattr(self.ops, "tune_library_products"):
             return 0
         shapes = set()
         for part in self.model.all_parts():
@@ -153,8 +155,17 @@ class Engine:
                 tensor = getattr(part, attr, None)
                 if param.role == "matrix" and tensor is not None and tensor.dim() == 2 and tensor.dtype == torch.bfloat16 and attr != "table":
                     shapes.add(tuple(tensor.shape))
-        counts = [m for m in token_counts if m > 64]  # smaller steps run on the engine's own kernels
-        return self.ops.tune_library_products(shapes, counts) if counts else 0
+        done = 0
+        recapture = False
+        for count in sorted(set(int(m) for m in token_counts)):
+            served = [shape for shape in shapes if self.ops.library_serves(count, *shape)]
+            if served:
+                done += self.ops.tune_library_products(served, [count])
+                recapture = recapture or count <= self.config.max_num_seqs
+        if recapture and self.runner.uses_graphs:
+            self.runner.capture_decode_graphs()
+            torch.cuda.synchronize()
+        return done
 
     # -- requests -----------------------------------------------------------------------
     def add_request(self, request: Request) -> None:

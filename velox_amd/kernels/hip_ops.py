@@ -150,6 +150,16 @@ class HipOps:
             return None
         return copies.get(stacked)
 
+    def library_serves(self, m: int, n: int, k: int) -> bool:
+        """Whether ``linear`` hands ``x[m, k] @ w[n, k]^T`` in bfloat16 to the matrix library, and the product is large
+        enough for the library's timing of its candidates to mean something (a weight of a few megabytes is timed
+        from the caches, which says little about a step that streams it from memory)."""
+        if not self.use_library_gemm:
+            return False
+        if m > 64:
+            return True
+        return m > 16 and n > 8192 and n * k >= (32 << 20)
+
     def tune_library_products(self, shapes, token_counts, seconds_per_shape: float = 0.2) -> int:
         """Lets PyTorch's TunableOp time the library's candidate kernels for ``x[M, K] @ w[N, K]^T`` at the given
         ``(N, K)`` shapes and ``M`` values, and keeps its choices for later calls.  Tuning stays off afterwards, so
