@@ -22,6 +22,8 @@
 // The accumulator of a tile is, per lane, rows 4g .. 4g+3 of column i: exactly the Frag of the next
 // product's right operand.  Values are cached transposed inside a page ([channel][offset]) so the
 // V^T tile is filled by contiguous copies.
+#include <type_traits>
+
 #include "common.h"
 
 #ifndef VELOX_HEAD_DIM
@@ -527,22 +529,21 @@ __device__ __forceinline__ void mask_frag(Frag<bf16_t>& f, int valid) {
 // 16-key tiles straight from global memory into MFMA operands (K rows as [key i][channels 16c + 4g ..], V^T rows
 // as [channel 16c + i][keys 4g ..], both 8- or 16-byte loads of contiguous cache lines), two tiles ahead of the
 // arithmetic, with no barrier in the loop.  The page ids of the workgroup's key range are copied into LDS first, so
-// that a tile's addresses do not wait for a second trip to memory.  The 4 waves of a workgroup interleave the
+// that a tile's addresses do not wait for a second trip to memory.  The WAVES waves of a workgroup interleave the
 // tiles of one (sequence, KV head, split) and merge their running (max, sum, output) through LDS at the end.
 constexpr int DECODE_PAGE_IDS = 2048;
 
-template <typename T>
-__global__ void __launch_bounds__(256) decode_attention_kernel(
+template <typename T, int DEPTH, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES) decode_attention_kernel(
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ kv_lens,
     T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
     int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens) {
   constexpr int NC = D / 16;
-  constexpr int NCW = (NC + 3) / 4;
-  constexpr int DEPTH = sizeof(T) * D <= 256 ? 3 : 2;  // register sets: one being computed, the others in flight
-  __shared__ __attribute__((aligned(16))) float4_t acc_all[4 * NC * 64];
-  __shared__ float m_all[4 * 16];
-  __shared__ float l_all[4 * 16];
+  constexpr int NCW = (NC + WAVES - 1) / WAVES;
+  __shared__ __attribute__((aligned(16))) float4_t acc_all[WAVES * NC * 64];
+  __shared__ float m_all[WAVES * 16];
+  __shared__ float l_all[WAVES * 16];
   __shared__ int page_ids[DECODE_PAGE_IDS];
 
   const int tid = threadIdx.x;
@@ -573,13 +574,23 @@ __global__ void __launch_bounds__(256) decode_attention_kernel(
   const int first_page = (n_begin + 16 * t_lo) >> page_shift;
   const int last_key = n_begin + 16 * t_hi < kv_len ? n_begin + 16 * t_hi : kv_len;
   const int num_pages = t_hi > t_lo ? ((last_key - 1) >> page_shift) - first_page + 1 : 0;
-  for (int p = tid; p < num_pages && p < DECODE_PAGE_IDS; p += 256) page_ids[p] = table[first_page + p];
+  {
+    // (each thread's first id without a branch around the load: it is on the way of everything that follows)
+    int at = first_page + (tid < num_pages ? tid : 0);
+    at = at < table_width ? at : table_width - 1;
+    const int id = table[at];
+    if (tid < num_pages) page_ids[tid] = id;
+    for (int p = tid + 64 * WAVES; p < num_pages && p < DECODE_PAGE_IDS; p += 64 * WAVES) page_ids[p] = table[first_page + p];
+  }
 
   Frag<T> qf[NC];
   {
     const T* qp = qkv + (size_t)b * qkv_stride + (size_t)head * D + 4 * g;
 #pragma unroll
-    for (int c = 0; c < NC; ++c) qf[c] = row_ok ? load_frag<T>(qp + 16 * c) : zero_frag<T>();
+    for (int c = 0; c < NC; ++c) {
+      qf[c] = load_frag<T>(qp + 16 * c);
+      if (!row_ok) qf[c] = zero_frag<T>();
+    }
   }
   __syncthreads();
   // (the launcher sends a step here only if a split's keys span at most DECODE_PAGE_IDS pages; the clamp keeps a
@@ -650,21 +661,37 @@ __global__ void __launch_bounds__(256) decode_attention_kernel(
     for (int c = 0; c < NC; ++c) acc_o[c] = mma16(tile.v[c], pf, acc_o[c] * alpha);
   };
 
-  // a ring of DEPTH register sets: while a tile is computed the next two are in flight
+  // A ring of DEPTH register sets: while a tile is computed the next DEPTH - 1 are in flight.  The loop is unrolled by
+  // the ring's length (register sets are named at compile time) and no load sits behind a branch: a tile beyond the
+  // wave's last one is read again from the last one and never used.
   Tile ring[DEPTH];
   const int t0 = t_lo + wave;
+  if (t0 < t_hi) {
+    const int t_last = t0 + (t_hi - 1 - t0) / WAVES * WAVES;  // this wave's last tile
+    auto step = [&](int t, Tile& cur, Tile& far) {
+      const int tn = t + WAVES * (DEPTH - 1);
+      load_tile(far, tn < t_hi ? tn : t_last);
+      compute_tile(cur, t);
+    };
 #pragma unroll
-  for (int s = 0; s < DEPTH - 1; ++s)
-    if (t0 + 4 * s < t_hi) load_tile(ring[s], t0 + 4 * s);
-  for (int t = t0; t < t_hi; t += 4 * DEPTH) {
-#pragma unroll
-    for (int s = 0; s < DEPTH; ++s) {
-      const int tc = t + 4 * s;
-      if (tc < t_hi) {
-        const int tn = tc + 4 * (DEPTH - 1);
-        if (tn < t_hi) load_tile(ring[(s + DEPTH - 1) % DEPTH], tn);
-        compute_tile(ring[s], tc);
+    for (int s = 0; s < DEPTH - 1; ++s) load_tile(ring[s], t0 + WAVES * s < t_hi ? t0 + WAVES * s : t_last);
+    // (set S is computed while set S - 1, the one computed last, is filled again)
+    auto round = [&](auto self, auto set, int& t) {
+      constexpr int S = decltype(set)::value;
+      step(t, ring[S], ring[(S + DEPTH - 1) % DEPTH]);
+      t += WAVES;
+      if constexpr (S + 1 < DEPTH) {
+        if (t < t_hi) self(self, std::integral_constant<int, S + 1>{}, t);
       }
+    };
+    for (int t = t0; t < t_hi;) round(round, std::integral_constant<int, 0>{}, t);
+    // Never true.  It keeps what was asked for ahead alive on the way out of the loop: otherwise the compiler moves
+    // those loads behind the loop's exit tests, to the place of their use, where nothing hides their latency.
+    if (splits < 0) {
+#pragma unroll
+      for (int s = 0; s < DEPTH; ++s)
+#pragma unroll
+        for (int c = 0; c < NC; ++c) acc_o[c] = mma16(ring[s].v[c], ring[s].k[c], acc_o[c]);
     }
   }
 
@@ -676,12 +703,12 @@ __global__ void __launch_bounds__(256) decode_attention_kernel(
   __syncthreads();
   float m_tot = -INFINITY;
 #pragma unroll
-  for (int w = 0; w < 4; ++w) m_tot = fmaxf(m_tot, m_all[w * 16 + i]);
+  for (int w = 0; w < WAVES; ++w) m_tot = fmaxf(m_tot, m_all[w * 16 + i]);
   const float m_ref = (m_tot == -INFINITY) ? 0.f : m_tot;
-  float weight[4];
+  float weight[WAVES];
   float l_tot = 0.f;
 #pragma unroll
-  for (int w = 0; w < 4; ++w) {
+  for (int w = 0; w < WAVES; ++w) {
     const float mw = m_all[w * 16 + i];
     weight[w] = (mw == -INFINITY) ? 0.f : softmax_exp<T>(mw - m_ref);
     l_tot += weight[w] * l_all[w * 16 + i];
@@ -691,11 +718,11 @@ __global__ void __launch_bounds__(256) decode_attention_kernel(
   const size_t slot = ((size_t)split * total_tokens + b) * nh + head;
 #pragma unroll
   for (int cc = 0; cc < NCW; ++cc) {
-    const int c = wave + 4 * cc;  // this wave writes channel blocks wave, wave + 4, ...
+    const int c = wave + WAVES * cc;  // this wave writes channel blocks wave, wave + WAVES, ...
     if (c >= NC) break;
     float4_t sum = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int w = 0; w < 4; ++w) sum += acc_all[(w * NC + c) * 64 + lane] * weight[w];
+    for (int w = 0; w < WAVES; ++w) sum += acc_all[(w * NC + c) * 64 + lane] * weight[w];
     sum = sum * inv;
     if (splits == 1) {
       T* dst = out + ((size_t)b * nh + head) * D + 16 * c + 4 * g;
@@ -757,8 +784,11 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
   const int keys_per_split = (((max_kv_len + 15) / 16 + splits - 1) / splits) * 16;
   const bool ids_fit = (keys_per_split >> page_shift) + 2 <= DECODE_PAGE_IDS;
   if (max_q_len == 1 && total_tokens == num_seqs && group <= 16 && page_shift >= 2 && sizeof(T) * D <= 512 && ids_fit) {
-    // every sequence decodes one token: the streaming kernel
-    decode_attention_kernel<T><<<dim3(splits, nkv, num_seqs), 256, 0, stream>>>(
+    // every sequence decodes one token: the streaming kernel.  Register sets per wave: one being computed, the others
+    // in flight.  (For steps with one workgroup per compute unit, twice as many sets and eight waves per workgroup
+    // were both measured slower on MI355X.)
+    constexpr int DEPTH = sizeof(T) * D <= 256 ? 3 : 2;
+    decode_attention_kernel<T, DEPTH, 4><<<dim3(splits, nkv, num_seqs), 256, 0, stream>>>(
         (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, kv_lens, (T*)out, part_o, part_lse,
         nh, nkv, page_shift, scale, window, splits, total_tokens);
     int status = (int)hipGetLastError();

@@ -519,16 +519,13 @@ class HipOps:
 
     # -- attention ------------------------------------------------------------------------------
     def choose_splits(self, num_seqs: int, num_kv_heads: int, row_tiles: int, max_kv_len: int, all_decode: bool) -> int:
-        """Splits of the key range for an all-decode step (reference ``src/decode_attention.py:237-252``:
-        enough workgroups to fill the GPU, at least 128 keys each)."""
+        """Splits of the key range for an all-decode step (reference ``src/decode_attention.py:237-252``: enough
+        workgroups to fill the GPU).  Measured on MI355X the streaming kernel runs best with one workgroup per compute
+        unit: more of them add partial results to write and merge and gain nothing.  At least 64 keys per split."""
         if not all_decode:
             return 1
         base = num_seqs * num_kv_heads * row_tiles
-        target = 2 * self.num_cus
-        if base >= target or max_kv_len < 256:
-            return 1
-        wanted = (target + base - 1) // base
-        return max(1, min(wanted, 32, max_kv_len // 128))
+        return max(1, min(self.num_cus // max(base, 1), 32, max_kv_len // 64))
 
     def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens,
                         max_q_len, max_kv_len, scale, window, all_decode, workspace, splits: Optional[int] = None):
