@@ -63,7 +63,7 @@ def make_engine(model_config, dtype, batch, context, chunk, graphs, seed=0):
         model_config, seed,
         EngineConfig(dtype=dtype, device="cuda:0", max_model_len=max_len, max_num_seqs=batch,
                      max_num_batched_tokens=max(chunk, batch), max_prefill_chunk_size=chunk, block_size=16,
-                     num_gpu_blocks=pages, enable_cuda_graphs=graphs, seed=seed),
+                     num_gpu_blocks=pages, enable_cuda_graphs=graphs, enable_prefix_caching=False, seed=seed),
         generator_device="cuda",
     )
 

@@ -12,7 +12,8 @@ from velox_amd.engine.request import FinishReason
 
 def engine_for(folder, name, **overrides):
     options = dict(model=folder, dtype="float32", device="cpu", max_model_len=128, max_num_seqs=4, max_num_batched_tokens=32,
-                   max_prefill_chunk_size=7, block_size=PAGE_SIZE[name], num_gpu_blocks=64, enable_cuda_graphs=False, seed=0)
+                   max_prefill_chunk_size=7, block_size=PAGE_SIZE[name], num_gpu_blocks=64, enable_cuda_graphs=False, seed=0,
+                   enable_prefix_caching=False)  # (as in the reference's numerics tests; the prefix cache has tests of its own)
     options.update(overrides)
     return Engine.from_pretrained(EngineConfig(**options), ops=TorchOps())
 

@@ -18,7 +18,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def engine_for(folder, name, dtype="float32", **overrides):
     options = dict(model=folder, dtype=dtype, device="cuda", max_model_len=160, max_num_seqs=4, max_num_batched_tokens=32,
-                   max_prefill_chunk_size=7, block_size=PAGE_SIZE[name], num_gpu_blocks=96, enable_cuda_graphs=False, seed=0)
+                   max_prefill_chunk_size=7, block_size=PAGE_SIZE[name], num_gpu_blocks=96, enable_cuda_graphs=False, seed=0,
+                   enable_prefix_caching=False)  # (as in the reference's numerics tests; the prefix cache has tests of its own)
     options.update(overrides)
     return Engine.from_pretrained(EngineConfig(**options))
 
@@ -168,6 +169,32 @@ def test_library_tuning_recaptures_the_decode_graphs_and_keeps_the_logits(tmp_pa
         logits = qwen2_logits(config, weights, prompt + request.output_token_ids[:-1])[len(prompt) - 1:]
         for step, token in enumerate(request.output_token_ids):
             assert logits[step][token] >= logits[step].max() - 0.05  # the chosen token is the best one up to rounding
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_requests_that_take_over_a_published_prefix(tmp_path, dtype):
+    """Prefix caching on the GPU, with captured decode steps: a request whose prompt begins like an earlier one computes
+    only what follows the shared pages, and its tokens are those of the whole sequence through the plain model."""
+    folder = make_folder(tmp_path, "A", dtype)
+    config, weights = read_model_folder(folder)
+    page = PAGE_SIZE["A"]
+    stem = random_tokens(config["vocab_size"], 4 * page + 3, seed=31)
+    prompts = [stem + random_tokens(config["vocab_size"], n, seed=60 + n) for n in (3, 1, 11, 6)]
+    engine = engine_for(folder, "A", dtype, enable_prefix_caching=True, enable_cuda_graphs=True)
+    assert engine.cache.prefix is not None
+    first = engine.generate(greedy(prompts[:1], 10, prefix="first"))[0]
+    rest = engine.generate(greedy(prompts[1:], 10, prefix="rest"))
+    assert first.num_cached_tokens == 0 and [r.num_cached_tokens for r in rest] == [4 * page] * 3
+    assert engine.runner.num_graph_replays > 0
+    for request, prompt in zip([first] + rest, prompts):
+        logits = qwen2_logits(config, weights, prompt + request.output_token_ids[:-1])[len(prompt) - 1:]
+        for step, token in enumerate(request.output_token_ids):
+            if dtype == "float32":
+                assert int(logits[step].argmax()) == token
+            else:
+                assert logits[step][token] >= logits[step].max() - 0.05  # the best token up to rounding
+    engine.cache.assert_consistent([])
+    assert engine.cache.num_used_pages() == engine.cache.prefix.num_nodes > 0
 
 
 def test_sampling_through_the_engine(tmp_path):

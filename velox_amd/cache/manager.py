@@ -30,6 +30,7 @@ import torch
 
 from ..parts.base import PagedNeed, StateNeed
 from .allocator import NULL_PAGE, OutOfPagesError, PageAllocator
+from .prefix import PrefixCache
 
 
 @dataclass
@@ -40,6 +41,8 @@ class SequenceCache:
     tables: List[List[int]]
     released: List[int]  # per group: number of leading table entries already given back
     version: int = 0  # counts the changes of ``tables``: whoever changes a table in place adds one
+    published: int = 0  # leading pages that are nodes of the prefix cache (matched at admission or published since)
+    publishing: bool = True  # false once another request's page stood where this one's would have gone
 
     def table_arrays(self) -> List[np.ndarray]:
         """The block tables as int32 arrays, converted again only after a change (see ``version``)."""
@@ -151,6 +154,7 @@ class CacheManager:
         device="cpu",
         max_model_len: Optional[int] = None,
         allocate_tensors: bool = True,
+        prefix_caching: bool = False,
     ) -> None:
         if page_size <= 0 or (page_size & (page_size - 1)) != 0:
             raise ValueError(f"page_size must be a power of two, got {page_size}")
@@ -178,6 +182,14 @@ class CacheManager:
         capacity = (num_pages - 1) * page_size
         self.max_model_len = min(max_model_len, capacity) if max_model_len else capacity
         self.max_pages_per_seq = (self.max_model_len + page_size - 1) // page_size
+        # Prefixes are shared only where a request holds every page of its past: no window gives pages back early,
+        # and no state of fixed size stands for tokens that a sharer would skip.
+        self.prefix: Optional[PrefixCache] = None
+        if prefix_caching and self.supports_prefix_caching():
+            self.prefix = PrefixCache([group.allocator for group in self.groups], page_size)
+
+    def supports_prefix_caching(self) -> bool:
+        return bool(self.groups) and not self.state_entries and all(group.need.window is None for group in self.groups)
 
     # -- sizes --------------------------------------------------------------------------
     def bytes_per_page(self) -> int:
@@ -188,8 +200,17 @@ class CacheManager:
         return min((g.allocator.num_total for g in self.groups), default=0)
 
     def num_free_pages(self) -> int:
-        """Free pages of the tightest group (what bounds growth)."""
+        """Free pages of the tightest group."""
         return min((g.allocator.num_free for g in self.groups), default=1 << 30)
+
+    def num_reclaimable_pages(self) -> int:
+        """Pages (per group) that only the prefix cache holds: they are given back when a request needs them."""
+        return self.prefix.num_reclaimable if self.prefix is not None else 0
+
+    def num_available_pages(self) -> int:
+        """Free plus reclaimable pages of the tightest group: what bounds growth (reference
+        ``src/block_manager.py:34-35``)."""
+        return self.num_free_pages() + self.num_reclaimable_pages()
 
     def num_used_pages(self) -> int:
         return max((g.allocator.num_used for g in self.groups), default=0)
@@ -211,15 +232,18 @@ class CacheManager:
         if num_computed + num_new > self.max_model_len:
             return False
         extra = self.pages_to_append(seq, num_computed, num_new)
-        return all(n <= g.allocator.num_free for n, g in zip(extra, self.groups))
+        reclaimable = self.num_reclaimable_pages()
+        return all(n <= g.allocator.num_free + reclaimable for n, g in zip(extra, self.groups))
 
     def max_new_tokens(self, seq: Optional[SequenceCache], num_computed: int, headroom_pages: Optional[int] = None) -> int:
         """How many tokens past ``num_computed`` fit in the pages the request has plus the free ones
         (less ``headroom_pages`` held back), capped by ``max_model_len`` (reference ``engine/scheduler.py:210-219``)."""
         limit = self.max_model_len - num_computed
+        reclaimable = self.num_reclaimable_pages()
         for index, group in enumerate(self.groups):
             have = len(seq.tables[index]) if seq is not None else 0
-            free = group.allocator.num_free if headroom_pages is None else min(group.allocator.num_free, headroom_pages)
+            free = group.allocator.num_free + reclaimable
+            free = free if headroom_pages is None else min(free, headroom_pages)
             pages = min(have + max(0, free), self.max_pages_per_seq)
             limit = min(limit, pages * group.page_size - num_computed)
         return max(0, limit)
@@ -229,14 +253,48 @@ class CacheManager:
         if num_computed + num_new > self.max_model_len:
             return False
         extra = self.pages_to_append(seq, num_computed, num_new)
+        reclaimable = self.num_reclaimable_pages()
         for n, group, table in zip(extra, self.groups, seq.tables):
-            if n > group.allocator.num_free or len(table) + n > self.max_pages_per_seq:
+            if n > group.allocator.num_free + reclaimable or len(table) + n > self.max_pages_per_seq:
+                return False
+        short = max((n - group.allocator.num_free for n, group in zip(extra, self.groups)), default=0)
+        if short > 0:
+            self.prefix.evict(short)  # (an evicted node gives back one page in every group)
+            if any(n > group.allocator.num_free for n, group in zip(extra, self.groups)):
                 return False
         for n, group, table in zip(extra, self.groups, seq.tables):
             if n:
                 table.extend(group.allocator.allocate_many(n))
                 seq.version += 1
         return True
+
+    # -- shared prefixes -----------------------------------------------------------------------
+    def match_prefix(self, seq: SequenceCache, tokens: Sequence[int]) -> int:
+        """For a request that holds nothing yet: puts the published pages of the longest known prefix of ``tokens``
+        into its tables and returns how many tokens they cover.  At least one token is left to compute, so that there
+        is a row to take logits from (reference ``src/block_manager.py:52-72``)."""
+        if self.prefix is None or any(seq.tables):
+            return 0
+        nodes = self.prefix.match(tokens, max_pages=min((len(tokens) - 1) // self.page_size, self.max_pages_per_seq))
+        for node in nodes:
+            for index, (group, page) in enumerate(zip(self.groups, node.pages)):
+                group.allocator.incref(page)
+                seq.tables[index].append(page)
+            self.prefix.page_taken(node.pages[0])
+        if nodes:
+            seq.version += 1
+        seq.published = len(nodes)
+        seq.publishing = True
+        return len(nodes) * self.page_size
+
+    def publish(self, seq: SequenceCache, tokens: Sequence[int], num_computed: int) -> None:
+        """Offers the pages that the request has filled since the last call to later requests (reference
+        ``src/block_manager.py:101-112``).  ``tokens[:num_computed]`` are in the cache."""
+        if self.prefix is None or not seq.publishing:
+            return
+        whole = min(num_computed // self.page_size, min(len(table) for table in seq.tables))
+        if whole > seq.published:
+            seq.published, seq.publishing = self.prefix.publish(tokens, seq.tables, seq.published, whole)
 
     def release_behind_window(self, seq: SequenceCache, num_computed: int) -> int:
         """Gives back pages no later query can read; their table entries become the null page."""
@@ -254,12 +312,17 @@ class CacheManager:
         return given_back
 
     def free_pages(self, seq: SequenceCache) -> None:
-        for index, group in enumerate(self.groups):
-            for page in seq.tables[index]:
+        for index in range(len(self.groups) - 1, -1, -1):  # (group 0 last: its count tells the prefix cache who holds a node)
+            group = self.groups[index]
+            for page in seq.tables[index]:  # (in table order, so that the request's last page is the next one handed out)
                 if page != NULL_PAGE:
                     group.allocator.free(page)
+                    if index == 0 and self.prefix is not None:
+                        self.prefix.page_dropped(page)
             seq.tables[index] = []
             seq.released[index] = 0
+        seq.published = 0
+        seq.publishing = True
         seq.version += 1
 
     def free_sequence(self, seq: SequenceCache) -> None:
@@ -296,18 +359,31 @@ class CacheManager:
 
     # -- invariants ---------------------------------------------------------------------
     def assert_consistent(self, live: Sequence[SequenceCache] = ()) -> None:
-        """Allocator invariants, and: the pages the live requests hold are exactly the used ones, each held once."""
+        """Allocator invariants, and: every used page is held by the live requests that list it and, if published, once
+        more by the prefix cache; no request lists a page twice; no page is lost."""
         self.state.assert_consistent()
+        if self.prefix is not None:
+            self.prefix.assert_consistent()
         for index, group in enumerate(self.groups):
             group.allocator.assert_consistent()
-            held: List[int] = [p for seq in live for p in seq.tables[index] if p != NULL_PAGE]
-            if len(set(held)) != len(held):
+            holders: Dict[int, int] = {}
+            for seq in live:
+                pages = [p for p in seq.tables[index] if p != NULL_PAGE]
+                if len(set(pages)) != len(pages):
+                    raise AssertionError(f"group {index}: a request lists a page twice")
+                for page in pages:
+                    holders[page] = holders.get(page, 0) + 1
+            published = set()
+            if self.prefix is not None:
+                published = {node.pages[index] for node in self.prefix._node_of.values()}
+            if self.prefix is None and any(count != 1 for count in holders.values()):
                 raise AssertionError(f"group {index}: a page is held twice")
-            for page in held:
-                if group.allocator.ref_count(page) != 1:
-                    raise AssertionError(f"group {index}: held page {page} has refcount {group.allocator.ref_count(page)}")
-            if live is not None and len(held) != group.allocator.num_used:
-                raise AssertionError(f"group {index}: {group.allocator.num_used} pages used but {len(held)} held (a page was lost)")
+            for page in set(holders) | published:
+                expected = holders.get(page, 0) + (page in published)
+                if group.allocator.ref_count(page) != expected:
+                    raise AssertionError(f"group {index}: page {page} has refcount {group.allocator.ref_count(page)}, expected {expected}")
+            if live is not None and len(set(holders) | published) != group.allocator.num_used:
+                raise AssertionError(f"group {index}: {group.allocator.num_used} pages used but {len(set(holders) | published)} accounted for (a page was lost)")
 
 
 def pages_that_fit(bytes_per_page: int, free_bytes: int, utilization: float, reserve_bytes: int) -> int:

@@ -51,7 +51,9 @@ class EngineConfig:
     gpu_memory_utilization: float = 0.90
     kv_cache_reserve_mb: int = 512
 
-    enable_prefix_caching: bool = False
+    # pages of a prompt prefix that an earlier request has computed are taken over instead of computed again (on by
+    # default as in the reference; models whose layers keep a window or a state of fixed size run without it)
+    enable_prefix_caching: bool = True
     enable_cuda_graphs: bool = True
     # a second copy of every bfloat16 weight in the order the decode kernels read it: faster decoding for the
     # weights' size again in memory (not a reference option)
@@ -79,5 +81,3 @@ class EngineConfig:
             raise ValueError("block_size must be a power of two")
         if self.max_prefill_chunk_size < 1 or self.max_model_len < 2:
             raise ValueError("max_prefill_chunk_size must be at least 1 and max_model_len at least 2")
-        if self.enable_prefix_caching:
-            raise ValueError("prefix caching is not implemented; leave enable_prefix_caching off")

@@ -130,7 +130,8 @@ class Engine:
             num_pages = pages_that_fit(probe.bytes_per_page(), free_bytes, config.gpu_memory_utilization, config.kv_cache_reserve_mb * 1024 * 1024)
             wanted = (config.max_num_seqs * max_model_len + config.block_size - 1) // config.block_size + 1
             num_pages = min(num_pages, max(2, wanted))
-        cache = CacheManager(needs, config.block_size, num_pages, config.max_num_seqs, dtype, device, max_model_len=max_model_len)
+        cache = CacheManager(needs, config.block_size, num_pages, config.max_num_seqs, dtype, device, max_model_len=max_model_len,
+                             prefix_caching=config.enable_prefix_caching)
         engine = cls(model, cache, config, ops, eos_token_ids=eos)
         engine.warmup()
         return engine

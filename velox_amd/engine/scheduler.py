@@ -179,7 +179,8 @@ class Scheduler:
                 return None
             for index, pages in enumerate(self.cache.pages_to_append(request.cache, after, 1)):
                 needed[index] += pages
-        if any(n > group.allocator.num_free for n, group in zip(needed, self.cache.groups)):
+        reclaimable = self.cache.num_reclaimable_pages()
+        if any(n > group.allocator.num_free + reclaimable for n, group in zip(needed, self.cache.groups)):
             return None
         for request in in_flight:
             if not self.cache.append(request.cache, request.num_computed_tokens + 1, 1):
@@ -241,15 +242,18 @@ class Scheduler:
             sequence = self.cache.new_sequence()
             if sequence is None:
                 break
-            wanted = min(request.num_uncomputed_tokens, budget, self.config.max_prefill_chunk_size)
-            headroom = self.cache.num_free_pages() - self._watermark_pages
-            chunk = min(wanted, self.cache.max_new_tokens(sequence, 0, headroom_pages=headroom))
-            if chunk <= 0 or not self.cache.append(sequence, 0, chunk):
+            # pages of a prefix that an earlier request has published are taken over, not computed (reference :268-277)
+            cached = self.cache.match_prefix(sequence, request.all_token_ids)
+            wanted = min(len(request.all_token_ids) - cached, budget, self.config.max_prefill_chunk_size)
+            headroom = self.cache.num_available_pages() - self._watermark_pages
+            chunk = min(wanted, self.cache.max_new_tokens(sequence, cached, headroom_pages=headroom))
+            if chunk <= 0 or not self.cache.append(sequence, cached, chunk):
                 self.cache.free_sequence(sequence)
                 break
             self.waiting.popleft()
             request.cache = sequence
-            request.num_computed_tokens = 0
+            request.num_computed_tokens = cached
+            request.num_cached_tokens = cached
             request.status = RequestStatus.RUNNING_PREFILL
             request.current_chunk_size = chunk
             self.running.append(request)
@@ -262,6 +266,7 @@ class Scheduler:
         request.num_computed_tokens += num_tokens
         if request.cache is not None:
             self.cache.release_behind_window(request.cache, request.num_computed_tokens)
+            self.cache.publish(request.cache, request.all_token_ids, request.num_computed_tokens)
 
     def stats(self) -> Dict[str, float]:
         total = self.cache.num_total_pages
@@ -273,6 +278,8 @@ class Scheduler:
             "num_finished": float(self.num_finished),
             "total_blocks": float(total),
             "free_blocks": float(self.cache.num_free_pages()),
+            "evictable_blocks": float(self.cache.num_reclaimable_pages()),
+            "prefix_hit_rate": 0.0 if self.cache.prefix is None else self.cache.prefix.hit_rate,
             "used_blocks": float(used),
             "usage": 0.0 if total == 0 else used / total,
         }
