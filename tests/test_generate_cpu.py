@@ -152,3 +152,48 @@ def test_abort_while_a_step_is_in_flight(tmp_path):
     assert drop.finish_reason is FinishReason.ABORT and len(drop.output_token_ids) < 12
     assert engine.cache.num_used_pages() == 0
     engine.cache.assert_consistent([])
+
+
+def test_requests_and_aborts_from_another_thread(tmp_path):
+    """``submit`` and ``request_abort`` may be called from any thread; the stepping thread takes them in at the start of
+    its next step (reference ``engine/engine.py:239-263``)."""
+    import threading
+
+    folder = make_folder(tmp_path, "A")
+    config, weights = read_model_folder(folder)
+    prompts = [random_tokens(config["vocab_size"], n, seed=120 + n) for n in (5, 8, 11)]
+    engine = engine_for(folder, "A")
+    first, second, dropped = greedy(prompts, 10)
+    engine.add_request(first)
+    for _ in range(3):
+        engine.step()
+
+    def client():
+        engine.submit(second)
+        engine.submit(dropped)
+        with pytest.raises(ValueError):
+            engine.submit(Request("too-long", [1] * engine.max_model_len, SamplingParams(max_tokens=1)))
+
+    thread = threading.Thread(target=client)
+    thread.start()
+    thread.join()
+    assert engine.has_work() and second.request_id not in engine.scheduler.requests  # not taken in before a step begins
+    engine.step()
+    assert second.request_id in engine.scheduler.requests and dropped.request_id in engine.scheduler.requests
+    aborter = threading.Thread(target=lambda: engine.request_abort(dropped.request_id))
+    aborter.start()
+    aborter.join()
+    while engine.has_work():
+        engine.step()
+    assert first.output_token_ids == plain_greedy(config, weights, prompts[0], 10)
+    assert second.output_token_ids == plain_greedy(config, weights, prompts[1], 10)
+    assert dropped.finish_reason is FinishReason.ABORT and len(dropped.output_token_ids) < 10
+    # a request id that is queued twice is refused when it is taken in, not in the submitting thread
+    again = greedy(prompts[:1], 2)[0]
+    twin = greedy(prompts[:1], 2)[0]
+    engine.submit(again)
+    engine.submit(twin)
+    engine.step()
+    assert twin.finish_reason is FinishReason.ABORT and not again.finished
+    assert engine.abort_all() == "aborted" and not engine.has_work()
+    assert engine.cache.num_used_pages() == 0

@@ -10,6 +10,8 @@ step function.  The one host wait per step is the read of the sampled tokens
 """
 from __future__ import annotations
 
+import logging
+import queue
 import time
 from dataclasses import dataclass
 from typing import Dict, FrozenSet, Iterable, List, Optional, Sequence
@@ -39,6 +41,8 @@ class _Flight:
     tokens: Optional[torch.Tensor]  # int32 [len(sampled)] on the device
     landing: Optional[tuple] = None  # (pinned host tensor the tokens are copied to, event recorded behind the copy)
 
+
+logger = logging.getLogger(__name__)
 
 _STAGES = ("scheduler_ms", "prepare_ms", "forward_ms", "sampling_ms", "cpu_sync_wait_ms", "step_ms")
 
@@ -79,6 +83,9 @@ class Engine:
         self.stats: Dict[str, List[float]] = {name: [] for name in _STAGES}
         self.num_steps = 0
         self._ahead: Optional[_Flight] = None
+        # requests and aborts handed over by other threads, taken in at the start of the next step
+        self._pending_adds: "queue.Queue[Request]" = queue.Queue()
+        self._pending_aborts: "queue.Queue[str]" = queue.Queue()
         self._landings = []
         self._next_landing = 0
         if self.device.type == "cuda":
@@ -179,8 +186,51 @@ class Engine:
         self.sampler.release(request_id)
         return self.scheduler.abort_request(request_id)
 
+    def abort_all(self) -> str:
+        self._drain_control_queue()
+        for request_id in list(self.scheduler.requests):
+            self.abort_request(request_id)
+        return "aborted"
+
+    def check_limits(self, num_prompt_tokens: int, max_tokens: int) -> None:
+        """Raises ValueError for a request that ``add_request`` would refuse for its length (reference ``:226-237``)."""
+        limit = self.max_model_len
+        if num_prompt_tokens >= limit:
+            raise ValueError(f"prompt of {num_prompt_tokens} tokens does not fit in max_model_len={limit} "
+                             "(at least one token must remain for generation)")
+        if num_prompt_tokens + max_tokens > limit:
+            raise ValueError(f"prompt of {num_prompt_tokens} tokens plus max_tokens={max_tokens} exceeds max_model_len={limit}")
+
+    def submit(self, request: Request) -> None:
+        """``add_request`` for other threads than the one that steps: the request is taken in when the next step begins
+        (reference ``:239-263``).  Its length is checked here, in the caller's thread."""
+        self.check_limits(request.num_prompt_tokens, request.sampling_params.max_tokens)
+        self._pending_adds.put(request)
+
+    def request_abort(self, request_id: str) -> None:
+        """``abort_request`` for other threads: carried out when the next step begins."""
+        self._pending_aborts.put(request_id)
+
+    def _drain_control_queue(self) -> None:
+        while True:
+            try:
+                request = self._pending_adds.get_nowait()
+            except queue.Empty:
+                break
+            try:
+                self.add_request(request)
+            except ValueError:
+                logger.exception("rejecting request %s", request.request_id)
+                request.finish(FinishReason.ABORT)
+        while True:
+            try:
+                request_id = self._pending_aborts.get_nowait()
+            except queue.Empty:
+                break
+            self.abort_request(request_id)
+
     def has_work(self) -> bool:
-        return self.scheduler.has_work()
+        return self.scheduler.has_work() or not self._pending_adds.empty()
 
     # -- one step -----------------------------------------------------------------------
     @torch.no_grad()
@@ -192,6 +242,7 @@ class Engine:
         tokens.  The device so never waits for the host between decode steps.  A request that stops on a token that
         was still in flight has a row in the successor that nobody reads."""
         step_start = time.perf_counter()
+        self._drain_control_queue()
         flight, self._ahead = self._ahead, None
         if flight is not None and not any(self._alive(r) for r in flight.sampled):
             flight = None  # launched for requests that have all stopped or been aborted since
