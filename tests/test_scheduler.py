@@ -277,3 +277,19 @@ def test_nothing_is_fixed_ahead_when_the_next_step_could_look_different():
         tables = [list(r.cache.tables[0]) for r in requests]
         assert s.schedule_ahead(out.decode_batch) is None
         assert s.cache.groups[0].allocator.num_free == free_before and [list(r.cache.tables[0]) for r in requests] == tables
+
+
+def test_listeners_hear_tokens_and_the_end_and_may_fail():
+    from velox_amd.engine.request import RequestEvent
+
+    r = request("r", 3, max_tokens=2)
+    heard = []
+    r.add_listener(lambda req, event: heard.append((req.request_id, event)))
+    r.add_listener(lambda req, event: 1 / 0)  # a failing listener is logged, the request goes on
+    r.append_token(7)
+    r.append_token(8)
+    assert r.num_output_tokens == 2 and r.max_tokens == 2 and r.tokens_for_chunk(2) == [1, 2]
+    r.finish(r.should_stop(8, frozenset()))
+    r.finish(FinishReason.ABORT)  # the second end is not heard
+    assert heard == [("r", RequestEvent("token", token_id=7)), ("r", RequestEvent("token", token_id=8)),
+                     ("r", RequestEvent("finish", finish_reason=FinishReason.LENGTH))]
