@@ -93,12 +93,13 @@ def run_workload(engine, prompts, sampling, label: str) -> Dict:
     itl = [(b - a) * 1000 for times in token_times.values() for a, b in zip(times, times[1:])]
     generated = sum(len(r.output_token_ids) for r in requests)
     prompt_tokens = sum(len(p) for p in prompts)
+    cached_tokens = sum(r.num_cached_tokens for r in requests)  # (of a preempted request: at its last admission)
     return {
         "label": label, "wall_seconds": wall, "num_requests": len(requests), "prompt_tokens": prompt_tokens,
         "generated_tokens": generated, "decode_throughput": generated / wall if wall else 0.0,
         "total_throughput": (prompt_tokens + generated) / wall if wall else 0.0,
         "ttft": summarise(ttft), "itl_ms": summarise(itl), "steps": engine.num_steps,
-        "preemptions": engine.scheduler.num_preemptions,
+        "preemptions": engine.scheduler.num_preemptions, "cached_prompt_tokens": cached_tokens,
         "max_running": max((entry[0] for entry in log), default=0), "max_blocks_used": max((entry[2] for entry in log), default=0),
         "outputs": {r.request_id: r.output_token_ids for r in requests},
     }
@@ -118,6 +119,8 @@ def report(result: Dict, engine, show_outputs: bool) -> None:
     print(f"  Peak running requests : {result['max_running']}")
     print(f"  Peak KV blocks in use : {result['max_blocks_used']}")
     print(f"  Preemptions           : {result['preemptions']}")
+    share = 100.0 * result['cached_prompt_tokens'] / max(1, result['prompt_tokens'])
+    print(f"  Prompt tokens cached  : {result['cached_prompt_tokens']} ({share:.1f}%, prefix caching {'on' if engine.cache.prefix is not None else 'off'})")
     ttft, itl = result["ttft"], result["itl_ms"]
     print(f"\n  TTFT (s)   mean={ttft['mean']:.3f}  p50={ttft['p50']:.3f}  p90={ttft['p90']:.3f}  p99={ttft['p99']:.3f}  max={ttft['max']:.3f}")
     print(f"  ITL (ms)   mean={itl['mean']:.2f}  p50={itl['p50']:.2f}  p90={itl['p90']:.2f}  p99={itl['p99']:.2f}  max={itl['max']:.2f}")
