@@ -50,13 +50,16 @@ def rule(title: str = "") -> None:
 SHARED_PREFIX_TOKENS = 96  # stands in for the reference's shared system prompt (``benchmark.py:42-47``, about 90 tokens)
 
 
-def build_prompts(workload: str, count: int, vocab: int, limit: int, fixed_len: Optional[int], seed: int, shared_prefix: bool = False) -> List[List[int]]:
+def build_prompts(workload: str, count: int, vocab: int, limit: int, fixed_len: Optional[int], seed: int, shared_prefix: bool = False,
+                  length_range: Optional[tuple] = None) -> List[List[int]]:
     rng = random.Random(seed)
     prefix = [rng.randrange(vocab) for _ in range(min(SHARED_PREFIX_TOKENS, max(0, limit - 1)))] if shared_prefix else []
     prompts = []
     for index in range(count):
         if fixed_len:
             length = fixed_len
+        elif length_range:
+            length = rng.randint(*length_range)
         else:
             kind = workload if workload != "mixed" else ("short", "long")[index % 2]
             lo, hi = WORKLOAD_LENGTHS[kind]
@@ -146,6 +149,7 @@ def parse_args(argv=None) -> argparse.Namespace:
     parser.add_argument("--dtype", default="auto")
     parser.add_argument("--workload", default="mixed", choices=["short", "long", "mixed"])
     parser.add_argument("--prompt-len", type=int, default=None, help="every prompt has this many tokens (overrides --workload)")
+    parser.add_argument("--prompt-len-range", default=None, metavar="LO,HI", help="prompt lengths uniform in [LO, HI] (overrides --workload)")
     parser.add_argument("--num-requests", type=int, default=16)
     parser.add_argument("--max-tokens", type=int, default=128)
     parser.add_argument("--temperature", type=float, default=0.0)
@@ -160,6 +164,8 @@ def parse_args(argv=None) -> argparse.Namespace:
     parser.add_argument("--no-prefix-caching", action="store_true", help="compute every prompt in full (no sharing of prompt prefixes between requests)")
     parser.add_argument("--no-cuda-graphs", "--no-hip-graphs", dest="no_graphs", action="store_true")
     parser.add_argument("--shared-system-prompt", action="store_true", help="every prompt starts with the same %d tokens" % SHARED_PREFIX_TOKENS)
+    parser.add_argument("--tune-library", action="store_true",
+                        help="let the matrix library time its kernels for the prefill chunk size and the larger decode batches first (bfloat16; takes seconds per shape)")
     parser.add_argument("--sweep-batch-size", default=None, help="comma-separated max_num_seqs values to sweep")
     parser.add_argument("--rounds", type=int, default=1, help="replay the workload N times")
     parser.add_argument("--show-outputs", action="store_true")
@@ -198,11 +204,16 @@ def main(argv=None) -> int:
     results = []
     for max_num_seqs in sizes:
         engine = make_engine(max_num_seqs)
+        if args.tune_library:
+            from velox_amd.engine.runner import decode_buckets
+
+            engine.tune_matrix_products([args.max_prefill_chunk_size] + [b for b in decode_buckets(max_num_seqs) if b > 16])
         vocab = engine.model.spec.vocab_size
         limit = engine.max_model_len - args.max_tokens - 1
         if limit < 1:
             raise SystemExit("--max-tokens leaves no room for a prompt under --max-model-len")
-        prompts = build_prompts(args.workload, args.num_requests, vocab, limit, args.prompt_len, args.seed, args.shared_system_prompt)
+        length_range = tuple(int(v) for v in args.prompt_len_range.split(",")) if args.prompt_len_range else None
+        prompts = build_prompts(args.workload, args.num_requests, vocab, limit, args.prompt_len, args.seed, args.shared_system_prompt, length_range)
         rule("ENGINE BENCHMARK")
         print(f"  Model            : {args.model or args.shape + ' (random weights)'}")
         print(f"  PyTorch / HIP    : {torch.__version__} / {torch.version.hip}")
