@@ -121,3 +121,56 @@ def test_trace_run_program(tmp_path):
                     torch.testing.assert_close(torch.from_numpy(outputs[record["step"]][row]), expected[entry["id"]][at[entry["id"]] + w], **TOL[dtype])
                     row += 1
                 at[entry["id"]] += len(entry["tokens"])
+
+
+QWEN25_7B_TWO_LAYERS = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "num_hidden_layers": 2, "hidden_size": 3584, "num_attention_heads": 28, "num_key_value_heads": 4,
+    "intermediate_size": 18944, "vocab_size": 152064, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": False, "use_sliding_window": False, "max_position_embeddings": 32768,
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layers_of_the_real_size_in_four_ways_of_cutting(tmp_path, dtype):
+    """Two layers with the sizes of Qwen2.5-7B (width 3584, 28 heads over 4 groups of size 128, 18944 inner columns, a
+    vocabulary of 152064): the sizes at which the decode kernels, the library's products and the wide attention kernel
+    take other paths than with the tiny models.  One engine serves all four traces, so pages are used again between
+    them as well."""
+    from velox_amd.weights import write_random_model
+
+    folder = write_random_model(QWEN25_7B_TWO_LAYERS, str(tmp_path / "real_size"), 3, dtype=storage_for(dtype))
+    config, weights = read_model_folder(folder)
+    requests = rc.request_set(config["vocab_size"], [97, 33, 150, 64], seed=41)
+    expected = rc.expected_logits(config, weights, requests)
+    traces = {"whole": rc.whole(requests), "tail": rc.tail_one_by_one(requests), "portions": rc.changing_portions(requests),
+              "mixed": rc.mixed(requests, seed=6)}
+    replayer = Replayer(folder, dtype, max(rc.tokens_needed(t, 16) for t in traces.values()), block_size=16)
+    if dtype == "float32":
+        # Sums of 3584 and 18944 float32 terms round differently in every order of adding, more than the tiny models'
+        # sums of a hundred terms do.  The yardstick is the plain model's own float32 rounding, measured against the same
+        # model in float64: the engine has to be as close to the exact logits as the plain float32 implementation is.
+        exact = {rid: qwen2_logits(config, weights, tokens, dtype=torch.float64) for rid, tokens in requests.items()}
+        rounding = max(float((expected[rid].double() - exact[rid]).abs().max()) for rid in requests)
+        assert 1e-6 < rounding < 2e-4, rounding
+        tol = dict(rtol=0.0, atol=3 * rounding)
+        expected = {rid: exact[rid].float() for rid in requests}
+    results = {}
+    for label, trace in traces.items():
+        results[label] = rc.collect(trace, rc.run_trace(replayer, trace), requests)
+        for rid in requests:
+            if dtype == "float32":
+                torch.testing.assert_close(results[label][rid], expected[rid], msg=lambda m: f"{dtype} {label} {rid}: {m}", **tol)
+                continue
+            # bfloat16: about twenty tensors on the way to a logit are rounded to 8 bits (relative error up to 2^-9 each,
+            # independent): the logits' error is then about 2^-9 * sqrt(20) = 0.9% of their spread in the root mean
+            # square, whatever the width.  Twice that is allowed, and eight such deviations for the worst of the 15
+            # million logits; a key read from a wrong place or a wrong position changes logits by their whole spread.
+            spread = float(expected[rid].std())
+            error = results[label][rid] - expected[rid]
+            assert float(error.pow(2).mean().sqrt()) < 0.0175 * spread, (label, rid, float(error.pow(2).mean().sqrt()), spread)
+            assert float(error.abs().max()) < 8 * 0.0175 * spread, (label, rid, float(error.abs().max()), spread)
+    if dtype == "float32":
+        for label in ("tail", "portions", "mixed"):
+            for rid in requests:
+                torch.testing.assert_close(results[label][rid], results["whole"][rid], **tol)

@@ -4,13 +4,18 @@
 // multiplied with plain fused multiply-adds, so a float32 run never touches a reduced-precision
 // matrix mode.  It also serves operand mixes no library call covers (bfloat16 activations with
 // weights a checkpoint stores in float32).  Each output element is summed over k in one fixed
-// order by one thread, so a row's result does not depend on the other rows of the batch.
+// order by one thread, so a row's result does not depend on the other rows of the batch.  The sum
+// is built from sums of GEMM_FOLD consecutive terms, each started at zero: the rounding error of a
+// long sum (the down projection adds 18944 terms) then grows with the square roots of the two
+// lengths and not with that of their product, which keeps the float32 path as close to the exact
+// result as a blocked library product on a CPU is.
 #include "common.h"
 
 #define GEMM_BM 64
 #define GEMM_BN 64
 #define GEMM_BK 16
 #define GEMM_PAD 4
+#define GEMM_FOLD 128  // terms per inner sum (a multiple of GEMM_BK)
 
 template <typename T>
 __device__ __forceinline__ void load4(const T* __restrict__ base, size_t row_offset, int k, int k_limit, bool row_ok, bool vec_ok, float (&v)[4]) {
@@ -46,13 +51,22 @@ __global__ void __launch_bounds__(256) gemm_fma_kernel(const TA* __restrict__ a,
   const size_t a_off = (size_t)(m0 + load_row) * k;
   const size_t w_off = (size_t)(n0 + load_row) * k;
 
-  float acc[4][4];
+  float acc[4][4], total[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int j = 0; j < 4; ++j) acc[i][j] = total[i][j] = 0.f;
 
   for (int k0 = 0; k0 < k; k0 += GEMM_BK) {
+    if (k0 % GEMM_FOLD == 0) {  // (also at 0: adds zeros)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          total[i][j] += acc[i][j];
+          acc[i][j] = 0.f;
+        }
+    }
     float av[4], wv[4];
     load4<TA>(a, a_off, k0 + load_k, k, a_row_ok, a_vec != 0, av);
     load4<TW>(w, w_off, k0 + load_k, k, w_row_ok, w_vec != 0, wv);
@@ -81,7 +95,7 @@ __global__ void __launch_bounds__(256) gemm_fma_kernel(const TA* __restrict__ a,
     for (int j = 0; j < 4; ++j) {
       const int col = n0 + tx * 4 + j;
       if (col >= n) continue;
-      float v = acc[i][j];
+      float v = total[i][j] + acc[i][j];
       if (bias) v += bias[col];
       out[(size_t)row * n + col] = from_f32<TO>(v);
     }
