@@ -197,6 +197,31 @@ def test_requests_that_take_over_a_published_prefix(tmp_path, dtype):
     assert engine.cache.num_used_pages() == engine.cache.prefix.num_nodes > 0
 
 
+def test_batches_of_every_size_class_with_layers_of_the_real_size(tmp_path):
+    """bfloat16, two layers with the sizes of Qwen2.5-7B, captured decode steps: 40 requests decode together (the 64-row
+    bucket: split-K products and the library), then 12 (the 16-row bucket: the fused decode kernels), then one.  Every
+    chosen token has to be the plain model's best one up to rounding (see the replay test of the same sizes: the
+    logits' error is about 1% of their spread of 1.2, eight times that for the worst of them)."""
+    from test_replay_gpu import QWEN25_7B_TWO_LAYERS
+    from velox_amd.weights import write_random_model
+
+    folder = write_random_model(QWEN25_7B_TWO_LAYERS, str(tmp_path / "real_size"), 4, dtype="bfloat16")
+    config, weights = read_model_folder(folder)
+    engine = Engine.from_pretrained(EngineConfig(model=folder, dtype="bfloat16", device="cuda", max_model_len=64, max_num_seqs=64,
+                                                 max_num_batched_tokens=256, max_prefill_chunk_size=128, num_gpu_blocks=300, seed=0))
+    assert sorted(engine.runner._graphs) == [1, 2, 4, 8, 16, 32, 64]
+    for count, seed in ((40, 200), (12, 300), (1, 400)):
+        prompts = [random_tokens(config["vocab_size"], 3 + (i % 7), seed=seed + i) for i in range(count)]
+        replays = engine.runner.num_graph_replays
+        done = engine.generate(greedy(prompts, 5, prefix=f"n{count}-"))
+        assert engine.runner.num_graph_replays >= replays + 4
+        for request, prompt in list(zip(done, prompts))[::max(1, count // 6)]:
+            logits = qwen2_logits(config, weights, prompt + request.output_token_ids[:-1])[len(prompt) - 1:]
+            for step, token in enumerate(request.output_token_ids):
+                assert logits[step][token] >= logits[step].max() - 0.2, (count, request.request_id, step)
+    engine.cache.assert_consistent([])
+
+
 def test_sampling_through_the_engine(tmp_path):
     folder = make_folder(tmp_path, "B")
     config, _ = read_model_folder(folder)
