@@ -174,3 +174,47 @@ def test_layers_of_the_real_size_in_four_ways_of_cutting(tmp_path, dtype):
         for label in ("tail", "portions", "mixed"):
             for rid in requests:
                 torch.testing.assert_close(results[label][rid], results["whole"][rid], **tol)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_context_in_large_portions_then_token_by_token(tmp_path, dtype):
+    """6,000 tokens: portions of 2,048 behind thousands of cached keys (the wide attention kernel and the one with two
+    sets of waves), then single tokens over a key range that is split many ways, beside a short request that decodes
+    in the same steps.  Queries and keys are sharpened so that a far key read wrongly shows."""
+    from velox_amd.weights import write_random_model
+
+    config = dict(CONFIGS["A"], max_position_embeddings=8192)
+    folder = write_random_model(config, str(tmp_path / "long"), 7, dtype=storage_for(dtype))
+    path = os.path.join(folder, "model.safetensors")
+    raw = load_file(path)
+    for layer in range(2):
+        for proj in ("q_proj", "k_proj"):
+            key = f"model.layers.{layer}.self_attn.{proj}.weight"
+            raw[key] = (raw[key].float() * 4.0).to(raw[key].dtype)
+    save_file(raw, path)
+    config, weights = read_model_folder(folder)
+    long_tokens = random_tokens(256, 6000, seed=77)
+    short_tokens = random_tokens(256, 40, seed=78)
+    expected = {"long": qwen2_logits(config, weights, long_tokens), "short": qwen2_logits(config, weights, short_tokens)}
+    trace, at = [], 0
+    for size in (2048, 2048, 1872):
+        trace.append({"step": len(trace), "entries": [{"id": "long", "tokens": long_tokens[at:at + size], "want": [0, size // 2, size - 1]}], "end": []})
+        at += size
+    trace.append({"step": len(trace), "entries": [{"id": "short", "tokens": short_tokens[:8], "want": [7]}], "end": []})
+    for i in range(32):
+        trace.append({"step": len(trace), "entries": [{"id": "long", "tokens": [long_tokens[at + i]], "want": [0]},
+                                                      {"id": "short", "tokens": [short_tokens[8 + i]], "want": [0]}],
+                      "end": ["long", "short"] if i == 31 else []})
+    assert at + 32 == 6000
+    replayer = Replayer(folder, dtype, rc.tokens_needed(trace, 4), block_size=4)
+    outputs = rc.run_trace(replayer, trace)
+    held = {"long": 0, "short": 0}
+    for record in trace:
+        row = 0
+        for entry in record["entries"]:
+            for w in entry["want"]:
+                got = torch.from_numpy(outputs[record["step"]][row].copy())
+                torch.testing.assert_close(got, expected[entry["id"]][held[entry["id"]] + w],
+                                           msg=lambda m: f"{dtype} step {record['step']} {entry['id']} position {held[entry['id']] + w}: {m}", **TOL[dtype])
+                row += 1
+            held[entry["id"]] += len(entry["tokens"])
