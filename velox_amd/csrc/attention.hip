@@ -133,13 +133,14 @@ constexpr int PREFILL_PAGE_IDS = 2048;
 // compiler is held to it (left alone it takes more registers than one wave per SIMD's worth buys back)
 constexpr int GENERAL_MIN_WAVES = D <= 128 ? 2 : 1;
 
-// CT = 16-row tiles per wave: a workgroup owns 64 * CT rows.  With CT = 2 every K and V^T operand read from LDS feeds
-// two matrix instructions, which is what long portions of prompts need; a row's arithmetic is the same for every CT.
+// CT = 16-row tiles per wave, WAVES = waves of a set: a workgroup owns 16 * WAVES * CT rows.  With CT = 2 every K and V^T
+// operand read from LDS feeds two matrix instructions, which is what long streams of keys need; a row's arithmetic
+// is the same for every CT and WAVES.
 // KSPLIT = 2: the workgroup has two sets of 4 waves that own the same rows and take the key tiles alternately, each
 // set staging its own tiles; at the end the second set hands its running (maximum, sum, output) to the first
 // through LDS.  The longest workgroups of a causal step, which decide how long the step takes, finish in half the time.
-template <typename T, int BN, int CT, int KSPLIT>
-__global__ void __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(GENERAL_MIN_WAVES, 2))) paged_attention_kernel(
+template <typename T, int BN, int CT, int KSPLIT, int WAVES = 4>
+__global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_waves_per_eu(GENERAL_MIN_WAVES, WAVES > 4 ? 4 : 2))) paged_attention_kernel(
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
     T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
@@ -157,7 +158,9 @@ __global__ void __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_
   constexpr int NKB = BN / KB;                  // contraction blocks of P V
   constexpr int TPB = KB / 16;                  // S^T tiles per key block
   constexpr int NC = D / 16;                    // 16-channel tiles of the output
-  constexpr int ROWS_PER_BLOCK = 64 * CT;
+  constexpr int SETW = 64 * WAVES;              // threads of a set of waves
+  static_assert(KSPLIT == 1 || WAVES == 4, "two sets of waves are sets of four");
+  constexpr int ROWS_PER_BLOCK = 16 * WAVES * CT;
   constexpr int TILE_ELEMS = BN * KS + D * VS;                      // one set's K tile and V^T tile
   constexpr int MERGE_FLOATS = KSPLIT > 1 ? 256 * CT * (4 * NC + 2) : 0;  // what the second set hands over at the end
   constexpr int TILE_BYTES = KSPLIT * TILE_ELEMS * (int)sizeof(T);
@@ -244,11 +247,11 @@ __global__ void __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_
   int first_page = (n_begin + tile_lo * BN) >> page_shift;  // first page of the window
   auto load_page_ids = [&]() {
     const int num_pages = last_page - first_page + 1;
-    for (int p = threadIdx.x; p < num_pages && p < PREFILL_PAGE_IDS; p += 256 * KSPLIT) page_ids[p] = table[first_page + p];
+    for (int p = threadIdx.x; p < num_pages && p < PREFILL_PAGE_IDS; p += SETW * KSPLIT) page_ids[p] = table[first_page + p];
   };
   load_page_ids();
   if constexpr (DP > D) {
-    for (int e = tid; e < BN * (DP - D); e += 256) k_tile[(e / (DP - D)) * KS + D + e % (DP - D)] = from_f32<T>(0.f);
+    for (int e = tid; e < BN * (DP - D); e += SETW) k_tile[(e / (DP - D)) * KS + D + e % (DP - D)] = from_f32<T>(0.f);
   }
   auto page_of = [&](int n) -> size_t { return (size_t)page_ids[(n >> page_shift) - first_page]; };
 
@@ -273,14 +276,14 @@ __global__ void __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_
   // ---- staging: global -> registers (issued a tile ahead) -> LDS; what does not change from tile to tile is computed once
   constexpr int VPR = D / VEC;              // vectors per key row of K
   constexpr int VECS = BN * D / VEC;        // vectors per tile (K and V^T alike)
-  constexpr int ITERS = (VECS + 255) / 256;
+  constexpr int ITERS = (VECS + SETW - 1) / SETW;
   const int run = page_size < BN ? page_size : BN;  // consecutive keys that are contiguous in a page of V
   const bool v_by_vectors = run >= VEC;
   const int run_shift = v_by_vectors ? __builtin_ctz(run / VEC) : 0;  // log2(vectors per run and channel)
   int k_key[ITERS], k_col[ITERS], v_dd[ITERS], v_key[ITERS], v_lds[ITERS];
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
-    const int v = tid + it * 256 < VECS ? tid + it * 256 : VECS - 1;  // (the spare threads of a last pass repeat its last vector)
+    const int v = tid + it * SETW < VECS ? tid + it * SETW : VECS - 1;  // (the spare threads of a last pass repeat its last vector)
     k_key[it] = v / VPR;
     k_col[it] = (v % VPR) * VEC;
     const int rn = (v >> run_shift) / D;            // run index within the tile
@@ -317,8 +320,8 @@ __global__ void __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_
   auto commit = [&](int n0) {
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-      if constexpr (VECS % 256 != 0) {
-        if (tid + it * 256 >= VECS) continue;
+      if constexpr (VECS % SETW != 0) {
+        if (tid + it * SETW >= VECS) continue;
       }
       if (n0 + k_key[it] >= kv_len) k_regs[it] = float4_t{0.f, 0.f, 0.f, 0.f};
       *reinterpret_cast<float4_t*>(k_tile + k_key[it] * KS + k_col[it]) = k_regs[it];
@@ -345,7 +348,7 @@ __global__ void __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_
     }
     if (!v_by_vectors) {  // pages shorter than a vector: element by element, straight from global memory
       const int per = D * run;
-      for (int v = tid; v < BN * D; v += 256) {
+      for (int v = tid; v < BN * D; v += SETW) {
         const int rn = v / per, rem = v % per;
         const int dd = rem / run, e = rem % run;
         const int nl = rn * run + e;
@@ -796,15 +799,26 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
     merge_splits_kernel<T><<<dim3(total_tokens, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens);
     return (int)hipGetLastError();
   }
-  // 128 rows per workgroup (two row tiles per wave) when bfloat16 portions are long enough to fill them
-  // and the step brings enough rows that the larger workgroups still fill the GPU
+  // Eight waves per workgroup when bfloat16 portions are long enough to fill their rows and the step brings enough rows
+  // that the larger workgroups still fill the GPU.  Behind few keys (a causal step's longest workgroup decides how
+  // long the step takes, and short streams of keys leave LDS idle) a wave takes one row tile, 128 rows per workgroup;
+  // behind many keys two, 256 rows per workgroup: every K and V^T operand read from LDS then feeds two matrix
+  // instructions.  Measured on MI355X: 2,048 tokens from an empty cache 75 us against 85, 4 x 512 tokens behind 8,192
+  // keys 315 us against 426 the other way round; the two meet where an average row reads about 1,300 keys.
   constexpr int WIDE = (sizeof(T) == 2 && D <= 128) ? 2 : 1;
   const int rows = max_q_len * group;
   if (WIDE == 2 && rows > 64 && (long long)total_tokens * group / 128 * nkv >= compute_units()) {
-    dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
-    paged_attention_kernel<T, BN, WIDE, 1><<<grid, 256, 0, stream>>>(
-        (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+    if (max_kv_len - max_q_len / 2 <= 1280 || rows < 192) {  // (keys an average row reads)
+      dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
+      paged_attention_kernel<T, BN, 1, 1, 8><<<grid, 512, 0, stream>>>(
+          (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+    } else {
+      dim3 grid((rows + 255) / 256, nkv, num_seqs * splits);
+      paged_attention_kernel<T, BN, WIDE, 1, 8><<<grid, 512, 0, stream>>>(
+          (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+    }
   } else if (WIDE == 2 && (long long)((rows + 63) / 64) * nkv * num_seqs * splits < 2 * compute_units() && max_kv_len >= 8 * BN) {
     // too few workgroups to fill the GPU and many keys each: two sets of waves share a workgroup's keys
     dim3 grid((rows + 63) / 64, nkv, num_seqs * splits);
