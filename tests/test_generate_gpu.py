@@ -222,6 +222,25 @@ def test_batches_of_every_size_class_with_layers_of_the_real_size(tmp_path):
     engine.cache.assert_consistent([])
 
 
+def test_a_small_pool_with_shared_prefixes_captured_steps_and_early_launches(tmp_path):
+    """float32 on the GPU with everything on at once: prefix caching, captured decode steps, the next step launched
+    early, and a pool so small that requests are preempted and published pages evicted.  The tokens are the plain
+    model's, request by request."""
+    folder = make_folder(tmp_path, "B", "float32")
+    config, weights = read_model_folder(folder)
+    page = PAGE_SIZE["B"]
+    stem = random_tokens(config["vocab_size"], 2 * page + 3, seed=9)
+    prompts = [stem + random_tokens(config["vocab_size"], 4 + 3 * i, seed=20 + i) for i in range(7)]
+    needed = max((len(p) + 14 + page - 1) // page for p in prompts)
+    engine = engine_for(folder, "B", "float32", enable_prefix_caching=True, enable_cuda_graphs=True,
+                        num_gpu_blocks=2 * needed + 3, max_model_len=needed * page)
+    done = engine.generate(greedy(prompts, 14))
+    for request, prompt in zip(done, prompts):
+        assert request.output_token_ids == plain_greedy(config, weights, prompt, 14), request.request_id
+    assert engine.scheduler.num_preemptions > 0 and engine.cache.prefix.num_hits > 0 and engine.runner.num_graph_replays > 0
+    engine.cache.assert_consistent([])
+
+
 def test_sampling_through_the_engine(tmp_path):
     folder = make_folder(tmp_path, "B")
     config, _ = read_model_folder(folder)
