@@ -161,6 +161,8 @@ def parse_args(argv=None) -> argparse.Namespace:
     parser.add_argument("--block-size", type=int, default=16)
     parser.add_argument("--num-gpu-blocks", type=int, default=None)
     parser.add_argument("--gpu-memory-utilization", type=float, default=0.85)
+    parser.add_argument("--kv-cache-dtype", default="auto", help="only 'auto' (the run dtype): quantized caches are not built")
+    parser.add_argument("--quantization", default=None, help="not built: anything but none is refused")
     parser.add_argument("--no-prefix-caching", action="store_true", help="compute every prompt in full (no sharing of prompt prefixes between requests)")
     parser.add_argument("--no-cuda-graphs", "--no-hip-graphs", dest="no_graphs", action="store_true")
     parser.add_argument("--shared-system-prompt", action="store_true", help="every prompt starts with the same %d tokens" % SHARED_PREFIX_TOKENS)
@@ -190,6 +192,7 @@ def main(argv=None) -> int:
             model=args.model or "", dtype=args.dtype, max_model_len=args.max_model_len, max_num_seqs=max_num_seqs,
             max_num_batched_tokens=max(args.max_num_batched_tokens, max_num_seqs), max_prefill_chunk_size=args.max_prefill_chunk_size,
             block_size=args.block_size, num_gpu_blocks=args.num_gpu_blocks, gpu_memory_utilization=args.gpu_memory_utilization,
+            kv_cache_dtype=args.kv_cache_dtype, quantization=args.quantization,
             enable_prefix_caching=not args.no_prefix_caching, enable_cuda_graphs=not args.no_graphs, seed=args.seed)
         if args.model:
             return Engine.from_pretrained(config)

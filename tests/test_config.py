@@ -89,7 +89,9 @@ def test_engine_config_checks():
     with pytest.raises(ValueError):
         resolve_dtype("int8")
     EngineConfig().validate()
+    EngineConfig(kv_cache_dtype="auto", quantization=None, download_dir="/nowhere").validate()  # the reference's defaults are accepted
     for bad in (dict(max_num_seqs=0), dict(max_num_batched_tokens=100, max_prefill_chunk_size=512), dict(block_size=12),
-                dict(gpu_memory_utilization=0.0), dict(max_num_batched_tokens=16, max_prefill_chunk_size=8, max_num_seqs=32)):
+                dict(gpu_memory_utilization=0.0), dict(max_num_batched_tokens=16, max_prefill_chunk_size=8, max_num_seqs=32),
+                dict(kv_cache_dtype="fp8"), dict(quantization="int8")):
         with pytest.raises(ValueError):
             EngineConfig(**bad).validate()

@@ -1,8 +1,10 @@
 """Engine options, with the reference's names and meanings (``engine/config.py:34-75``).
 
-Left out: ``download_dir`` (no hub), ``kv_cache_dtype`` and ``quantization`` (the cache
-holds the run dtype).  Added: ``watermark`` (the reference keeps it in its scheduler
-configuration, ``engine/scheduler.py:23``).  ``enable_cuda_graphs`` keeps the reference's
+``download_dir``, ``kv_cache_dtype`` and ``quantization`` are accepted at their reference
+defaults only, so that the reference's call sites keep working: there is no hub to
+download from, and the cache and the weights hold the run dtype (anything else is refused).
+Added: ``watermark`` (the reference keeps it in its scheduler configuration,
+``engine/scheduler.py:23``).  ``enable_cuda_graphs`` keeps the reference's
 name; what it switches here is HIP-graph capture of the all-decode step.
 """
 from __future__ import annotations
@@ -41,6 +43,8 @@ class EngineConfig:
     dtype: str = "auto"
     device: str = "cuda"
 
+    download_dir: Optional[str] = None
+
     max_model_len: int = 4096
     max_num_seqs: int = 32
     max_num_batched_tokens: int = 2048
@@ -54,6 +58,8 @@ class EngineConfig:
     # pages of a prompt prefix that an earlier request has computed are taken over instead of computed again (on by
     # default as in the reference; models whose layers keep a window or a state of fixed size run without it)
     enable_prefix_caching: bool = True
+    kv_cache_dtype: str = "auto"
+    quantization: Optional[str] = None
     enable_cuda_graphs: bool = True
     # a second copy of every bfloat16 weight in the order the decode kernels read it: faster decoding for the
     # weights' size again in memory (not a reference option)
@@ -81,3 +87,7 @@ class EngineConfig:
             raise ValueError("block_size must be a power of two")
         if self.max_prefill_chunk_size < 1 or self.max_model_len < 2:
             raise ValueError("max_prefill_chunk_size must be at least 1 and max_model_len at least 2")
+        if (self.kv_cache_dtype or "auto").lower() not in ("auto", str(self.dtype).lower()):
+            raise ValueError(f"kv_cache_dtype={self.kv_cache_dtype!r}: the cache holds the run dtype; quantized caches are not built")
+        if self.quantization not in (None, "", "none"):
+            raise ValueError(f"quantization={self.quantization!r}: weight quantization is not built")
