@@ -145,6 +145,7 @@ def main() -> int:
     parser.add_argument("--no-graphs", action="store_true")
     parser.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     parser.add_argument("--no-tune", action="store_true", help="do not let the matrix library pick its kernels for the prefill shapes")
+    parser.add_argument("--no-probes", action="store_true", help="skip the probes of what the card delivers (streaming read, bfloat16 matrix instructions)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine (single-GPU tier)")
@@ -207,6 +208,14 @@ def main() -> int:
         },
         "points": {f"decode_b{b}": round(b / s, 2) for b, s in step_s.items() if b != args.batch},
     }
+    if not args.no_probes:
+        # what this card delivers to a kernel that only reads, and to one that only issues matrix instructions: the
+        # fractions above are of the published peaks, these say how much of the gap is the card's own
+        read_gbs, mfma_tflops = engine.ops.probe_read_bandwidth(), engine.ops.probe_mfma_rate()
+        result["probes"] = {
+            "hbm_read_gbs": round(read_gbs, 1), "mfma_bf16_tflops": round(mfma_tflops, 1),
+            "decode_frac_of_read": round(achieved / read_gbs, 4),
+        }
     print(json.dumps(result))
     return 0
 

@@ -599,3 +599,11 @@ def test_skinny_gemm_splitk_and_norm_that_adds_the_partials(ops, ref, m, n, k):
         rows = torch.tensor([m - 1, 0, 3], dtype=torch.int32).cuda()
         torch.testing.assert_close(ops.add_rmsnorm_rows(r_hip, part, rows, weight, 1e-6, torch.float32),
                                    ref.add_rmsnorm_rows(r_ref, part, rows, weight, 1e-6, torch.float32), rtol=1e-4, atol=1e-4)
+
+
+def test_probes_report_rates_below_the_published_peaks(ops):
+    # a sanity band, not a benchmark: the read streams 256 MiB, the matrix loop is short
+    read = ops.probe_read_bandwidth(num_bytes=(256 << 20) + 48, repeats=3)
+    mfma = ops.probe_mfma_rate(iterations=2000, repeats=3)
+    assert 500.0 < read < 8000.0 * 3  # part of 256 MiB may come from the caches
+    assert 100.0 < mfma <= 2600.0

@@ -23,7 +23,7 @@ SOURCE_DIR = os.path.join(PACKAGE_DIR, "csrc")
 ARCH = "gfx950"
 # hipcc -O3 must not form packed float32 operations from scalar code on this target
 FLAGS = ["-O3", f"--offload-arch={ARCH}", "-shared", "-fPIC", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-CORE_SOURCES = ["elementwise.hip", "gemm.hip", "skinny_gemm.hip", "sampling.hip"]
+CORE_SOURCES = ["elementwise.hip", "gemm.hip", "skinny_gemm.hip", "sampling.hip", "probe.hip"]
 ATTENTION_SOURCES = ["attention.hip"]
 HEADERS = ["common.h"]
 # head sizes built ahead of time by build_all(); any other multiple of 16 up to 256 is built at first use

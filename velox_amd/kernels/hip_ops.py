@@ -84,6 +84,10 @@ class HipOps:
         c.velox_argmax.argtypes = [_P, _P, _P, _I, _I, _I, _P]
         c.velox_sample.argtypes = [_P, _P, _P, _I, _I, _P]
         c.velox_apply_penalties.argtypes = [_P, _P, _P, _P, _I, _I, _I, _P]
+        c.velox_probe_read.argtypes = [_P, ctypes.c_longlong, _P, _I, _P]
+        c.velox_probe_read.restype = _I
+        c.velox_probe_mfma.argtypes = [_I, _I, _P, _P]
+        c.velox_probe_mfma.restype = _I
         for fn in (c.velox_embed, c.velox_add_rmsnorm, c.velox_silu_mul, c.velox_rope_kv_write, c.velox_gemm_fma,
                    c.velox_argmax, c.velox_sample, c.velox_apply_penalties):
             fn.restype = _I
@@ -603,3 +607,34 @@ class HipOps:
         self._check("coeffs", coeffs, torch.float32, (rows, 3))
         status = self._core.velox_apply_penalties(_ptr(logits), _ptr(tokens), _ptr(lengths), _ptr(coeffs), rows, vocab, tokens.shape[1], self._stream())
         self._launched(status, "apply_penalties")
+
+    # -- probes ---------------------------------------------------------------------------------
+    def _timed(self, launch, repeats: int) -> float:
+        """Seconds per call of ``launch`` (the best of ``repeats`` after one untimed call)."""
+        launch()
+        torch.cuda.synchronize(self.device)
+        best = float("inf")
+        for _ in range(repeats):
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            launch()
+            end.record()
+            end.synchronize()
+            best = min(best, start.elapsed_time(end) * 1e-3)
+        return best
+
+    def probe_read_bandwidth(self, num_bytes: int = 4 << 30, repeats: int = 5) -> float:
+        """GB/s at which a kernel that only reads streams ``num_bytes`` of device memory (far more than the caches hold)."""
+        num_bytes -= num_bytes % 16
+        data = torch.empty(num_bytes, dtype=torch.uint8, device=self.device).zero_()
+        sink = torch.zeros(1, dtype=torch.int32, device=self.device)
+        blocks = self.num_cus * 8
+        seconds = self._timed(lambda: self._launched(self._core.velox_probe_read(_ptr(data), num_bytes, _ptr(sink), blocks, self._stream()), "probe_read"), repeats)
+        return num_bytes / seconds * 1e-9
+
+    def probe_mfma_rate(self, iterations: int = 20000, repeats: int = 5) -> float:
+        """TFLOP/s of independent bfloat16 32x32x16 matrix instructions, two workgroups of four waves per compute unit."""
+        sink = torch.zeros(1, dtype=torch.float32, device=self.device)
+        blocks = self.num_cus * 2
+        seconds = self._timed(lambda: self._launched(self._core.velox_probe_mfma(blocks, iterations, _ptr(sink), self._stream()), "probe_mfma"), repeats)
+        return blocks * 4 * iterations * 4 * 32768.0 / seconds * 1e-12
