@@ -173,7 +173,11 @@ def parse_args(argv=None) -> argparse.Namespace:
     parser.add_argument("--show-outputs", action="store_true")
     parser.add_argument("--output-json", default=None)
     parser.add_argument("--seed", type=int, default=0)
-    return parser.parse_args(argv)
+    parser.add_argument("--compare-hf", action="store_true", help="not built (the reference compares with another library's model; this engine's yardstick is the plain model under tests/)")
+    args = parser.parse_args(argv)
+    if args.compare_hf:
+        parser.error("--compare-hf is not built: no library model is part of this engine; tests/plain_qwen2.py is the yardstick")
+    return args
 
 
 def main(argv=None) -> int:
