@@ -218,3 +218,34 @@ def test_a_long_context_in_large_portions_then_token_by_token(tmp_path, dtype):
                                            msg=lambda m: f"{dtype} step {record['step']} {entry['id']} position {held[entry['id']] + w}: {m}", **TOL[dtype])
                 row += 1
             held[entry["id"]] += len(entry["tokens"])
+
+
+ODD_CONFIGS = {
+    # one KV head of size 256 for two query heads, pages of 64 tokens
+    "wide_heads": dict(num_hidden_layers=2, hidden_size=512, num_attention_heads=2, num_key_value_heads=1, intermediate_size=384,
+                       vocab_size=777, rope_theta=20000.0, rms_norm_eps=1e-5, tie_word_embeddings=True, page=64),
+    # 18 query heads on one KV head (more rows than one tile of 16), inner width and vocabulary that no tile divides, pages of 2
+    "large_group": dict(num_hidden_layers=2, hidden_size=288, num_attention_heads=18, num_key_value_heads=1, intermediate_size=100,
+                        vocab_size=1001, rope_theta=1e5, rms_norm_eps=1e-3, tie_word_embeddings=False, page=2),
+    # heads whose sizes add up to more than the width, every head with keys of its own
+    "own_head_size": dict(num_hidden_layers=3, hidden_size=104, num_attention_heads=5, num_key_value_heads=5, head_dim=64,
+                          intermediate_size=72, vocab_size=90, rope_theta=300.0, rms_norm_eps=1e-6, tie_word_embeddings=False, page=32),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(ODD_CONFIGS))
+def test_sizes_at_the_edges_of_what_the_kernels_take(tmp_path, name, dtype):
+    from velox_amd.weights import write_random_model
+
+    config = dict(ODD_CONFIGS[name], architectures=["Qwen2ForCausalLM"], model_type="qwen2", use_sliding_window=False, max_position_embeddings=512)
+    page = config.pop("page")
+    folder = write_random_model(config, str(tmp_path / name), 5, dtype=storage_for(dtype))
+    config, weights = read_model_folder(folder)
+    requests = rc.request_set(config["vocab_size"], [83, 40, 130], seed=51)
+    expected = rc.expected_logits(config, weights, requests)
+    for label, trace in (("whole", rc.whole(requests)), ("tail", rc.tail_one_by_one(requests)), ("mixed", rc.mixed(requests, seed=4, max_live=2))):
+        replayer = Replayer(folder, dtype, rc.tokens_needed(trace, max(page, 64)), block_size=page)
+        got = rc.collect(trace, rc.run_trace(replayer, trace), requests)
+        for rid in requests:
+            torch.testing.assert_close(got[rid], expected[rid], msg=lambda m: f"{name} {dtype} {label} {rid}: {m}", **TOL[dtype])
