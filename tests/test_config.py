@@ -95,3 +95,16 @@ def test_engine_config_checks():
                 dict(kv_cache_dtype="fp8"), dict(quantization="int8")):
         with pytest.raises(ValueError):
             EngineConfig(**bad).validate()
+
+
+def test_head_sizes_the_kernels_do_not_take_are_refused_when_the_model_is_built():
+    import torch
+
+    from velox_amd.engine.engine import build_model
+
+    for head_dim in (40, 8, 272):
+        cfg = config_from_dict({**TINY_A, "head_dim": head_dim})
+        with pytest.raises(ValueError) as err:
+            build_model(cfg, torch.float32, torch.device("cpu"))
+        assert f"head_dim={head_dim}" in str(err.value) and "multiples of 16" in str(err.value)
+    build_model(config_from_dict({**TINY_A, "head_dim": 80}), torch.float32, torch.device("cpu"))
