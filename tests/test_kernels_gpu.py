@@ -221,6 +221,52 @@ def test_qkv_projection_with_rotation_and_cache_write_in_one_kernel(ops, ref, m,
     assert torch.equal(before, k_cache)
 
 
+@pytest.mark.parametrize("m", [17, 40, 64])
+@pytest.mark.parametrize("nh,nkv,d,k,page,rotate", [(4, 2, 64, 128, 4, True), (28, 4, 128, 3584, 16, True), (3, 1, 32, 192, 1, True), (2, 2, 96, 1024, 8, False),
+                                                    (5, 5, 48, 320, 32, True)])
+def test_qkv_projection_at_17_to_64_rows_with_partial_sums_added_by_the_rotation(ops, ref, m, nh, nkv, d, k, page, rotate):
+    """Split-K partial sums -> (sum, bias, rotation, cache write) in one kernel, against the same steps in float32; slots
+    in runs of consecutive tokens (a prompt's portion) and scattered (decoding requests)."""
+    pages = 80
+    width = (nh + 2 * nkv) * d
+    half = d // 2
+    x = rand((m, k), torch.bfloat16, 90)
+    w = rand((width, k), torch.bfloat16, 91, 0.05)
+    bias = rand((width,), torch.float32, 92, 0.3)
+    positions = torch.randint(0, 500, (m,), generator=torch.Generator().manual_seed(93)).to(torch.int32).cuda()
+    scattered = torch.randperm((pages - 1) * page, generator=torch.Generator().manual_seed(94))[:m] + page
+    consecutive = torch.arange(m) + page + 3
+    angles = torch.outer(torch.arange(512, dtype=torch.float32), 1.0 / (10000.0 ** (torch.arange(half, dtype=torch.float32) / half)))
+    cos, sin = (angles.cos().cuda(), angles.sin().cuda()) if rotate else (None, None)
+    ops.register_weight(w, rotary_heads=(nh, nkv, d))
+    scale = float(ref.linear(x, w, None, torch.float32).abs().max())
+    for slots in (scattered, consecutive):
+        slots = slots.to(torch.int32).cuda()
+        for use_bias in (bias, None):
+            k32 = torch.full((pages, nkv, page, d), 7.0, dtype=torch.float32, device="cuda")
+            v32 = torch.full((pages, nkv, d, page), 7.0, dtype=torch.float32, device="cuda")
+            wide = ref.linear(x, w, None, torch.float32)
+            ref.rope_kv_write(wide, nh, nkv, d, positions, cos, sin, slots, k32, v32, page, write_kv=True, bias=use_bias)
+            k_cache = torch.full((pages, nkv, page, d), 7.0, dtype=torch.bfloat16, device="cuda")
+            v_cache = torch.full((pages, nkv, d, page), 7.0, dtype=torch.bfloat16, device="cuda")
+            for splits in (None, 1, 3):
+                partial = ops.skinny_gemm_splitk(x, w, splits=splits, packed=ops.packed_weight(w))
+                q = ops.rope_kv_write_partial(partial, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, bias=use_bias)
+                bound = dict(rtol=1e-2, atol=1e-2 * scale)
+                torch.testing.assert_close(q[:, : nh * d].float(), wide[:, : nh * d], **bound)
+                torch.testing.assert_close(k_cache.float(), k32, **bound)
+                torch.testing.assert_close(v_cache.float(), v32, **bound)
+            # the route the engine takes for this many rows is this one
+            k2, v2 = torch.full_like(k_cache, 7.0), torch.full_like(v_cache, 7.0)
+            q2 = ops.qkv_rope_write(x, w, use_bias, nh, nkv, d, positions, cos, sin, slots, k2, v2, page)
+            torch.testing.assert_close(q2[:, : nh * d].float(), wide[:, : nh * d], rtol=1e-2, atol=1e-2 * scale)
+            torch.testing.assert_close(k2.float(), k32, rtol=1e-2, atol=1e-2 * scale)
+    # a layer that reads another layer's cache writes nothing
+    before = k_cache.clone()
+    ops.qkv_rope_write(x, w, bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, write_kv=False)
+    assert torch.equal(before, k_cache)
+
+
 @pytest.mark.parametrize("m", [1, 7, 16])
 @pytest.mark.parametrize("hidden,inner", [(64, 128), (3584, 3584), (200, 320), (96, 18944)])
 def test_residual_add_and_norm_split_between_two_products(ops, ref, m, hidden, inner):

@@ -282,16 +282,57 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
 
 // The same with 16-byte accesses, for the usual case that the whole head rotates (2 * half == d) or nothing does.
 // An item is a run of N = 16 / sizeof(T) channels of the low half of a head together with the matching run of the high half.
-template <typename T>
-__global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, const float* __restrict__ bias, const int* __restrict__ positions,
-                                         const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+// PARTIAL = true: the rows come as `parts` float32 partial sums, partial[s][token][column] (what the split-K product
+// leaves), added here in the order s = 0, 1, ...; qkv is then only written.  Otherwise qkv is read and written in place.
+template <typename T, bool PARTIAL>
+struct RowSource {
+  const T* qkv;
+  const float* partial;
+  int parts;
+  size_t part_stride;  // elements between two partial sums
+  __device__ __forceinline__ float at(size_t index) const {
+    if constexpr (PARTIAL) {
+      float sum = partial[index];
+      for (int s = 1; s < parts; ++s) sum += partial[s * part_stride + index];
+      return sum;
+    } else {
+      return to_f32(qkv[index]);
+    }
+  }
+  // N consecutive elements from a 16-byte aligned index
+  template <int N> __device__ __forceinline__ void run(size_t index, float* out) const {
+    if constexpr (PARTIAL) {
+#pragma unroll
+      for (int piece = 0; piece < N / 4; ++piece) reinterpret_cast<float4_t*>(out)[piece] = reinterpret_cast<const float4_t*>(partial + index)[piece];
+      for (int s = 1; s < parts; ++s) {
+#pragma unroll
+        for (int piece = 0; piece < N / 4; ++piece) {
+          const float4_t more = reinterpret_cast<const float4_t*>(partial + s * part_stride + index)[piece];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) out[4 * piece + j] += more[j];
+        }
+      }
+    } else {
+      const float4_t raw = *reinterpret_cast<const float4_t*>(qkv + index);
+      const T* values = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+      for (int j = 0; j < N; ++j) out[j] = to_f32(values[j]);
+    }
+  }
+};
+
+template <typename T, bool PARTIAL>
+__global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, const float* __restrict__ partial, int parts, const float* __restrict__ bias,
+                                         const int* __restrict__ positions, const float* __restrict__ cos_table, const float* __restrict__ sin_table,
                                          const int* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache,
                                          int nh, int nkv, int d, int page_size, int write_kv) {
   constexpr int N = 16 / sizeof(T);
   const int t = blockIdx.x;
   const int half = d / 2;
   const int width = (nh + 2 * nkv) * d;
-  T* row = qkv + (size_t)t * width;
+  const RowSource<T, PARTIAL> source{qkv, partial, parts, (size_t)gridDim.x * width};
+  const size_t row_at = (size_t)t * width;
+  T* row = qkv + row_at;
   const int pos = positions[t];
   const float* cs = cos_table ? cos_table + (size_t)pos * half : nullptr;
   const float* sn = sin_table ? sin_table + (size_t)pos * half : nullptr;
@@ -307,10 +348,9 @@ __global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, const float* __res
     const int head = local / runs;
     const int c0 = (local % runs) * N;
     const int base = (is_k ? nh * d : 0) + head * d;
-    float4_t lo_v = *reinterpret_cast<const float4_t*>(row + base + c0);
-    float4_t hi_v = *reinterpret_cast<const float4_t*>(row + base + half + c0);
-    T* lo = reinterpret_cast<T*>(&lo_v);
-    T* hi = reinterpret_cast<T*>(&hi_v);
+    __attribute__((aligned(16))) float x_lo[N], x_hi[N];
+    source.template run<N>(row_at + base + c0, x_lo);
+    source.template run<N>(row_at + base + half + c0, x_hi);
     // bias and angles of the run, as 16-byte loads (c0 and half are multiples of N, the tables' rows of half)
     __attribute__((aligned(16))) float b_lo[N], b_hi[N], cos_run[N], sin_run[N];
 #pragma unroll
@@ -321,9 +361,12 @@ __global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, const float* __res
       reinterpret_cast<float4_t*>(cos_run)[piece] = cs ? reinterpret_cast<const float4_t*>(cs + c0)[piece] : zero;
       reinterpret_cast<float4_t*>(sin_run)[piece] = sn ? reinterpret_cast<const float4_t*>(sn + c0)[piece] : zero;
     }
+    float4_t lo_v, hi_v;
+    T* lo = reinterpret_cast<T*>(&lo_v);
+    T* hi = reinterpret_cast<T*>(&hi_v);
 #pragma unroll
     for (int j = 0; j < N; ++j) {
-      const float x0 = to_f32(lo[j]) + b_lo[j], x1 = to_f32(hi[j]) + b_hi[j];
+      const float x0 = x_lo[j] + b_lo[j], x1 = x_hi[j] + b_hi[j];
       float y0 = x0, y1 = x1;
       if (cs) {
         y0 = x0 * cos_run[j] - x1 * sin_run[j];
@@ -354,7 +397,7 @@ __global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, const float* __res
       // neighbouring lanes take neighbouring channels, so that a store instruction touches as few cache lines as the layout allows
       for (int item = threadIdx.x; item < nkv * d; item += blockDim.x) {
         const int head = item / d, c = item % d;
-        float x = to_f32(row[v_base + item]);
+        float x = source.at(row_at + v_base + item);
         if (bias) x += bias[v_base + item];
         v_cache[((page * nkv + head) * d + c) * page_size + offset] = from_f32<T>(x);
       }
@@ -364,7 +407,7 @@ __global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, const float* __res
         const float b = bias ? bias[v_base + item] : 0.f;
         __attribute__((aligned(16))) T run[RUN];
 #pragma unroll
-        for (int j = 0; j < RUN; ++j) run[j] = from_f32<T>(to_f32(qkv[(size_t)(t + j) * width + v_base + item]) + b);
+        for (int j = 0; j < RUN; ++j) run[j] = from_f32<T>(source.at((size_t)(t + j) * width + v_base + item) + b);
         T* dst = v_cache + ((page * nkv + head) * d + c) * page_size + offset;
 #pragma unroll
         for (int piece = 0; piece < (int)(RUN * sizeof(T) / 16); ++piece)
@@ -372,6 +415,21 @@ __global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, const float* __res
       }
     }
   }
+}
+
+// Rows that come as float32 partial sums partial[parts][tokens][(nh + 2 nkv) d] (bfloat16 only): their sum, plus bias, is
+// rotated; queries go to qkv[tokens][(nh + 2 nkv) d] (only the query columns are written), keys and values to the cache.
+// Needs a rotation of the whole head or none, d / 2 a multiple of 8, and 16-byte aligned operands.
+extern "C" int velox_rope_kv_write_partial_bf16(void* qkv, const float* partial, int parts, const float* bias, const int* positions,
+                                                const float* cos_table, const float* sin_table, int half, const int* slots, void* k_cache,
+                                                void* v_cache, int tokens, int nh, int nkv, int d, int page_size, int write_kv, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  const bool whole_head = (cos_table == nullptr || 2 * half == d) && (d / 2) % 8 == 0;
+  const bool aligned = (((uintptr_t)qkv | (uintptr_t)partial | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)bias | (uintptr_t)cos_table | (uintptr_t)sin_table) & 15) == 0;
+  if (!whole_head || !aligned || parts < 1) return (int)hipErrorInvalidValue;
+  rope_kv_write_vec_kernel<bf16_t, true><<<tokens, 256, 0, stream>>>((bf16_t*)qkv, partial, parts, bias, positions, cos_table, sin_table, slots,
+                                                                    (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, page_size, write_kv);
+  VELOX_RETURN_LAUNCH_STATUS();
 }
 
 extern "C" int velox_rope_kv_write(void* qkv, const float* bias, const int* positions, const float* cos_table, const float* sin_table,
@@ -383,10 +441,10 @@ extern "C" int velox_rope_kv_write(void* qkv, const float* bias, const int* posi
   const bool aligned = (((uintptr_t)qkv | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)bias | (uintptr_t)cos_table | (uintptr_t)sin_table) & 15) == 0;
   if (whole_head && aligned) {
     if (dtype == VELOX_BF16)
-      rope_kv_write_vec_kernel<bf16_t><<<tokens, 256, 0, stream>>>((bf16_t*)qkv, bias, positions, cos_table, sin_table, slots,
+      rope_kv_write_vec_kernel<bf16_t, false><<<tokens, 256, 0, stream>>>((bf16_t*)qkv, nullptr, 0, bias, positions, cos_table, sin_table, slots,
                                                                   (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, page_size, write_kv);
     else
-      rope_kv_write_vec_kernel<float><<<tokens, 256, 0, stream>>>((float*)qkv, bias, positions, cos_table, sin_table, slots,
+      rope_kv_write_vec_kernel<float, false><<<tokens, 256, 0, stream>>>((float*)qkv, nullptr, 0, bias, positions, cos_table, sin_table, slots,
                                                                  (float*)k_cache, (float*)v_cache, nh, nkv, d, page_size, write_kv);
     VELOX_RETURN_LAUNCH_STATUS();
   }

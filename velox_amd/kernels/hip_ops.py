@@ -72,6 +72,8 @@ class HipOps:
         c.velox_skinny_qkv_rotary_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _P]
         c.velox_silu_mul.argtypes = [_P, _P, _I, _I, _I, _P]
         c.velox_rope_kv_write.argtypes = [_P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_rope_kv_write_partial_bf16.argtypes = [_P, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_rope_kv_write_partial_bf16.restype = _I
         c.velox_gemm_fma.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
         c.velox_skinny_gemm_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _P]
         c.velox_skinny_residual_norm_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]
@@ -479,6 +481,37 @@ class HipOps:
             tokens, num_heads, num_kv_heads, head_dim, block_size, 1 if write_kv else 0, _code(qkv.dtype), self._stream())
         self._launched(status, "rope_kv_write")
 
+    def rope_kv_write_partial(self, partial, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size,
+                              write_kv=True, bias=None) -> torch.Tensor:
+        """``rope_kv_write`` on rows that come as float32 partial sums ``[S, M, (heads + 2 kv_heads) * head_dim]`` (bfloat16
+        caches): returns bfloat16 ``[M, width]`` whose query columns hold the rotated queries (the others are not written)."""
+        if partial.dim() != 3:
+            raise KernelError("rope_kv_write_partial: partial sums are [S, M, width]")
+        parts, tokens, width = partial.shape
+        if width != (num_heads + 2 * num_kv_heads) * head_dim or head_dim % 16 != 0:
+            raise KernelError(f"rope_kv_write_partial: rows of {width} elements do not hold {num_heads} + 2 x {num_kv_heads} heads of {head_dim}")
+        self._check("partial", partial, torch.float32, (parts, tokens, width), align=16)
+        self._check("positions", positions, torch.int32, (tokens,))
+        self._check("slot_mapping", slot_mapping, torch.int32, (tokens,))
+        if bias is not None:
+            self._check("bias", bias, torch.float32, (width,), align=16)
+        half = 0
+        if cos is not None:
+            self._check("cos", cos, torch.float32, align=16)
+            self._check("sin", sin, torch.float32, tuple(cos.shape), align=16)
+            half = cos.shape[1]
+            if 2 * half != head_dim:
+                raise KernelError("rope_kv_write_partial: the rotation has to span the whole head")
+        pages = k_cache.shape[0]
+        self._check("k_cache", k_cache, torch.bfloat16, (pages, num_kv_heads, block_size, head_dim), align=16)
+        self._check("v_cache", v_cache, torch.bfloat16, (pages, num_kv_heads, head_dim, block_size), align=16)
+        out = torch.empty((tokens, width), dtype=torch.bfloat16, device=self.device)
+        status = self._core.velox_rope_kv_write_partial_bf16(
+            _ptr(out), _ptr(partial), parts, _ptr(bias), _ptr(positions), _ptr(cos), _ptr(sin), half, _ptr(slot_mapping), _ptr(k_cache), _ptr(v_cache),
+            tokens, num_heads, num_kv_heads, head_dim, block_size, 1 if write_kv else 0, self._stream())
+        self._launched(status, "rope_kv_write_partial")
+        return out
+
     def qkv_rope_write(self, x, weight, bias, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache,
                        block_size, write_kv=True, waves: Optional[int] = None, fused: Optional[bool] = None) -> torch.Tensor:
         """Projects ``x`` with ``weight = [Wq; Wk; Wv]``, adds ``bias``, rotates queries and keys and writes keys and values
@@ -497,6 +530,15 @@ class HipOps:
         elif fused and not can_fuse:
             raise KernelError("qkv_rope_write: this call cannot run fused")
         if not fused:
+            n = weight.shape[0]
+            if (deferred is None and self.use_skinny_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16
+                    and 16 < m <= 64 and k % 64 == 0 and n <= 8192 and n == (num_heads + 2 * num_kv_heads) * head_dim and head_dim % 16 == 0
+                    and (cos is None or 2 * cos.shape[1] == head_dim)):
+                # 17 .. 64 rows: the split-K kernel streams the weight faster than the library's choice (measured on
+                # MI355X: 15 us against 21 for 4608 x 3584 at 64 rows), and the rotation adds its partial sums
+                partial = self.skinny_gemm_splitk(x, weight, packed=self.packed_weight(weight))
+                return self.rope_kv_write_partial(partial, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache,
+                                                  block_size, write_kv=write_kv, bias=bias)
             qkv = self.linear(deferred if deferred is not None else x, weight, None, x.dtype)
             self.rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size,
                                write_kv=write_kv, bias=bias)
