@@ -98,10 +98,21 @@ __global__ void add_rmsnorm_rows_in_registers_kernel(float* __restrict__ residua
     if (at < hidden) {
       r[c] = *reinterpret_cast<const float4_t*>(res + at);
       if (del) {
-        for (int p = 0; p < partials; ++p) {
-          const Quad<TD> d = *reinterpret_cast<const Quad<TD>*>(del + p * partial_stride + at);
+        // four partial sums are asked for together (the last one again where fewer are left) and added in order
+        for (int p = 0; p < partials; p += 4) {
+          Quad<TD> d[4];
 #pragma unroll
-          for (int j = 0; j < 4; ++j) r[c][j] += d.get(j);
+          for (int u = 0; u < 4; ++u) {
+            const int pu = p + u < partials ? p + u : partials - 1;
+            d[u] = *reinterpret_cast<const Quad<TD>*>(del + pu * partial_stride + at);
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            if (p + u < partials) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) r[c][j] += d[u].get(j);
+            }
+          }
         }
       }
       if (write_back) *reinterpret_cast<float4_t*>(res + at) = r[c];
@@ -303,13 +314,24 @@ struct RowSource {
   template <int N> __device__ __forceinline__ void run(size_t index, float* out) const {
     if constexpr (PARTIAL) {
 #pragma unroll
-      for (int piece = 0; piece < N / 4; ++piece) reinterpret_cast<float4_t*>(out)[piece] = reinterpret_cast<const float4_t*>(partial + index)[piece];
-      for (int s = 1; s < parts; ++s) {
+      for (int j = 0; j < N; ++j) out[j] = 0.f;
+      // three partial sums are asked for together (the last one again where fewer are left) and added in order
+      for (int s = 0; s < parts; s += 3) {
+        float4_t more[3][N / 4];
 #pragma unroll
-        for (int piece = 0; piece < N / 4; ++piece) {
-          const float4_t more = reinterpret_cast<const float4_t*>(partial + s * part_stride + index)[piece];
+        for (int u = 0; u < 3; ++u) {
+          const int su = s + u < parts ? s + u : parts - 1;
 #pragma unroll
-          for (int j = 0; j < 4; ++j) out[4 * piece + j] += more[j];
+          for (int piece = 0; piece < N / 4; ++piece) more[u][piece] = reinterpret_cast<const float4_t*>(partial + su * part_stride + index)[piece];
+        }
+#pragma unroll
+        for (int u = 0; u < 3; ++u) {
+          if (s + u < parts) {
+#pragma unroll
+            for (int piece = 0; piece < N / 4; ++piece)
+#pragma unroll
+              for (int j = 0; j < 4; ++j) out[4 * piece + j] += more[u][piece][j];
+          }
         }
       }
     } else {
