@@ -342,15 +342,16 @@ class HipOps:
     @staticmethod
     def pack_rows(weight: torch.Tensor, matrices: int = 1) -> torch.Tensor:
         """``weight`` [N, K] bfloat16 (``matrices`` stacked matrices of N / matrices rows each) in the order the skinny
-        kernels' lanes read it: [row tile of 16][block of 64 indices][lane = 16 * (index / 16) + row][16 elements], each
-        matrix padded with zero rows to whole tiles.  A wave's load of a block is then one contiguous kilobyte."""
+        kernels' lanes read it: [row tile of 16][block of 64 indices][half h][lane = 16 * g + row][8 elements] holds index
+        ``16 g + 8 h + e`` of the block; each matrix is padded with zero rows to whole tiles.  Each of a wave's two loads of
+        a block is then one contiguous kilobyte."""
         n_all, k = weight.shape
         n = n_all // matrices
         tiles = (n + 15) // 16
         padded = torch.zeros((matrices, tiles * 16, k), dtype=weight.dtype, device=weight.device)
         padded[:, :n] = weight.view(matrices, n, k)
-        # [matrix, tile, row i, block, group g, 16] -> [matrix, tile, block, g, i, 16]
-        return padded.view(matrices, tiles, 16, k // 64, 4, 16).permute(0, 1, 3, 4, 2, 5).contiguous().view(-1)
+        # [matrix, tile, row i, block, group g, half h, 8] -> [matrix, tile, block, h, g, i, 8]
+        return padded.view(matrices, tiles, 16, k // 64, 4, 2, 8).permute(0, 1, 3, 5, 4, 2, 6).contiguous().view(-1)
 
     def skinny_gemm(self, x, weight, bias, out_dtype, waves: Optional[int] = None, row_tiles: Optional[int] = None, packed: Optional[torch.Tensor] = None, n: Optional[int] = None,
                     row_scale: Optional[DeferredNorm] = None):
