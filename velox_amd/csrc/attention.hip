@@ -529,12 +529,33 @@ __device__ __forceinline__ void mask_frag(Frag<bf16_t>& f, int valid) {
 
 // Decode: every sequence brings one token, and the G <= 16 query heads of a KV head are the 16 columns of the
 // MFMA tiles.  The step is bound by reading the cache once, so nothing is staged: each wave streams its own
-// 16-key tiles straight from global memory into MFMA operands (K rows as [key i][channels 16c + 4g ..], V^T rows
-// as [channel 16c + i][keys 4g ..], both 8- or 16-byte loads of contiguous cache lines), two tiles ahead of the
+// 16-key tiles straight from global memory into MFMA operands (K rows as [key i][channels 16c + 4g ..], or
+// [channels 32c + 8g ..] where KeyOps below allows, V^T rows as [channel 16c + i][keys 4g ..], 8- or 16-byte loads of
+// contiguous cache lines), two tiles ahead of the
 // arithmetic, with no barrier in the loop.  The page ids of the workgroup's key range are copied into LDS first, so
 // that a tile's addresses do not wait for a second trip to memory.  The WAVES waves of a workgroup interleave the
 // tiles of one (sequence, KV head, split) and merge their running (max, sum, output) through LDS at the end.
 constexpr int DECODE_PAGE_IDS = 2048;
+
+// Operands of S^T = K Q^T in the decode kernel.  For bfloat16 heads of a multiple of 32 channels a lane reads 16 bytes of
+// its key's row (channels 32c + 8g ..) and one v_mfma_f32_16x16x32_bf16 takes them: half as many loads, each touching
+// half as many cache lines, as with the 16-channel fragments that every other case uses.
+template <typename T, bool WIDE> struct KeyOps {
+  static constexpr int STEPS = D / 16, SPAN = 16, LANE = 4;
+  typedef Frag<T> Operand;
+  static __device__ __forceinline__ Operand load(const T* p) { return load_frag<T>(p); }
+  static __device__ __forceinline__ Operand zero() { return zero_frag<T>(); }
+  static __device__ __forceinline__ float4_t mma(const Operand& a, const Operand& b, float4_t c) { return mma16(a, b, c); }
+};
+template <> struct KeyOps<bf16_t, true> {
+  static constexpr int STEPS = D / 32, SPAN = 32, LANE = 8;
+  typedef bf16x8_t Operand;
+  static __device__ __forceinline__ Operand load(const bf16_t* p) { return *reinterpret_cast<const bf16x8_t*>(p); }
+  static __device__ __forceinline__ Operand zero() { return __builtin_bit_cast(bf16x8_t, float4_t{0.f, 0.f, 0.f, 0.f}); }
+  static __device__ __forceinline__ float4_t mma(const Operand& a, const Operand& b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
 
 template <typename T, int DEPTH, int WAVES>
 __global__ void __launch_bounds__(64 * WAVES) decode_attention_kernel(
@@ -544,6 +565,7 @@ __global__ void __launch_bounds__(64 * WAVES) decode_attention_kernel(
     int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens) {
   constexpr int NC = D / 16;
   constexpr int NCW = (NC + WAVES - 1) / WAVES;
+  typedef KeyOps<T, sizeof(T) == 2 && D % 32 == 0> KO;
   __shared__ __attribute__((aligned(16))) float4_t acc_all[WAVES * NC * 64];
   __shared__ float m_all[WAVES * 16];
   __shared__ float l_all[WAVES * 16];
@@ -586,13 +608,13 @@ __global__ void __launch_bounds__(64 * WAVES) decode_attention_kernel(
     for (int p = tid + 64 * WAVES; p < num_pages && p < DECODE_PAGE_IDS; p += 64 * WAVES) page_ids[p] = table[first_page + p];
   }
 
-  Frag<T> qf[NC];
+  typename KO::Operand qf[KO::STEPS];
   {
-    const T* qp = qkv + (size_t)b * qkv_stride + (size_t)head * D + 4 * g;
+    const T* qp = qkv + (size_t)b * qkv_stride + (size_t)head * D + KO::LANE * g;
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
-      qf[c] = load_frag<T>(qp + 16 * c);
-      if (!row_ok) qf[c] = zero_frag<T>();
+    for (int c = 0; c < KO::STEPS; ++c) {
+      qf[c] = KO::load(qp + KO::SPAN * c);
+      if (!row_ok) qf[c] = KO::zero();
     }
   }
   __syncthreads();
@@ -604,7 +626,7 @@ __global__ void __launch_bounds__(64 * WAVES) decode_attention_kernel(
   };
 
   struct Tile {
-    Frag<T> k[NC];
+    typename KO::Operand k[KO::STEPS];
     Frag<T> v[NC];
   };
   // No branch surrounds a load, so the loads of a tile do not wait for those of the tiles before it: a key beyond the
@@ -615,12 +637,18 @@ __global__ void __launch_bounds__(64 * WAVES) decode_attention_kernel(
     int n_v = n_begin + 16 * t + 4 * g;  // the first of the four keys whose values this lane reads
     n_k = n_k < kv_len ? n_k : kv_len - 1;
     n_v = n_v < kv_len ? n_v : (kv_len - 1) & ~3;
-    const T* kp = k_cache + ((page_of(n_k) * nkv + kvh) * page_size + (n_k & (page_size - 1))) * D + 4 * g;
+    const T* kp = k_cache + ((page_of(n_k) * nkv + kvh) * page_size + (n_k & (page_size - 1))) * D + KO::LANE * g;
     const T* vp = v_cache + ((page_of(n_v) * nkv + kvh) * D + i) * page_size + (n_v & (page_size - 1));
 #pragma unroll
-    for (int c = 0; c < NC; ++c) tile.k[c] = load_frag<T>(kp + 16 * c);
+    for (int c = 0; c < KO::STEPS; ++c) tile.k[c] = KO::load(kp + KO::SPAN * c);
 #pragma unroll
-    for (int c = 0; c < NC; ++c) tile.v[c] = load_frag<T>(vp + (size_t)16 * c * page_size);
+    // (values are read once and a load instruction covers whole cache lines of V^T where pages hold 16 tokens: the
+    // non-temporal hint then streams them faster, 80 us against 96 for 537 MB on MI355X; on the half lines of a K
+    // load it costs speed)
+    for (int c = 0; c < NC; ++c) {
+      if constexpr (sizeof(T) == 4) tile.v[c].v = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(vp + (size_t)16 * c * page_size));
+      else tile.v[c].v = __builtin_nontemporal_load(reinterpret_cast<const short4_t*>(vp + (size_t)16 * c * page_size));
+    }
   };
 
   float m_i = -INFINITY, l_i = 0.f;
@@ -636,7 +664,7 @@ __global__ void __launch_bounds__(64 * WAVES) decode_attention_kernel(
     }
     float4_t s = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int c = 0; c < NC; ++c) s = mma16(tile.k[c], qf[c], s);
+    for (int c = 0; c < KO::STEPS; ++c) s = KO::mma(tile.k[c], qf[c], s);
     float mx = -INFINITY;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -692,9 +720,12 @@ __global__ void __launch_bounds__(64 * WAVES) decode_attention_kernel(
     // those loads behind the loop's exit tests, to the place of their use, where nothing hides their latency.
     if (splits < 0) {
 #pragma unroll
-      for (int s = 0; s < DEPTH; ++s)
+      for (int s = 0; s < DEPTH; ++s) {
 #pragma unroll
-        for (int c = 0; c < NC; ++c) acc_o[c] = mma16(ring[s].v[c], ring[s].k[c], acc_o[c]);
+        for (int c = 0; c < NC; ++c) acc_o[c] = mma16(ring[s].v[c], ring[s].v[c], acc_o[c]);
+#pragma unroll
+        for (int c = 0; c < KO::STEPS; ++c) acc_o[0] = KO::mma(ring[s].k[c], ring[s].k[c], acc_o[0]);
+      }
     }
   }
 
