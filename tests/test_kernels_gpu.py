@@ -268,7 +268,7 @@ def test_qkv_projection_at_17_to_64_rows_with_partial_sums_added_by_the_rotation
 
 
 @pytest.mark.parametrize("m", [1, 7, 16])
-@pytest.mark.parametrize("hidden,inner", [(64, 128), (3584, 3584), (200, 320), (96, 18944)])
+@pytest.mark.parametrize("hidden,inner", [(64, 128), (3584, 3584), (200, 320), (96, 18944), (5120, 192), (8192, 64)])
 def test_residual_add_and_norm_split_between_two_products(ops, ref, m, hidden, inner):
     """The decode fusion: a product adds itself to the residual and applies the norm weight (DeferredNorm); the next
     product (plain, gate/up + SiLU, or q/k/v with rotation) scales its rows.  Against residual add -> RMSNorm -> product
@@ -308,6 +308,11 @@ def test_residual_add_and_norm_split_between_two_products(ops, ref, m, hidden, i
     torch.testing.assert_close(ops.linear(deferred, w_next, bias, torch.float32), ref.linear(normed_bf16, w_next, bias, torch.float32), **tol)  # unregistered: materialised
     ops.register_weight(w_next)
     torch.testing.assert_close(ops.linear(deferred, w_next, bias, torch.float32), ref.linear(normed_bf16, w_next, bias, torch.float32), **tol)
+    # 64 rows of the weight per wave (the variant for very tall weights), four and eight waves
+    for waves in (4, 8):
+        if hidden // 16 <= 64 * waves:
+            got = ops.skinny_gemm(deferred.x, w_next, bias, torch.float32, waves=waves, row_tiles=4, packed=ops.packed_weight(w_next), row_scale=deferred)
+            torch.testing.assert_close(got, ref.linear(normed_bf16, w_next, bias, torch.float32), **tol)
     ops.register_weight(w_next, stacked=2)
     want_glu = ref.linear_silu_mul(normed_bf16, w_next, torch.bfloat16).float()
     torch.testing.assert_close(ops.linear_silu_mul(deferred, w_next, torch.bfloat16).float(), want_glu, rtol=3e-2, atol=3e-2 * float(want_glu.abs().max()))

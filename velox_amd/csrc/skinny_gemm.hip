@@ -58,11 +58,20 @@ __device__ __forceinline__ Run16 zero_run() {
 // PACKED = true: W is stored tile by tile in the order the lanes read it, [row tile of 16][block of 64 indices][half of a
 // run][lane][8 elements] (rows padded with zeros to a multiple of 16; for GLU gate and up are padded separately), so that
 // each of a wave's two loads of a block is one contiguous kilobyte.
+struct NoHooks {
+  __device__ __forceinline__ void after_first() const {}
+  __device__ __forceinline__ void before_barrier() const {}
+};
+
 // The products of one workgroup: every wave multiplies its share of K and leaves its sums in partial[wave]; after
 // the barrier at the end each tile's sum is partial[0][tile] + partial[1][tile] + ... (to be added in that order).
-template <int RT, int CT, int WAVES, bool GLU, bool PACKED>
+// hooks.after_first() runs once, behind the first round of loads and products: the place for loads that the epilogue
+// needs and whose addresses depend on loads issued before this function (they then fly with the second round of
+// weights).  hooks.before_barrier() runs behind the main loop, before the barrier: the place to leave further things
+// in LDS for the epilogue.
+template <int RT, int CT, int WAVES, bool GLU, bool PACKED, typename Hooks = NoHooks>
 __device__ __forceinline__ void skinny_partial_sums(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, int m, int n, int k,
-                                                    float4_t (&partial)[WAVES][RT * CT][64]) {
+                                                    float4_t (&partial)[WAVES][RT * CT][64], Hooks hooks = Hooks()) {
   constexpr int UNROLL = 4;  // blocks of 64 indices whose loads are issued together
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int g = lane >> 4, i = lane & 15;
@@ -129,18 +138,20 @@ __device__ __forceinline__ void skinny_partial_sums(const bf16_t* __restrict__ a
           acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wr[u][rt].lo, ar[u][ct].lo, acc[rt][ct], 0, 0, 0);
           acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wr[u][rt].hi, ar[u][ct].hi, acc[rt][ct], 0, 0, 0);
         }
+    if (kb == kb_lo) hooks.after_first();
   }
 
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) partial[wave][rt * CT + ct][lane] = acc[rt][ct];
+  hooks.before_barrier();
   __syncthreads();
 }
 
 // Rows of A that still have to be normalised: A holds x * norm_weight in bfloat16 and the producer (the kernel
 // below that adds a product to the residual stream) left sums of squares of x, one per workgroup and row; a product with
-// such an A is scaled row by row with rstd[m] = rsqrt(sum_b partial[b][m] / width + eps) in its epilogue, which is the
+// such an A is scaled row by row with rstd[m] = rsqrt(sum_b partial[m][b] / width + eps) in its epilogue, which is the
 // same as normalising A first.  The sums are added in a fixed order.  Only for M <= 16.
 struct RowScale {
   const float* partial;  // [16][blocks] (row m's sums are contiguous), or null: rows are used as they are
@@ -148,46 +159,93 @@ struct RowScale {
   float inv_width, eps;
 };
 
-// The table of sums is copied into LDS by loads that write LDS directly: issued before the main loop, they fly while
-// the weights stream and hold no registers meanwhile.  After the main loop's barrier row_scale_of adds a row's entries.
-constexpr int ROW_SCALE_BLOCKS = 512;  // room in LDS: residual widths up to 16 * 512
+// How a workgroup adds a row's sums: wave v takes the blocks [v * share, (v + 1) * share), lane (g, row) of it every fourth
+// of them.  The loads write LDS directly (lane's value of round t lands at stage[wave][t][lane]): issued before the
+// weights stream, they hold no registers meanwhile and are back long before the main loop ends, so no trip to memory
+// is left for the epilogue.  Behind the main loop a wave reads its own values back, adds them and leaves one number
+// per row in LDS; whoever needs rstd[m] adds the waves' numbers in wave order.
+constexpr int ROW_SCALE_ROUNDS = 16;      // loads per lane: residual widths up to 16 * 64 * WAVES
+constexpr int ROW_SCALE_BLOCKS = 64 * 8;  // what the eight-wave kernels take
 
 template <int WAVES>
-__device__ __forceinline__ void row_scale_copy(const RowScale& rs, int m, float* table) {
-  if (rs.partial == nullptr) return;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int count = rs.blocks * m;  // the rows in use come first
-  for (int first = wave * 64; first < count; first += WAVES * 64) {
-    const int at = first + lane < count ? first + lane : count - 1;  // (the spare lanes of a last pass repeat the last entry)
-    // lane's 4 bytes land at table[first + lane]
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(rs.partial + at),
-                                     (__attribute__((address_space(3))) void*)(table + first), 4, 0, 0);
+struct RowScaleLoads {
+  typedef float Stage[WAVES][ROW_SCALE_ROUNDS][64];
+  struct Share {
+    int first, end, rounds;  // this lane's first block, the end of its wave's share, loads per lane
+  };
+  // (computed where it is needed rather than kept: the main loop has no registers to spare)
+  static __device__ __forceinline__ Share share_of(const RowScale& rs) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int share = ((rs.blocks + WAVES - 1) / WAVES + 3) & ~3;
+    return Share{wave * share + (lane >> 4), (wave + 1) * share < rs.blocks ? (wave + 1) * share : rs.blocks, share / 4};
   }
-}
 
-// after the barrier that follows the main loop; every lane of the wave has to call it (l = its lane)
-__device__ __forceinline__ float row_scale_of(const RowScale& rs, int m, const float* table, int l) {
+  static __device__ __forceinline__ void issue(const RowScale& rs, int m, Stage& stage) {
+    if (rs.partial == nullptr) return;  // (the same for every thread of the launch)
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int row = (lane & 15) < m ? (lane & 15) : 0;  // (a row beyond M reads row 0's sums; nobody uses its scale)
+    const Share sh = share_of(rs);
+    const float* p = rs.partial + (size_t)row * rs.blocks;
+    for (int t = 0; t < sh.rounds; ++t) {
+      const int b = sh.first + 4 * t;  // (what lies beyond the share is read from the row's last block and dropped below)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(p + (b < sh.end ? b : rs.blocks - 1)),
+                                       (__attribute__((address_space(3))) void*)(&stage[wave][t][0]), 4, 0, 0);
+    }
+  }
+
+  // behind the main loop: this wave's part of every row's sum goes to part[wave][row]
+  static __device__ __forceinline__ void leave(const RowScale& rs, const Stage& stage, float (&part)[WAVES][16]) {
+    if (rs.partial == nullptr) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const Share sh = share_of(rs);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the wave's own loads into LDS have landed (the weights were waited for already)
+    float total = 0.f;
+    for (int t = 0; t < sh.rounds; ++t) total += sh.first + 4 * t < sh.end ? stage[wave][t][lane] : 0.f;
+    total += __shfl_xor(total, 16, VELOX_WAVE);  // the four lane groups took every fourth block: a fixed order
+    total += __shfl_xor(total, 32, VELOX_WAVE);
+    if (lane < 16) part[wave][lane] = total;
+  }
+};
+
+// after the barrier that follows the main loop
+template <int WAVES>
+__device__ __forceinline__ float row_scale_of(const RowScale& rs, const float (&part)[WAVES][16], int row) {
   if (rs.partial == nullptr) return 1.f;
-  const int row = l & 15, grp = l >> 4;
-  float total = 0.f;
-  if (row < m)
-    for (int b = grp; b < rs.blocks; b += 4) total += table[row * rs.blocks + b];
-  total += __shfl_xor(total, 16, VELOX_WAVE);  // the four lane groups took every fourth block: a fixed order
-  total += __shfl_xor(total, 32, VELOX_WAVE);
+  float total = part[0][row];
+#pragma unroll
+  for (int wv = 1; wv < WAVES; ++wv) total += part[wv][row];
   return rsqrtf(total * rs.inv_width + rs.eps);
 }
 
-// SCALED = true: the instantiation that can scale its rows (it carries the table in LDS); rs.partial is set then.
+template <int WAVES, typename After>
+struct ScaleHooks {
+  const RowScale& rs;
+  const typename RowScaleLoads<WAVES>::Stage& stage;
+  float (&part)[WAVES][16];
+  After after;
+  __device__ __forceinline__ void after_first() const { after(); }
+  __device__ __forceinline__ void before_barrier() const { RowScaleLoads<WAVES>::leave(rs, stage, part); }
+};
+struct Nothing {
+  __device__ __forceinline__ void operator()() const {}
+};
+
+// SCALED = true: the instantiation that can scale its rows; rs.partial is set then.
 template <int RT, int CT, int WAVES, typename TO, bool GLU = false, bool PACKED = false, bool SCALED = false>
 __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
                                                                  const float* __restrict__ bias, TO* __restrict__ out, int m, int n, int k,
                                                                  RowScale rs) {
   __shared__ float4_t partial[WAVES][RT * CT][64];
-  __shared__ float scale_table[SCALED ? ROW_SCALE_BLOCKS * 16 : 1];
+  __shared__ float scale_part[SCALED ? WAVES : 1][16];
+  __shared__ float scale_stage[SCALED ? WAVES : 1][SCALED ? ROW_SCALE_ROUNDS : 1][SCALED ? 64 : 1];
   constexpr int RTO = GLU ? RT / 2 : RT;
   const int n0 = blockIdx.x * 16 * RTO;
-  if constexpr (SCALED) row_scale_copy<WAVES>(rs, m, scale_table);
-  skinny_partial_sums<RT, CT, WAVES, GLU, PACKED>(a, w, m, n, k, partial);
+  if constexpr (SCALED) {
+    RowScaleLoads<WAVES>::issue(rs, m, scale_stage);
+    skinny_partial_sums<RT, CT, WAVES, GLU, PACKED>(a, w, m, n, k, partial, ScaleHooks<WAVES, Nothing>{rs, scale_stage, scale_part, Nothing()});
+  } else {
+    skinny_partial_sums<RT, CT, WAVES, GLU, PACKED>(a, w, m, n, k, partial);
+  }
   // add the waves' partial sums in wave order; each tile's 64 lanes are spread over the workgroup
   for (int item = threadIdx.x; item < RTO * CT * 64; item += WAVES * 64) {
     const int tile = item >> 6, l = item & 63;
@@ -196,7 +254,7 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
     for (int wv = 1; wv < WAVES; ++wv) sum += partial[wv][tile][l];
     float row_scale = 1.f;  // (unless the rows of A wait for their norm)
     if constexpr (SCALED) {
-      row_scale = row_scale_of(rs, m, scale_table, l);
+      row_scale = row_scale_of<WAVES>(rs, scale_part, l & 15);
       sum = sum * row_scale;
     }
     if constexpr (GLU) {
@@ -276,6 +334,7 @@ extern "C" int velox_skinny_gemm_bf16(const void* a, const void* w, const float*
                                       float inv_width, float eps, hipStream_t stream) {
   if (m <= 0 || n <= 0) return 0;
   if (k % 64 != 0 || m > 64 || (scale_partial != nullptr && (m > 16 || scale_blocks > ROW_SCALE_BLOCKS))) return -1;
+  if (scale_partial != nullptr && waves < 8) waves = 8;  // (rows are scaled by the eight-wave kernels)
   const RowScale rs{scale_partial, scale_blocks, inv_width, eps};
 #define PICK(RT, CT, W) return launch_skinny<RT, CT, W>(a, w, bias, out, m, n, k, out_dtype, packed != 0, rs, stream)
   if (m <= 16 && row_tiles >= 4) {
@@ -321,13 +380,36 @@ template <int WAVES>
 __global__ void __launch_bounds__(WAVES * 64) skinny_qkv_rotary_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
                                                                        RotaryWrite args, int m, int n, int k, RowScale rs) {
   __shared__ float4_t partial[WAVES][2][64];
-  __shared__ float scale_table[ROW_SCALE_BLOCKS * 16];
-  row_scale_copy<WAVES>(rs, m, scale_table);
-  skinny_partial_sums<2, 1, WAVES, false, true>(a, w, m, n, k, partial);
+  __shared__ float scale_part[WAVES][16];
+  __shared__ float scale_stage[WAVES][ROW_SCALE_ROUNDS][64];
+  // What the epilogue reads is asked for before and inside the main loop (no branch around a load: every thread asks, a
+  // row beyond M for row 0's; the first 64 threads use it): the slot and the position first, the bias and, behind the
+  // first round of weights, the angles at that position, so that none of these trips to memory is left for the end.
   const int l = threadIdx.x;
-  if (l >= 64) return;
-  const float row_scale = row_scale_of(rs, m, scale_table, l);
   const int row = l & 15;  // batch row
+  const int row_in = row < m ? row : 0;
+  const int d = args.d, half = d / 2;
+  const int pairs_per_head = d / 32;
+  const int head = blockIdx.x / pairs_per_head, j = blockIdx.x % pairs_per_head;
+  const int r4 = 4 * ((l & 63) >> 4);
+  const bool rotated = head < args.heads + args.kv_heads;
+  const int c = (rotated ? 16 : 32) * j + r4;  // first of four channels; their partners are half (16 for values) further on
+  const int slot = args.slots[row_in];
+  const int position = args.positions[row_in];
+  // (without a bias the same loads read the start of the angle table and their values are dropped)
+  const float* bias_at = args.bias ? args.bias + (size_t)head * d + c : args.cos_table;
+  float4_t bias_first = *reinterpret_cast<const float4_t*>(bias_at);
+  float4_t bias_second = *reinterpret_cast<const float4_t*>(bias_at + (args.bias ? (rotated ? half : 16) : 0));
+  float4_t cs = float4_t{1.f, 1.f, 1.f, 1.f}, sn = float4_t{0.f, 0.f, 0.f, 0.f};
+  auto fetch_angles = [&]() {
+    const size_t angle = (size_t)position * half + (rotated ? c : 0);
+    cs = *reinterpret_cast<const float4_t*>(args.cos_table + angle);
+    sn = *reinterpret_cast<const float4_t*>(args.sin_table + angle);
+  };
+  RowScaleLoads<WAVES>::issue(rs, m, scale_stage);
+  skinny_partial_sums<2, 1, WAVES, false, true>(a, w, m, n, k, partial, ScaleHooks<WAVES, decltype(fetch_angles)>{rs, scale_stage, scale_part, fetch_angles});
+  if (l >= 64) return;
+  const float row_scale = row_scale_of<WAVES>(rs, scale_part, row_in);
   if (row >= m) return;
   float4_t first = partial[0][0][l], second = partial[0][1][l];
 #pragma unroll
@@ -335,28 +417,12 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_qkv_rotary_kernel(const bf1
     first += partial[wv][0][l];
     second += partial[wv][1][l];
   }
-  first = first * row_scale;
-  second = second * row_scale;
-  const int d = args.d, half = d / 2;
-  const int pairs_per_head = d / 32;
-  const int head = blockIdx.x / pairs_per_head, j = blockIdx.x % pairs_per_head;
-  const int r4 = 4 * (l >> 4);
-  const int slot = args.slots[row];
+  if (!args.bias) bias_first = bias_second = float4_t{0.f, 0.f, 0.f, 0.f};
+  first = first * row_scale + bias_first;
+  second = second * row_scale + bias_second;
   const size_t page = (size_t)(slot / args.page_size);
   const int offset = slot % args.page_size;
-  if (head < args.heads + args.kv_heads) {
-    const int c = 16 * j + r4;  // channels c .. c + 3 of the low half and their partners
-    if (args.bias) {
-      const float* b = args.bias + (size_t)head * d + c;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        first[e] += b[e];
-        second[e] += b[half + e];
-      }
-    }
-    const size_t angle = (size_t)args.positions[row] * half + c;
-    const float4_t cs = *reinterpret_cast<const float4_t*>(args.cos_table + angle);
-    const float4_t sn = *reinterpret_cast<const float4_t*>(args.sin_table + angle);
+  if (rotated) {
     __attribute__((aligned(8))) bf16_t lo[4];
     __attribute__((aligned(8))) bf16_t hi[4];
 #pragma unroll
@@ -372,15 +438,6 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_qkv_rotary_kernel(const bf1
     *reinterpret_cast<float2_t*>(dst + half) = *reinterpret_cast<const float2_t*>(hi);
   } else {
     const int vh = head - args.heads - args.kv_heads;
-    const int c = 32 * j + r4;  // channels c .. c + 3 and c + 16 .. c + 19
-    if (args.bias) {
-      const float* b = args.bias + (size_t)head * d + c;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        first[e] += b[e];
-        second[e] += b[16 + e];
-      }
-    }
     bf16_t* dst = args.v_cache + ((page * args.kv_heads + vh) * d + c) * args.page_size + offset;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -477,6 +534,7 @@ extern "C" int velox_skinny_gemm_glu_bf16(const void* a, const void* w, void* ou
   if (m <= 0 || n <= 0) return 0;
   if (k % 64 != 0 || m > 32 || (scale_partial != nullptr && (m > 16 || scale_blocks > ROW_SCALE_BLOCKS))) return -1;
   const RowScale rs{scale_partial, scale_blocks, inv_width, eps};
+  if (scale_partial != nullptr && waves < 8) waves = 8;  // (rows are scaled by the eight-wave kernels)
   if (m <= 16) {
     if (pairs >= 2) {
       if (waves >= 8) return launch_skinny_glu<4, 1, 8>(a, w, out, m, n, k, packed != 0, rs, stream);

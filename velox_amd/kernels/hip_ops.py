@@ -551,7 +551,7 @@ class HipOps:
         self._check("positions", positions, torch.int32, (m,))
         self._check("slot_mapping", slot_mapping, torch.int32, (m,))
         if bias is not None:
-            self._check("bias", bias, torch.float32, (width,))
+            self._check("bias", bias, torch.float32, (width,), align=16)
         self._check("cos", cos, torch.float32, align=16)
         self._check("sin", sin, torch.float32, tuple(cos.shape), align=16)
         pages = k_cache.shape[0]
