@@ -333,6 +333,68 @@ def test_residual_add_and_norm_split_between_two_products(ops, ref, m, hidden, i
         torch.testing.assert_close(got, want, rtol=3e-2, atol=3e-2 * max(1.0, float(want.abs().max())))
 
 
+def _rows_from_lanes_order(twin, k):
+    """[k / 64 * 1024] in the order the skinny kernels' lanes read activations -> [16, k]."""
+    return twin.view(k // 64, 2, 4, 16, 8).permute(3, 0, 2, 1, 4).reshape(16, k)
+
+
+@pytest.mark.parametrize("m", [1, 5, 13, 16])
+def test_decode_activations_handed_on_in_the_lanes_order(ops, ref, m, monkeypatch):
+    """The gate/up kernel and the residual-add kernel leave their result a second time in the order the next product's
+    lanes read it; a product gives the same bits whether it reads that copy or the row-major one."""
+    from velox_amd.parts.base import DeferredNorm, ResidualSink
+    from velox_amd.parts.norms import RMSNorm
+
+    # (the engine asks for the copy from 13 rows on, where it pays; the kernels take any number up to 16)
+    monkeypatch.setattr(ops, "_room_for_packed_rows", lambda rows, n: torch.empty(n // 64 * 1024, dtype=torch.bfloat16, device="cuda") if rows <= 16 and n % 64 == 0 else None)
+    hidden, inner = 256, 448
+    x = rand((m, hidden), torch.bfloat16, 90)
+    w_gu = rand((2 * inner, hidden), torch.bfloat16, 91, 0.05)
+    w_down = rand((hidden, inner), torch.bfloat16, 92, 0.05)
+    ops.register_weight(w_gu, stacked=2)
+    ops.register_weight(w_down)
+    act = ops.linear_silu_mul(x, w_gu, torch.bfloat16)
+    twin, version = act._velox_packed_rows
+    assert version == act._version and torch.equal(_rows_from_lanes_order(twin, inner)[:m], act)
+    norm = RMSNorm("", hidden, 1e-6)
+    norm.weight = 1.0 + rand((hidden,), torch.float32, 93, 0.1)
+    results = []
+    for use_twin in (True, False):
+        source = act if use_twin else act.clone()  # (a clone is another tensor object: no copy hangs on it)
+        assert (ops._packed_rows_of(source, inner) is not None) == use_twin
+        residual = rand((m, hidden), torch.float32, 94)
+        deferred = ops.linear(source, w_down, None, torch.bfloat16, partials_ok=True, residual_norm=ResidualSink(residual, norm))
+        assert isinstance(deferred, DeferredNorm)
+        next_twin = ops._packed_rows_of(deferred.x, hidden)
+        assert torch.equal(_rows_from_lanes_order(next_twin, hidden)[:m], deferred.x)
+        results.append((residual, deferred.x.clone(), deferred.sums[:m].clone(), deferred))
+    for a, b in zip(results[0][:3], results[1][:3]):
+        assert torch.equal(a, b)
+    # the consumers of a DeferredNorm, with and without its copy
+    deferred = results[0][3]
+    plain = DeferredNorm(deferred.x.clone(), deferred.sums, deferred.width, deferred.eps, deferred.norm)
+    bias = rand((2 * inner,), torch.float32, 95)
+    assert torch.equal(ops.linear(deferred, w_gu, bias, torch.float32), ops.linear(plain, w_gu, bias, torch.float32))
+    assert torch.equal(ops.linear_silu_mul(deferred, w_gu, torch.bfloat16), ops.linear_silu_mul(plain, w_gu, torch.bfloat16))
+    nh, nkv, d, page, pages = 3, 2, 128, 16, 6  # (3 + 2 * 2) * 128 = 896 = 2 * inner rows
+    ops.register_weight(w_gu, rotary_heads=(nh, nkv, d))
+    positions = torch.arange(m, dtype=torch.int32, device="cuda") * 7
+    slots = (torch.randperm((pages - 1) * page, generator=torch.Generator().manual_seed(96))[:m] + page).to(torch.int32).cuda()
+    angles = torch.outer(torch.arange(128, dtype=torch.float32), 1.0 / (10000.0 ** (torch.arange(d // 2, dtype=torch.float32) / (d // 2))))
+    cos, sin = angles.cos().cuda(), angles.sin().cuda()
+    outs = []
+    for source in (deferred, plain):
+        k_cache = torch.zeros((pages, nkv, page, d), dtype=torch.bfloat16, device="cuda")
+        v_cache = torch.zeros((pages, nkv, d, page), dtype=torch.bfloat16, device="cuda")
+        q = ops.qkv_rope_write(source, w_gu, bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, fused=True)
+        outs.append((q, k_cache, v_cache))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    # a copy goes stale with its tensor
+    act.add_(1)
+    assert ops._packed_rows_of(act, inner) is None
+
+
 def _attention_case(dtype, nh, nkv, d, page, seqs, seed, garbage=False):
     """seqs: list of (q_len, kv_len).  Builds a paged cache with shuffled pages and a flat qkv."""
     g = torch.Generator().manual_seed(seed)

@@ -44,6 +44,15 @@ __device__ __forceinline__ Run16 load_run_packed(const bf16_t* p) {
   return r;
 }
 
+// the two halves `half` elements apart (8: one run of 32 bytes; 512: the packed layout, read through the caches)
+__device__ __forceinline__ Run16 load_run_halves(const bf16_t* p, int half) {
+  Run16 r;
+  const float4_t a = *reinterpret_cast<const float4_t*>(p), b = *reinterpret_cast<const float4_t*>(p + half);
+  r.lo = __builtin_bit_cast(bf16x8_t, a);
+  r.hi = __builtin_bit_cast(bf16x8_t, b);
+  return r;
+}
+
 __device__ __forceinline__ Run16 zero_run() {
   Run16 r;
   const float4_t z = {0.f, 0.f, 0.f, 0.f};
@@ -58,6 +67,15 @@ __device__ __forceinline__ Run16 zero_run() {
 // PACKED = true: W is stored tile by tile in the order the lanes read it, [row tile of 16][block of 64 indices][half of a
 // run][lane][8 elements] (rows padded with zeros to a multiple of 16; for GLU gate and up are padded separately), so that
 // each of a wave's two loads of a block is one contiguous kilobyte.
+// Activations in the order the lanes read them (M <= 16): [block of 64 indices][half h][lane = 16 g + row][8 elements]
+// holds index 16 g + 8 h + e of the block, the layout of one 16-row tile of a packed W.  A kernel that writes the
+// activations of the next product can leave them like this (beside the row-major copy); the next product's two loads
+// of a block are then one contiguous kilobyte each instead of sixteen pieces of sixteen rows.  Rows beyond M are never
+// written and hold whatever was there: they only reach output columns that nobody stores.
+__device__ __forceinline__ size_t packed_row_offset(int row, int index) {
+  return (size_t)(index >> 6) * 1024 + (size_t)(((index >> 3) & 1) * 512 + ((((index >> 4) & 3) * 16 + row) << 3) + (index & 7));
+}
+
 struct NoHooks {
   __device__ __forceinline__ void after_first() const {}
   __device__ __forceinline__ void before_barrier() const {}
@@ -69,8 +87,9 @@ struct NoHooks {
 // needs and whose addresses depend on loads issued before this function (they then fly with the second round of
 // weights).  hooks.before_barrier() runs behind the main loop, before the barrier: the place to leave further things
 // in LDS for the epilogue.
+// a_packed != 0: the activations come in the lanes' order (see packed_row_offset; only with CT = 1).
 template <int RT, int CT, int WAVES, bool GLU, bool PACKED, typename Hooks = NoHooks>
-__device__ __forceinline__ void skinny_partial_sums(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, int m, int n, int k,
+__device__ __forceinline__ void skinny_partial_sums(const bf16_t* __restrict__ a, int a_packed, const bf16_t* __restrict__ w, int m, int n, int k,
                                                     float4_t (&partial)[WAVES][RT * CT][64], Hooks hooks = Hooks()) {
   constexpr int UNROLL = 4;  // blocks of 64 indices whose loads are issued together
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -103,11 +122,13 @@ __device__ __forceinline__ void skinny_partial_sums(const bf16_t* __restrict__ a
   }
   const bf16_t* a_ptr[CT];
   bool a_ok[CT];
+  const int a_block = a_packed ? 1024 : 64;  // elements from one block of 64 indices to the next
+  const int a_half = a_packed ? 512 : 8;     // and from the first half of a lane's run to the second
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
     const int row = 16 * ct + i;
-    a_ok[ct] = row < m;
-    a_ptr[ct] = a + (size_t)(a_ok[ct] ? row : 0) * k + 16 * g;
+    a_ok[ct] = a_packed ? true : row < m;
+    a_ptr[ct] = a_packed ? a + lane * 8 : a + (size_t)(a_ok[ct] ? row : 0) * k + 16 * g;
   }
 
   float4_t acc[RT][CT];
@@ -127,7 +148,7 @@ __device__ __forceinline__ void skinny_partial_sums(const bf16_t* __restrict__ a
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) wr[u][rt] = (in_range && w_ok[rt]) ? (PACKED ? load_run_packed(w_ptr[rt] + w0) : load_run(w_ptr[rt] + w0)) : zero_run();
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct) ar[u][ct] = (in_range && a_ok[ct]) ? load_run(a_ptr[ct] + k0) : zero_run();
+      for (int ct = 0; ct < CT; ++ct) ar[u][ct] = (in_range && a_ok[ct]) ? load_run_halves(a_ptr[ct] + (size_t)(kb + u) * a_block, a_half) : zero_run();
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
@@ -234,7 +255,7 @@ struct Nothing {
 template <int RT, int CT, int WAVES, typename TO, bool GLU = false, bool PACKED = false, bool SCALED = false>
 __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
                                                                  const float* __restrict__ bias, TO* __restrict__ out, int m, int n, int k,
-                                                                 RowScale rs) {
+                                                                 RowScale rs, int a_packed, bf16_t* __restrict__ out_packed) {
   __shared__ float4_t partial[WAVES][RT * CT][64];
   __shared__ float scale_part[SCALED ? WAVES : 1][16];
   __shared__ float scale_stage[SCALED ? WAVES : 1][SCALED ? ROW_SCALE_ROUNDS : 1][SCALED ? 64 : 1];
@@ -242,9 +263,9 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
   const int n0 = blockIdx.x * 16 * RTO;
   if constexpr (SCALED) {
     RowScaleLoads<WAVES>::issue(rs, m, scale_stage);
-    skinny_partial_sums<RT, CT, WAVES, GLU, PACKED>(a, w, m, n, k, partial, ScaleHooks<WAVES, Nothing>{rs, scale_stage, scale_part, Nothing()});
+    skinny_partial_sums<RT, CT, WAVES, GLU, PACKED>(a, a_packed, w, m, n, k, partial, ScaleHooks<WAVES, Nothing>{rs, scale_stage, scale_part, Nothing()});
   } else {
-    skinny_partial_sums<RT, CT, WAVES, GLU, PACKED>(a, w, m, n, k, partial);
+    skinny_partial_sums<RT, CT, WAVES, GLU, PACKED>(a, a_packed, w, m, n, k, partial);
   }
   // add the waves' partial sums in wave order; each tile's 64 lanes are spread over the workgroup
   for (int item = threadIdx.x; item < RTO * CT * 64; item += WAVES * 64) {
@@ -269,58 +290,65 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
     const int col_m = 16 * ct + (l & 15);           // batch row
     const int row_n = n0 + 16 * rt + 4 * (l >> 4);  // first of four output columns
     if (col_m >= m) continue;
+    __attribute__((aligned(8))) bf16_t four[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
+      four[j] = from_f32<bf16_t>(0.f);
       if (row_n + j >= n) break;
       float v = sum[j];
       if (bias) v += bias[row_n + j];
       out[(size_t)col_m * n + row_n + j] = from_f32<TO>(v);
+      four[j] = from_f32<bf16_t>(v);
+    }
+    if constexpr (GLU && CT == 1) {  // the same values in the order the next product's lanes read them (n % 64 == 0 then)
+      typedef float float2_t __attribute__((ext_vector_type(2)));
+      if (out_packed) *reinterpret_cast<float2_t*>(out_packed + packed_row_offset(col_m, row_n)) = *reinterpret_cast<const float2_t*>(four);
     }
   }
 }
 
 template <int RT, int CT, int WAVES>
-static int launch_skinny_glu(const void* a, const void* w, void* out, int m, int n, int k, bool packed, RowScale rs, hipStream_t stream) {
+static int launch_skinny_glu(const void* a, const void* w, void* out, int m, int n, int k, bool packed, RowScale rs, int a_packed, void* out_packed, hipStream_t stream) {
   const int blocks = (n + 8 * RT - 1) / (8 * RT);
   if (packed && rs.partial != nullptr) {
     if constexpr (CT == 1)  // (rows are scaled only for M <= 16)
-      skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true, true, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k, rs);
+      skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true, true, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k, rs, a_packed, (bf16_t*)out_packed);
     else
       return -1;
   } else if (rs.partial != nullptr) {
     return -1;  // (only the packed weight's kernels scale rows)
   } else if (packed)
-    skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k, rs);
+    skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k, rs, a_packed, (bf16_t*)out_packed);
   else
-    skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k, rs);
+    skinny_gemm_kernel<RT, CT, WAVES, bf16_t, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, nullptr, (bf16_t*)out, m, n, k, rs, a_packed, (bf16_t*)out_packed);
   return (int)hipGetLastError();
 }
 
 template <int RT, int CT, int WAVES>
-static int launch_skinny(const void* a, const void* w, const float* bias, void* out, int m, int n, int k, int out_dtype, bool packed, RowScale rs, hipStream_t stream) {
+static int launch_skinny(const void* a, const void* w, const float* bias, void* out, int m, int n, int k, int out_dtype, bool packed, RowScale rs, int a_packed, hipStream_t stream) {
   const int blocks = (n + 16 * RT - 1) / (16 * RT);
   if (rs.partial != nullptr) {
     if constexpr (CT == 1) {  // (rows are scaled only for M <= 16, and only by the packed weight's kernels)
       if (!packed) return -1;
       if (out_dtype == VELOX_BF16)
-        skinny_gemm_kernel<RT, CT, WAVES, bf16_t, false, true, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (bf16_t*)out, m, n, k, rs);
+        skinny_gemm_kernel<RT, CT, WAVES, bf16_t, false, true, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (bf16_t*)out, m, n, k, rs, a_packed, nullptr);
       else
-        skinny_gemm_kernel<RT, CT, WAVES, float, false, true, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (float*)out, m, n, k, rs);
+        skinny_gemm_kernel<RT, CT, WAVES, float, false, true, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (float*)out, m, n, k, rs, a_packed, nullptr);
       return (int)hipGetLastError();
     }
     return -1;
   }
   if (packed) {
     if (out_dtype == VELOX_BF16)
-      skinny_gemm_kernel<RT, CT, WAVES, bf16_t, false, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (bf16_t*)out, m, n, k, rs);
+      skinny_gemm_kernel<RT, CT, WAVES, bf16_t, false, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (bf16_t*)out, m, n, k, rs, a_packed, nullptr);
     else
-      skinny_gemm_kernel<RT, CT, WAVES, float, false, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (float*)out, m, n, k, rs);
+      skinny_gemm_kernel<RT, CT, WAVES, float, false, true><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (float*)out, m, n, k, rs, a_packed, nullptr);
     return (int)hipGetLastError();
   }
   if (out_dtype == VELOX_BF16)
-    skinny_gemm_kernel<RT, CT, WAVES, bf16_t><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (bf16_t*)out, m, n, k, rs);
+    skinny_gemm_kernel<RT, CT, WAVES, bf16_t><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (bf16_t*)out, m, n, k, rs, a_packed, nullptr);
   else
-    skinny_gemm_kernel<RT, CT, WAVES, float><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (float*)out, m, n, k, rs);
+    skinny_gemm_kernel<RT, CT, WAVES, float><<<blocks, WAVES * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, bias, (float*)out, m, n, k, rs, a_packed, nullptr);
   return (int)hipGetLastError();
 }
 
@@ -329,14 +357,15 @@ static int launch_skinny(const void* a, const void* w, const float* bias, void* 
 // row_tiles: 16-row tiles of W per wave for M <= 16 (1 or 4).  With 4 a wave reuses each activation fragment for 64 rows
 // of W, which quarters the traffic of the activations; worth it when N is large enough that N / 64 workgroups still fill the GPU.
 // scale_partial (or null), scale_blocks, inv_width, eps: see RowScale; only with M <= 16.
+// a_packed != 0: a is in the lanes' order (see packed_row_offset); only with M <= 16.
 extern "C" int velox_skinny_gemm_bf16(const void* a, const void* w, const float* bias, void* out, int m, int n, int k, int out_dtype,
                                       int waves, int row_tiles, int packed, const float* scale_partial, int scale_blocks,
-                                      float inv_width, float eps, hipStream_t stream) {
+                                      float inv_width, float eps, int a_packed, hipStream_t stream) {
   if (m <= 0 || n <= 0) return 0;
-  if (k % 64 != 0 || m > 64 || (scale_partial != nullptr && (m > 16 || scale_blocks > ROW_SCALE_BLOCKS))) return -1;
+  if (k % 64 != 0 || m > 64 || (scale_partial != nullptr && (m > 16 || scale_blocks > ROW_SCALE_BLOCKS)) || (a_packed && m > 16)) return -1;
   if (scale_partial != nullptr && waves < 8) waves = 8;  // (rows are scaled by the eight-wave kernels)
   const RowScale rs{scale_partial, scale_blocks, inv_width, eps};
-#define PICK(RT, CT, W) return launch_skinny<RT, CT, W>(a, w, bias, out, m, n, k, out_dtype, packed != 0, rs, stream)
+#define PICK(RT, CT, W) return launch_skinny<RT, CT, W>(a, w, bias, out, m, n, k, out_dtype, packed != 0, rs, a_packed, stream)
   if (m <= 16 && row_tiles >= 4) {
     if (waves >= 8) PICK(4, 1, 8);
     PICK(4, 1, 4);
@@ -378,7 +407,7 @@ struct RotaryWrite {
 
 template <int WAVES>
 __global__ void __launch_bounds__(WAVES * 64) skinny_qkv_rotary_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
-                                                                       RotaryWrite args, int m, int n, int k, RowScale rs) {
+                                                                       RotaryWrite args, int m, int n, int k, RowScale rs, int a_packed) {
   __shared__ float4_t partial[WAVES][2][64];
   __shared__ float scale_part[WAVES][16];
   __shared__ float scale_stage[WAVES][ROW_SCALE_ROUNDS][64];
@@ -407,7 +436,7 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_qkv_rotary_kernel(const bf1
     sn = *reinterpret_cast<const float4_t*>(args.sin_table + angle);
   };
   RowScaleLoads<WAVES>::issue(rs, m, scale_stage);
-  skinny_partial_sums<2, 1, WAVES, false, true>(a, w, m, n, k, partial, ScaleHooks<WAVES, decltype(fetch_angles)>{rs, scale_stage, scale_part, fetch_angles});
+  skinny_partial_sums<2, 1, WAVES, false, true>(a, a_packed, w, m, n, k, partial, ScaleHooks<WAVES, decltype(fetch_angles)>{rs, scale_stage, scale_part, fetch_angles});
   if (l >= 64) return;
   const float row_scale = row_scale_of<WAVES>(rs, scale_part, row_in);
   if (row >= m) return;
@@ -453,7 +482,7 @@ extern "C" int velox_skinny_qkv_rotary_bf16(const void* a, const void* w, const 
                                             const float* cos_table, const float* sin_table, const int* slots, void* q_out,
                                             void* k_cache, void* v_cache, int m, int k, int heads, int kv_heads, int d,
                                             int page_size, int waves, const float* scale_partial, int scale_blocks, float inv_width,
-                                            float eps, hipStream_t stream) {
+                                            float eps, int a_packed, hipStream_t stream) {
   if (m <= 0) return 0;
   if (m > 16 || k % 64 != 0 || d % 32 != 0 || heads < 1 || kv_heads < 1 || page_size < 1) return -1;
   if (scale_partial != nullptr && scale_blocks > ROW_SCALE_BLOCKS) return -1;
@@ -463,7 +492,7 @@ extern "C" int velox_skinny_qkv_rotary_bf16(const void* a, const void* w, const 
   const int n = (heads + 2 * kv_heads) * d;
   const int blocks = n / 32;
   (void)waves;  // (16 waves leave 128 registers per lane, which this kernel does not fit without spilling, and measured no faster)
-  skinny_qkv_rotary_kernel<8><<<blocks, 8 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, args, m, n, k, rs);
+  skinny_qkv_rotary_kernel<8><<<blocks, 8 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, args, m, n, k, rs, a_packed);
   return (int)hipGetLastError();
 }
 
@@ -476,7 +505,8 @@ extern "C" int velox_skinny_qkv_rotary_bf16(const void* a, const void* w, const 
 template <int WAVES>
 __global__ void __launch_bounds__(WAVES * 64) skinny_residual_norm_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
                                                                           float* __restrict__ residual, const float* __restrict__ norm_weight,
-                                                                          bf16_t* __restrict__ next, float* __restrict__ sums, int m, int n, int k) {
+                                                                          bf16_t* __restrict__ next, float* __restrict__ sums, int m, int n, int k,
+                                                                          int a_packed, bf16_t* __restrict__ next_packed) {
   __shared__ float4_t partial[WAVES][1][64];
   // what the epilogue reads is fetched before the main loop (by the 64 threads that will need it)
   const int l = threadIdx.x;
@@ -489,22 +519,28 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_residual_norm_kernel(const 
     old_residual[j] = inside ? residual[(size_t)row * n + col + j] : 0.f;
     weight[j] = inside ? norm_weight[col + j] : 0.f;
   }
-  skinny_partial_sums<1, 1, WAVES, false, true>(a, w, m, n, k, partial);
+  skinny_partial_sums<1, 1, WAVES, false, true>(a, a_packed, w, m, n, k, partial);
   if (l >= 64) return;
   float4_t sum = partial[0][0][l];
 #pragma unroll
   for (int wv = 1; wv < WAVES; ++wv) sum += partial[wv][0][l];
   float squares = 0.f;
   if (row < m) {
+    __attribute__((aligned(8))) bf16_t four[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
+      four[j] = from_f32<bf16_t>(0.f);
       if (col + j >= n) break;
       const size_t at = (size_t)row * n + col + j;
       const float r = old_residual[j] + sum[j];
       residual[at] = r;
-      next[at] = from_f32<bf16_t>(r * weight[j]);
+      four[j] = from_f32<bf16_t>(r * weight[j]);
+      next[at] = four[j];
       squares += r * r;
     }
+    // the same values in the order the next product's lanes read them (n % 64 == 0 then)
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    if (next_packed) *reinterpret_cast<float2_t*>(next_packed + packed_row_offset(row, col)) = *reinterpret_cast<const float2_t*>(four);
   }
   // the four lane groups hold four columns each of the same rows: added in a fixed order
   squares += __shfl_xor(squares, 16, VELOX_WAVE);
@@ -512,39 +548,45 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_residual_norm_kernel(const 
   if (l < 16) sums[(size_t)l * gridDim.x + blockIdx.x] = squares;
 }
 
-// a [M, K] bfloat16 (M <= 16), w packed [N, K]; sums: float32 [16][ceil(N / 16)].  waves: 4, 8 or 16.
+// a [M, K] bfloat16 (M <= 16; a_packed != 0: in the lanes' order, see packed_row_offset), w packed [N, K]; sums: float32
+// [16][ceil(N / 16)].  next_packed (or null; needs N % 64 == 0): room for N / 64 * 1024 elements, `next` once more in the
+// lanes' order.  waves: 4, 8 or 16.
 extern "C" int velox_skinny_residual_norm_bf16(const void* a, const void* w, float* residual, const float* norm_weight, void* next,
-                                               float* sums, int m, int n, int k, int waves, hipStream_t stream) {
+                                               float* sums, int m, int n, int k, int waves, int a_packed, void* next_packed, hipStream_t stream) {
   if (m <= 0 || n <= 0) return 0;
-  if (m > 16 || k % 64 != 0) return -1;
+  if (m > 16 || k % 64 != 0 || (next_packed != nullptr && n % 64 != 0)) return -1;
   const int blocks = (n + 15) / 16;
   if (waves >= 16)
-    skinny_residual_norm_kernel<16><<<blocks, 16 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, residual, norm_weight, (bf16_t*)next, sums, m, n, k);
+    skinny_residual_norm_kernel<16><<<blocks, 16 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, residual, norm_weight, (bf16_t*)next, sums, m, n, k, a_packed, (bf16_t*)next_packed);
   else if (waves >= 8)
-    skinny_residual_norm_kernel<8><<<blocks, 8 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, residual, norm_weight, (bf16_t*)next, sums, m, n, k);
+    skinny_residual_norm_kernel<8><<<blocks, 8 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, residual, norm_weight, (bf16_t*)next, sums, m, n, k, a_packed, (bf16_t*)next_packed);
   else
-    skinny_residual_norm_kernel<4><<<blocks, 4 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, residual, norm_weight, (bf16_t*)next, sums, m, n, k);
+    skinny_residual_norm_kernel<4><<<blocks, 4 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, residual, norm_weight, (bf16_t*)next, sums, m, n, k, a_packed, (bf16_t*)next_packed);
   return (int)hipGetLastError();
 }
 
 // out[M, n] = silu(A Wgate^T) * (A Wup^T) with W = [Wgate; Wup] of 2n rows, bfloat16 in and out, M <= 32.
 // pairs: gate/up tile pairs per wave (1 or 2).
+// a_packed != 0: a is in the lanes' order (see packed_row_offset); out_packed (or null; needs n % 64 == 0): room for
+// n / 64 * 1024 elements, the result once more in that order.  Both only with M <= 16.
 extern "C" int velox_skinny_gemm_glu_bf16(const void* a, const void* w, void* out, int m, int n, int k, int waves, int pairs, int packed,
-                                          const float* scale_partial, int scale_blocks, float inv_width, float eps, hipStream_t stream) {
+                                          const float* scale_partial, int scale_blocks, float inv_width, float eps, int a_packed,
+                                          void* out_packed, hipStream_t stream) {
   if (m <= 0 || n <= 0) return 0;
   if (k % 64 != 0 || m > 32 || (scale_partial != nullptr && (m > 16 || scale_blocks > ROW_SCALE_BLOCKS))) return -1;
+  if ((a_packed || out_packed != nullptr) && (m > 16 || (out_packed != nullptr && n % 64 != 0))) return -1;
   const RowScale rs{scale_partial, scale_blocks, inv_width, eps};
   if (scale_partial != nullptr && waves < 8) waves = 8;  // (rows are scaled by the eight-wave kernels)
   if (m <= 16) {
     if (pairs >= 2) {
-      if (waves >= 8) return launch_skinny_glu<4, 1, 8>(a, w, out, m, n, k, packed != 0, rs, stream);
-      return launch_skinny_glu<4, 1, 4>(a, w, out, m, n, k, packed != 0, rs, stream);
+      if (waves >= 8) return launch_skinny_glu<4, 1, 8>(a, w, out, m, n, k, packed != 0, rs, a_packed, out_packed, stream);
+      return launch_skinny_glu<4, 1, 4>(a, w, out, m, n, k, packed != 0, rs, a_packed, out_packed, stream);
     }
-    if (waves >= 8) return launch_skinny_glu<2, 1, 8>(a, w, out, m, n, k, packed != 0, rs, stream);
-    return launch_skinny_glu<2, 1, 4>(a, w, out, m, n, k, packed != 0, rs, stream);
+    if (waves >= 8) return launch_skinny_glu<2, 1, 8>(a, w, out, m, n, k, packed != 0, rs, a_packed, out_packed, stream);
+    return launch_skinny_glu<2, 1, 4>(a, w, out, m, n, k, packed != 0, rs, a_packed, out_packed, stream);
   }
-  if (waves >= 8) return launch_skinny_glu<2, 2, 8>(a, w, out, m, n, k, packed != 0, rs, stream);
-  return launch_skinny_glu<2, 2, 4>(a, w, out, m, n, k, packed != 0, rs, stream);
+  if (waves >= 8) return launch_skinny_glu<2, 2, 8>(a, w, out, m, n, k, packed != 0, rs, a_packed, out_packed, stream);
+  return launch_skinny_glu<2, 2, 4>(a, w, out, m, n, k, packed != 0, rs, a_packed, out_packed, stream);
 }
 
 // ---------------------------------------------------------------------------------------------------------------

@@ -69,17 +69,18 @@ class HipOps:
         c = self._core
         c.velox_embed.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
         c.velox_add_rmsnorm.argtypes = [_P, _P, _P, _P, _P, _I, _I, _F, _I, _I, _I, ctypes.c_longlong, _P]
-        c.velox_skinny_qkv_rotary_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _P]
+        c.velox_skinny_qkv_rotary_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _I, _P]
         c.velox_silu_mul.argtypes = [_P, _P, _I, _I, _I, _P]
         c.velox_rope_kv_write.argtypes = [_P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_rope_kv_write_partial_bf16.argtypes = [_P, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
         c.velox_rope_kv_write_partial_bf16.restype = _I
         c.velox_gemm_fma.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
-        c.velox_skinny_gemm_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _P]
-        c.velox_skinny_residual_norm_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]
+        c.velox_skinny_gemm_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _I, _P]
+        c.velox_skinny_residual_norm_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P]
+        c.velox_skinny_residual_norm_bf16.restype = _I
         c.velox_row_scale_apply.argtypes = [_P, _P, _I, _F, _F, _P, _I, _I, _P]
         c.velox_skinny_gemm_bf16.restype = _I
-        c.velox_skinny_gemm_glu_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _P]
+        c.velox_skinny_gemm_glu_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _I, _P, _P]
         c.velox_skinny_gemm_glu_bf16.restype = _I
         c.velox_skinny_gemm_splitk_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P]
         c.velox_skinny_gemm_splitk_bf16.restype = _I
@@ -262,6 +263,23 @@ class HipOps:
             return _P(0), 0, 0.0, 0.0
         return _ptr(deferred.sums), int(deferred.sums.shape[1]), 1.0 / deferred.width, float(deferred.eps)
 
+    def _packed_rows_of(self, x: torch.Tensor, k: int) -> Optional[torch.Tensor]:
+        """The copy of decode-sized activations ``x`` [M <= 16, k] in the order the skinny kernels' lanes read them, if the
+        kernel that wrote ``x`` left one (it hangs on the tensor object), else None."""
+        twin, version = getattr(x, "_velox_packed_rows", (None, None))
+        if (twin is None or version != x._version or x.dim() != 2 or x.shape[0] > 16 or x.shape[1] != k or k % 64 != 0
+                or twin.numel() != k // 64 * 1024 or twin.dtype != torch.bfloat16):
+            return None
+        return twin
+
+    def _room_for_packed_rows(self, m: int, n: int) -> Optional[torch.Tensor]:
+        """Room for ``[m, n]`` activations in the lanes' order, if the kernels can write and read them like that and it
+        pays: the copy always has 16 rows, and what a product's activations cost is their bytes, not the pieces they come in
+        (measured on MI355X, 3584 x 18944: 12 rows row-major 28.5 us, 16 rows 30.9 us, the copy 28.4 us at any number)."""
+        if not 13 <= m <= 16 or n % 64 != 0 or not self.pack_decode_weights:
+            return None
+        return torch.empty(n // 64 * 1024, dtype=torch.bfloat16, device=self.device)
+
     def materialize(self, x):
         """A ``DeferredNorm`` as the plain normalised tensor (one small kernel); anything else is returned as it is."""
         if not isinstance(x, DeferredNorm):
@@ -294,7 +312,7 @@ class HipOps:
         if bias is not None:
             self._check("bias", bias, torch.float32, (n,))
         if deferred is not None:
-            return self.skinny_gemm(x, weight, bias, out_dtype, packed=self.packed_weight(weight), row_scale=deferred)
+            return self.skinny_gemm(x, weight, bias, out_dtype, packed=self.packed_weight(weight), row_scale=deferred, x_packed=self._packed_rows_of(x, k))
         if residual_norm is not None and bias is None:
             fused = self._linear_into_residual(x, weight, residual_norm)
             if fused is not None:
@@ -304,7 +322,7 @@ class HipOps:
             return self.skinny_gemm_splitk(x, weight, packed=self.packed_weight(weight))
         skinny_rows = 16 if n > 8192 else 32  # measured on MI355X: beyond this the library's kernels stream faster
         if self.use_skinny_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and m <= skinny_rows and k % 64 == 0:
-            return self.skinny_gemm(x, weight, bias, out_dtype, packed=self.packed_weight(weight))
+            return self.skinny_gemm(x, weight, bias, out_dtype, packed=self.packed_weight(weight), x_packed=self._packed_rows_of(x, k))
         if self.use_library_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and bias is None:
             if out_dtype == torch.bfloat16:
                 return torch.nn.functional.linear(x, weight)
@@ -334,9 +352,14 @@ class HipOps:
         blocks = (n + 15) // 16
         out = torch.empty((m, n), dtype=torch.bfloat16, device=self.device)
         sums = torch.empty((16, blocks), dtype=torch.float32, device=self.device)
-        status = self._core.velox_skinny_residual_norm_bf16(_ptr(x), _ptr(packed), _ptr(residual), _ptr(norm_weight), _ptr(out), _ptr(sums),
-                                                            m, n, k, int(waves or 8), self._stream())
+        x_packed = self._packed_rows_of(x, k)
+        out_packed = self._room_for_packed_rows(m, n)
+        status = self._core.velox_skinny_residual_norm_bf16(_ptr(x if x_packed is None else x_packed), _ptr(packed), _ptr(residual), _ptr(norm_weight),
+                                                            _ptr(out), _ptr(sums), m, n, k, int(waves or 8), int(x_packed is not None), _ptr(out_packed),
+                                                            self._stream())
         self._launched(status, "skinny_residual_norm")
+        if out_packed is not None:
+            out._velox_packed_rows = (out_packed, out._version)
         return DeferredNorm(out, sums, n, float(eps), sink.norm)
 
     @staticmethod
@@ -354,7 +377,7 @@ class HipOps:
         return padded.view(matrices, tiles, 16, k // 64, 4, 2, 8).permute(0, 1, 3, 5, 4, 2, 6).contiguous().view(-1)
 
     def skinny_gemm(self, x, weight, bias, out_dtype, waves: Optional[int] = None, row_tiles: Optional[int] = None, packed: Optional[torch.Tensor] = None, n: Optional[int] = None,
-                    row_scale: Optional[DeferredNorm] = None):
+                    row_scale: Optional[DeferredNorm] = None, x_packed: Optional[torch.Tensor] = None):
         """Few rows (M <= 64) times a bfloat16 weight: the weight-streaming kernel of the decode step.  ``packed`` is
         ``pack_rows(weight)``, used instead of ``weight`` when given (``n`` = rows of the weight).  ``row_scale``: ``x`` is
         its ``.x`` and the result rows are scaled as it says (M <= 16)."""
@@ -381,8 +404,11 @@ class HipOps:
         out = torch.empty((m, n), dtype=out_dtype, device=self.device)
         if row_scale is not None and m > 16:
             raise KernelError("skinny_gemm: rows are scaled only for M <= 16")
-        status = self._core.velox_skinny_gemm_bf16(_ptr(x), _ptr(weight_arg), _ptr(bias), _ptr(out), m, n, k, _code(out_dtype), int(waves), int(row_tiles),
-                                                   1 if packed is not None else 0, *self._scale_args(row_scale), self._stream())
+        if x_packed is not None and (m > 16 or x_packed.dtype != torch.bfloat16 or x_packed.numel() != k // 64 * 1024):
+            raise KernelError("skinny_gemm: the packed activations do not match M and K")
+        status = self._core.velox_skinny_gemm_bf16(_ptr(x if x_packed is None else x_packed), _ptr(weight_arg), _ptr(bias), _ptr(out), m, n, k, _code(out_dtype),
+                                                   int(waves), int(row_tiles), 1 if packed is not None else 0, *self._scale_args(row_scale),
+                                                   int(x_packed is not None), self._stream())
         self._launched(status, "skinny_gemm")
         return out
 
@@ -410,9 +436,14 @@ class HipOps:
         if waves is None:
             waves = 8
         out = torch.empty((m, n), dtype=out_dtype, device=self.device)
-        status = self._core.velox_skinny_gemm_glu_bf16(_ptr(x), _ptr(packed if packed is not None else gate_up_weight), _ptr(out), m, n, k, int(waves), int(pairs),
-                                                       1 if packed is not None else 0, *self._scale_args(deferred), self._stream())
+        x_packed = self._packed_rows_of(x, k)
+        out_packed = self._room_for_packed_rows(m, n)
+        status = self._core.velox_skinny_gemm_glu_bf16(_ptr(x if x_packed is None else x_packed), _ptr(packed if packed is not None else gate_up_weight), _ptr(out),
+                                                       m, n, k, int(waves), int(pairs), 1 if packed is not None else 0, *self._scale_args(deferred),
+                                                       int(x_packed is not None), _ptr(out_packed), self._stream())
         self._launched(status, "skinny_gemm_glu")
+        if out_packed is not None:
+            out._velox_packed_rows = (out_packed, out._version)
         return out
 
     def skinny_gemm_splitk(self, x, weight, splits: Optional[int] = None, packed: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -558,9 +589,11 @@ class HipOps:
         self._check("k_cache", k_cache, torch.bfloat16, (pages, num_kv_heads, block_size, head_dim), align=16)
         self._check("v_cache", v_cache, torch.bfloat16, (pages, num_kv_heads, head_dim, block_size), align=16)
         q = torch.empty((m, num_heads * head_dim), dtype=torch.bfloat16, device=self.device)
+        x_packed = self._packed_rows_of(x, k)
         status = self._core.velox_skinny_qkv_rotary_bf16(
-            _ptr(x), _ptr(packed), _ptr(bias), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping), _ptr(q), _ptr(k_cache),
-            _ptr(v_cache), m, k, num_heads, num_kv_heads, head_dim, block_size, int(waves or 8), *self._scale_args(deferred), self._stream())
+            _ptr(x if x_packed is None else x_packed), _ptr(packed), _ptr(bias), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping), _ptr(q), _ptr(k_cache),
+            _ptr(v_cache), m, k, num_heads, num_kv_heads, head_dim, block_size, int(waves or 8), *self._scale_args(deferred),
+            int(x_packed is not None), self._stream())
         self._launched(status, "skinny_qkv_rotary")
         return q
 
