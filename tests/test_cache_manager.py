@@ -33,6 +33,31 @@ def test_allocator_order_and_errors():
     a.assert_consistent()
 
 
+@pytest.mark.parametrize("num_pages", [2, 3, 4, 5, 17, 64, 1000, 7201])
+def test_scattered_first_hand_outs(num_pages):
+    """``scatter=True``: every page is still handed out exactly once, never page 0, freed pages come back most recent
+    first, and pages handed out one after the other (or 256 hand-outs apart, as the same place of two sequences) lie
+    far from each other and at no common power-of-two distance."""
+    a = PageAllocator(num_pages, scatter=True)
+    order = a.allocate_many(num_pages - 1)
+    assert sorted(order) == list(range(1, num_pages))
+    with pytest.raises(OutOfPagesError):
+        a.allocate()
+    if num_pages > 2:
+        a.free(order[0])
+        a.free(order[-1])
+        assert a.allocate() == order[-1] and a.allocate() == order[0]
+    a.assert_consistent()
+    if num_pages >= 64:
+        count = num_pages - 1
+        gaps = [min((x - y) % count, (y - x) % count) for x, y in zip(order, order[1:])]
+        assert min(gaps) > count // 4
+        if num_pages >= 1000:
+            far = [(order[i + 256] - order[i]) % count for i in range(0, len(order) - 256, 37)]
+            assert len(set(far)) == 1 and far[0] % 16 != 0  # one stride for all, and not a multiple of a power of two
+    assert PageAllocator(num_pages).allocate_many(num_pages - 1) == list(range(1, num_pages))
+
+
 def _manager(needs, pages=9, page=4, seqs=4, max_len=None):
     return CacheManager(needs, page, pages, seqs, torch.float32, "cpu", max_model_len=max_len)
 

@@ -56,11 +56,12 @@ class SequenceCache:
 
 
 class PageGroup:
-    def __init__(self, need: PagedNeed, entries: List[int], num_pages: int, page_size: int, dtype: torch.dtype, device, allocate_tensors: bool) -> None:
+    def __init__(self, need: PagedNeed, entries: List[int], num_pages: int, page_size: int, dtype: torch.dtype, device, allocate_tensors: bool,
+                 scatter_pages: bool = False) -> None:
         self.need = need
         self.entries = list(entries)
         self.page_size = int(page_size)
-        self.allocator = PageAllocator(num_pages)
+        self.allocator = PageAllocator(num_pages, scatter=scatter_pages)
         self.dtype = dtype
         self.keys: Optional[torch.Tensor] = None
         self.values: Optional[torch.Tensor] = None
@@ -155,6 +156,7 @@ class CacheManager:
         max_model_len: Optional[int] = None,
         allocate_tensors: bool = True,
         prefix_caching: bool = False,
+        scatter_pages: bool = False,
     ) -> None:
         if page_size <= 0 or (page_size & (page_size - 1)) != 0:
             raise ValueError(f"page_size must be a power of two, got {page_size}")
@@ -174,7 +176,7 @@ class CacheManager:
                 raise TypeError(f"schedule entry {entry}: unknown cache need {need!r}")
         for need, entries in by_need.items():
             index = len(self.groups)
-            self.groups.append(PageGroup(need, entries, num_pages, page_size, dtype, self.device, allocate_tensors))
+            self.groups.append(PageGroup(need, entries, num_pages, page_size, dtype, self.device, allocate_tensors, scatter_pages))
             for position, entry in enumerate(entries):
                 self.entry_group[entry] = (index, position)
         self.state = StateSlots(state_needs, max_num_seqs, dtype, self.device, allocate_tensors)

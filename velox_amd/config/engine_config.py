@@ -64,6 +64,9 @@ class EngineConfig:
     # a second copy of every bfloat16 weight in the order the decode kernels read it: faster decoding for the
     # weights' size again in memory (not a reference option)
     pack_decode_weights: bool = True
+    # fresh pages are handed out all over the pool instead of 1, 2, 3, ...: sequences decoded together then do not read
+    # the same memory channels at the same moment (not a reference option)
+    scatter_pages: bool = True
     # launch a decode step's successor before reading the step's tokens (not a reference option)
     decode_lookahead: bool = True
     watermark: float = 0.01

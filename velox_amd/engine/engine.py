@@ -138,7 +138,7 @@ class Engine:
             wanted = (config.max_num_seqs * max_model_len + config.block_size - 1) // config.block_size + 1
             num_pages = min(num_pages, max(2, wanted))
         cache = CacheManager(needs, config.block_size, num_pages, config.max_num_seqs, dtype, device, max_model_len=max_model_len,
-                             prefix_caching=config.enable_prefix_caching)
+                             prefix_caching=config.enable_prefix_caching, scatter_pages=config.scatter_pages)
         engine = cls(model, cache, config, ops, eos_token_ids=eos)
         engine.warmup()
         return engine
