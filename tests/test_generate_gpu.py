@@ -72,6 +72,30 @@ def test_graph_decode_equals_eager_decode_and_preemption_keeps_tokens(tmp_path):
     assert tight_engine.cache.num_used_pages() == 0
 
 
+def test_captured_steps_behind_few_keys_and_behind_many(tmp_path):
+    """With a long context allowed, a bucket has two captures: one whose attention splits the keys as the longest context
+    needs, one for steps whose sequences all hold few keys (one workgroup per sequence and KV head).  A request that grows
+    past the bound moves from the one to the other; tokens as without graphs (float32: bit for bit)."""
+    from velox_amd.engine.runner import SHORT_CONTEXT_KEYS
+
+    folder = make_folder(tmp_path, "B", "float32")
+    config, _ = read_model_folder(folder)
+    assert config["max_position_embeddings"] >= 1024
+    prompts = [random_tokens(config["vocab_size"], n, seed=70 + n) for n in (SHORT_CONTEXT_KEYS - 14, 40)]
+    options = dict(max_model_len=1024, max_num_batched_tokens=512, max_prefill_chunk_size=256, num_gpu_blocks=400)
+    eager = engine_for(folder, "B", "float32", **options).generate(greedy(prompts, 30))
+    engine = engine_for(folder, "B", "float32", enable_cuda_graphs=True, **options)
+    assert sorted(engine.runner._short_graphs) == [1, 2, 4]
+    graphed = engine.generate(greedy(prompts, 30))
+    assert [r.output_token_ids for r in graphed] == [r.output_token_ids for r in eager]
+    assert 10 <= engine.runner.num_short_graph_replays <= 20 and engine.runner.num_graph_replays >= 29
+    # the short request alone stays behind few keys to its end
+    before = engine.runner.num_short_graph_replays
+    alone = engine.generate(greedy(prompts[1:], 30, prefix="alone"))
+    assert alone[0].output_token_ids == eager[1].output_token_ids
+    assert engine.runner.num_short_graph_replays - before >= 29
+
+
 @pytest.mark.parametrize("graphs", [False, True])
 def test_launching_the_next_step_early_changes_no_token(tmp_path, graphs):
     """decode_lookahead on the GPU, eager and through graphs: the next decode step is queued, with its token ids taken

@@ -35,6 +35,13 @@ def decode_buckets(max_num_seqs: int) -> List[int]:
     return buckets
 
 
+# A captured decode step fixes how many workgroups share a sequence's keys (the split count is part of the launch).
+# Chosen for the longest context the engine allows, that count is too many behind few keys, where one workgroup per
+# sequence and KV head is quicker than splits and their merge; so steps whose sequences all hold at most this many
+# keys have a capture of their own.
+SHORT_CONTEXT_KEYS = 384
+
+
 class ModelRunner:
     def __init__(
         self,
@@ -58,9 +65,11 @@ class ModelRunner:
         self.workspace = Workspace(self.device)
         self.enable_graphs = bool(enable_graphs) and self.device.type == "cuda"
         self._graphs: Dict[int, Tuple[object, torch.Tensor, torch.Tensor]] = {}
+        self._short_graphs: Dict[int, Tuple[object, torch.Tensor, torch.Tensor]] = {}  # the same buckets behind few keys
         self._graph_buffers: Dict[int, torch.Tensor] = {}
         self._graph_pool = None
         self.num_graph_replays = 0
+        self.num_short_graph_replays = 0  # those of them through the captures for short contexts
 
     # -- the step -----------------------------------------------------------------------
     @torch.no_grad()
@@ -105,24 +114,41 @@ class ModelRunner:
             return
         buckets = list(buckets) if buckets is not None else decode_buckets(self.max_num_seqs)
         self._graph_pool = torch.cuda.graph_pool_handle()
+        self._short_graphs.clear()
         for bucket in buckets:
             capacity = self.builder.section_total(bucket, bucket, bucket, self.builder.width)
             self._graph_buffers[bucket] = torch.zeros(capacity, dtype=torch.int32, device=self.device)
-            ctx = self._graph_context(bucket)
-            stream = torch.cuda.Stream(device=self.device)
-            stream.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(stream):
-                for _ in range(warmup_iters):
-                    self._forward(ctx)
-            torch.cuda.current_stream().wait_stream(stream)
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
-                logits = self._forward(ctx)
-            self._graphs[bucket] = (graph, logits, ctx)
+            self._graphs[bucket] = self._capture(self._graph_context(bucket, self.cache.max_model_len), warmup_iters)
+            if self.cache.max_model_len > SHORT_CONTEXT_KEYS and self._splits_differ(bucket):
+                self._short_graphs[bucket] = self._capture(self._graph_context(bucket, SHORT_CONTEXT_KEYS), warmup_iters)
         torch.cuda.synchronize()
 
-    def _graph_context(self, bucket: int) -> StepContext:
+    def _capture(self, ctx: StepContext, warmup_iters: int):
+        stream = torch.cuda.Stream(device=self.device)
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            for _ in range(warmup_iters):
+                self._forward(ctx)
+        torch.cuda.current_stream().wait_stream(stream)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, pool=self._graph_pool):
+            logits = self._forward(ctx)
+        return graph, logits, ctx
+
+    def _splits_differ(self, bucket: int) -> bool:
+        """Whether any paged group's attention would split the keys of a ``bucket``-row step behind the longest context
+        but not behind a short one (only then is a second capture worth its memory)."""
+        choose = getattr(self.ops, "choose_splits", None)
+        if choose is None:
+            return False
+        for group in self.cache.groups:
+            heads = group.need.num_kv_heads
+            if choose(bucket, heads, 1, self.cache.max_model_len, True) != choose(bucket, heads, 1, SHORT_CONTEXT_KEYS, True):
+                return True
+        return False
+
+    def _graph_context(self, bucket: int, max_kv_len: int) -> StepContext:
         """A context of ``bucket`` padded rows only (all on the null page), laid out in the bucket's buffer."""
         from ..cache.manager import SequenceCache
 
@@ -133,14 +159,17 @@ class ModelRunner:
             device_buffer=self._graph_buffers[bucket], pad_to=bucket, width=self.builder.width,
         )
         ctx.all_decode = True
-        # lengths are read from device memory at replay; the capture must not specialise on them
+        # lengths are read from device memory at replay; the capture must not specialise on them beyond their bound
         for group in ctx.groups:
-            group.max_kv_len = self.cache.max_model_len
+            group.max_kv_len = max_kv_len
         ctx.rows = ctx.rows[:bucket]
         return ctx
 
     def _replay(self, bucket: int, entries: Sequence[StepEntry], ids_on_device: Optional[tuple] = None) -> torch.Tensor:
         graph, logits, _ = self._graphs[bucket]
+        if bucket in self._short_graphs and all(e.start < SHORT_CONTEXT_KEYS for e in entries):
+            graph, logits, _ = self._short_graphs[bucket]
+            self.num_short_graph_replays += 1
         self._padded_entries_context(bucket, entries, ids_on_device)  # refreshes the bucket's buffer in place
         graph.replay()
         self.num_graph_replays += 1
