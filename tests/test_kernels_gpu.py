@@ -688,6 +688,26 @@ def test_skinny_gemm_with_silu_epilogue(ops, ref, m, inter, k):
     torch.testing.assert_close(ops.linear_silu_mul(big, w, torch.bfloat16).float(), ref.linear_silu_mul(big, w, torch.bfloat16).float(), rtol=3e-2, atol=3e-2 * scale)
 
 
+@pytest.mark.parametrize("m,inter,k", [(17, 18944, 3584), (64, 18944, 3584), (32, 150, 128), (33, 1000, 192), (40, 16, 64), (64, 81, 1600), (24, 400, 320)])
+def test_gate_up_product_with_silu_epilogue_at_17_to_64_rows(ops, ref, m, inter, k):
+    """A registered [Wgate; Wup] at 17 .. 64 rows: one kernel (ten waves per workgroup, five pairs of gate and up tiles)
+    against the product in float32 followed by silu(gate) * up; widths that are no multiple of 16 or of 80, a K that
+    is no multiple of a chunk of 256."""
+    x = rand((m, k), torch.bfloat16, 53)
+    w = rand((2 * inter, k), torch.bfloat16, 54, 0.05)
+    gate_up = ref.linear(x, w, None, torch.float32)
+    want = (torch.nn.functional.silu(gate_up[:, :inter]) * gate_up[:, inter:])
+    scale = float(want.abs().max())
+    unregistered = ops.linear_silu_mul(x, w, torch.bfloat16).float()  # (product + SiLU kernel)
+    ops.register_weight(w, stacked=2)
+    got = ops.linear_silu_mul(x, w, torch.bfloat16).float()
+    torch.testing.assert_close(got, want, rtol=1e-2, atol=1e-2 * scale)
+    torch.testing.assert_close(got, unregistered, rtol=2e-2, atol=2e-2 * scale)
+    # rows of a batch do not depend on one another: the first rows alone give the same bits
+    few = ops.linear_silu_mul(x[:17].contiguous(), w, torch.bfloat16).float()
+    assert torch.equal(few, got[:17])
+
+
 @pytest.mark.parametrize("m,n,k", [(17, 3584, 18944), (64, 3584, 3584), (33, 100, 640), (64, 4608, 3584), (40, 260, 128), (64, 72, 1600)])
 def test_skinny_gemm_splitk_and_norm_that_adds_the_partials(ops, ref, m, n, k):
     x = rand((m, k), torch.bfloat16, 60)

@@ -729,3 +729,166 @@ extern "C" int velox_skinny_gemm_splitk_bf16(const void* a, const void* w, float
     skinny_gemm_splitk_kernel<4, false><<<grid, 256, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, partial, m, n, k, per_split);
   return (int)hipGetLastError();
 }
+
+// ---------------------------------------------------------------------------------------------------------------
+// silu(A Wgate^T) * (A Wup^T) for 17 .. 64 rows: the gate/up product of a decode step at those sizes with its
+// activation as the epilogue, so that the [M, 2n] product is never written.  W = [Wgate; Wup] packed, each matrix
+// padded to whole 16-row tiles.  A workgroup of ten waves owns five gate tiles (waves 0 .. 4) and the five up tiles of
+// the same output columns (waves 5 .. 9) and all of K; the up waves hand their sums to the gate waves through LDS at
+// the end.  37888 rows of W are 1184 pairs, 237 workgroups: one round on 256 compute units.  As in the split-K kernel
+// W streams through a ring of three register sets, two chunks (of 4 blocks of 64 indices) ahead of the arithmetic,
+// and the activations of a chunk are asked for one chunk ahead, staged in LDS once per workgroup and read by all waves.
+// ---------------------------------------------------------------------------------------------------------------
+// GLU_ROWS_PAIRS: pairs of (gate, up) tiles per workgroup, chosen by the caller so that the launch is one round of
+// workgroups (up to 6: twelve waves leave a lane the registers the ring needs).
+template <int CT, int GLU_ROWS_PAIRS>
+__global__ void __launch_bounds__(128 * GLU_ROWS_PAIRS) skinny_glu_rows_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
+                                                                              bf16_t* __restrict__ out, int m, int n, int k) {
+  constexpr int CHUNK = 4;
+  constexpr int THREADS = 128 * GLU_ROWS_PAIRS;
+  constexpr int ROWS = 16 * CT;
+  constexpr int AS = 64 + 8;
+  constexpr int A_VECS = ROWS * CHUNK * 8;
+  constexpr int A_ITERS = (A_VECS + THREADS - 1) / THREADS;
+  constexpr int TILE_BYTES = CHUNK * ROWS * AS * 2, HAND_BYTES = GLU_ROWS_PAIRS * CT * 64 * 16;
+  __shared__ __attribute__((aligned(16))) char smem[TILE_BYTES > HAND_BYTES ? TILE_BYTES : HAND_BYTES];
+  bf16_t* const a_tile = reinterpret_cast<bf16_t*>(smem);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 4, i = lane & 15;
+  const int tiles = (n + 15) / 16;  // per matrix
+  const bool is_up = wave >= GLU_ROWS_PAIRS;
+  const int pair = blockIdx.x * GLU_ROWS_PAIRS + (is_up ? wave - GLU_ROWS_PAIRS : wave);
+  const bool pair_ok = pair < tiles;
+  const int blocks_total = k / 64;
+  const int kb_hi = blocks_total;
+  // (a pair beyond N: tile 0 stands in and nothing is stored)
+  const bf16_t* w_ptr = w + (size_t)((pair_ok ? pair : 0) + (is_up ? tiles : 0)) * blocks_total * 1024 + lane * 8;
+
+  float4_t acc[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) acc[ct] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  Run16 w_ring[3][CHUNK];
+  float4_t a_next[A_ITERS];
+  auto fetch_w = [&](int kb, Run16 (&set)[CHUNK]) {  // no branch around a load: a block beyond K is read from the last block
+#pragma unroll
+    for (int u = 0; u < CHUNK; ++u) {
+      const int block = kb + u < kb_hi ? kb + u : kb_hi - 1;
+      set[u] = load_run_packed(w_ptr + (size_t)block * 1024);
+    }
+  };
+  auto fetch_a = [&](int kb) {
+#pragma unroll
+    for (int it = 0; it < A_ITERS; ++it) {
+      int v = tid + it * THREADS;  // vector index: (block u, row r, 16-byte piece p)
+      v = v < A_VECS ? v : A_VECS - 1;
+      const int u = v / (ROWS * 8), r = (v / 8) % ROWS, p = v % 8;
+      const int block = kb + u < kb_hi ? kb + u : kb_hi - 1;
+      a_next[it] = *reinterpret_cast<const float4_t*>(a + (size_t)(r < m ? r : 0) * k + (size_t)block * 64 + p * 8);
+    }
+  };
+  auto step = [&](int kb, Run16 (&w_cur)[CHUNK], Run16 (&w_far)[CHUNK]) {
+    __syncthreads();  // the previous chunk has been read by every wave
+#pragma unroll
+    for (int it = 0; it < A_ITERS; ++it) {
+      const int v = tid + it * THREADS;
+      if (v < A_VECS) {
+        const int u = v / (ROWS * 8), r = (v / 8) % ROWS, p = v % 8;
+        if (kb + u >= kb_hi) a_next[it] = float4_t{0.f, 0.f, 0.f, 0.f};  // (only in the last chunk)
+        *reinterpret_cast<float4_t*>(a_tile + (u * ROWS + r) * AS + p * 8) = a_next[it];
+      }
+    }
+    __syncthreads();
+    fetch_a(kb + CHUNK);
+    fetch_w(kb + 2 * CHUNK, w_far);
+#pragma unroll
+    for (int u = 0; u < CHUNK; ++u)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+        const bf16_t* src = a_tile + (u * ROWS + 16 * ct + i) * AS + 16 * g;
+        const bf16x8_t lo = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const float4_t*>(src));
+        const bf16x8_t hi = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const float4_t*>(src + 8));
+        acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[u].lo, lo, acc[ct], 0, 0, 0);
+        acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[u].hi, hi, acc[ct], 0, 0, 0);
+      }
+  };
+
+  fetch_a(0);
+  fetch_w(0, w_ring[0]);
+  fetch_w(CHUNK, w_ring[1]);
+  for (int kb = 0; kb < kb_hi;) {  // (unrolled by the ring's length: register sets are named at compile time)
+    step(kb, w_ring[0], w_ring[2]);
+    if ((kb += CHUNK) >= kb_hi) break;
+    step(kb, w_ring[1], w_ring[0]);
+    if ((kb += CHUNK) >= kb_hi) break;
+    step(kb, w_ring[2], w_ring[1]);
+    kb += CHUNK;
+  }
+  // Never true; keeps the loads that were asked for ahead alive on the way out of the loop (otherwise the compiler moves
+  // them behind the loop's exit tests, where nothing hides their latency).
+  if (k < 0) {
+    float4_t keep = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int it = 0; it < A_ITERS; ++it) keep += a_next[it];
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+      for (int u = 0; u < CHUNK; ++u) keep += __builtin_bit_cast(float4_t, w_ring[r][u].lo) + __builtin_bit_cast(float4_t, w_ring[r][u].hi);
+    acc[0] += keep;
+  }
+  // the up waves' sums go to the gate waves through LDS (the last chunk's activations are no longer needed)
+  __syncthreads();
+  float4_t* const handed = reinterpret_cast<float4_t*>(smem);
+  if (is_up) {
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) handed[((wave - GLU_ROWS_PAIRS) * CT + ct) * 64 + lane] = acc[ct];
+  }
+  __syncthreads();
+  if (is_up || !pair_ok) return;
+  const int col_n = pair * 16 + 4 * g;  // first of this lane's four output columns
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int col_m = 16 * ct + i;
+    if (col_m >= m) continue;
+    const float4_t up = handed[(wave * CT + ct) * 64 + lane];
+    __attribute__((aligned(8))) bf16_t four[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) four[j] = from_f32<bf16_t>(acc[ct][j] / (1.f + expf(-acc[ct][j])) * up[j]);
+    bf16_t* dst = out + (size_t)col_m * n + col_n;
+    if (col_n + 3 < n && n % 4 == 0) {
+      typedef float float2_t __attribute__((ext_vector_type(2)));
+      *reinterpret_cast<float2_t*>(dst) = *reinterpret_cast<const float2_t*>(four);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (col_n + j < n) dst[j] = four[j];
+    }
+  }
+}
+
+template <int P>
+static int launch_glu_rows(const void* a, const void* w, void* out, int m, int n, int k, hipStream_t stream) {
+  const int tiles = (n + 15) / 16;
+  const int blocks = (tiles + P - 1) / P;
+  if (m <= 32)
+    skinny_glu_rows_kernel<2, P><<<blocks, 128 * P, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, (bf16_t*)out, m, n, k);
+  else
+    skinny_glu_rows_kernel<4, P><<<blocks, 128 * P, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, (bf16_t*)out, m, n, k);
+  return (int)hipGetLastError();
+}
+
+// a [M, K] bfloat16 (17 <= M <= 64 pays; any M <= 64 works), w: [Wgate; Wup] packed (2n rows), out [M, n] bfloat16.
+// pairs: pairs of (gate, up) tiles per workgroup, 2 .. 6 (the caller aims at one workgroup per compute unit).
+extern "C" int velox_skinny_glu_rows_bf16(const void* a, const void* w, void* out, int m, int n, int k, int pairs, hipStream_t stream) {
+  if (m <= 0 || n <= 0) return 0;
+  if (k % 64 != 0 || k < 64 || m > 64) return -1;
+  switch (pairs) {
+    case 2: return launch_glu_rows<2>(a, w, out, m, n, k, stream);
+    case 3: return launch_glu_rows<3>(a, w, out, m, n, k, stream);
+    case 4: return launch_glu_rows<4>(a, w, out, m, n, k, stream);
+    case 5: return launch_glu_rows<5>(a, w, out, m, n, k, stream);
+    case 6: return launch_glu_rows<6>(a, w, out, m, n, k, stream);
+    default: return -1;
+  }
+}

@@ -82,6 +82,8 @@ class HipOps:
         c.velox_skinny_gemm_bf16.restype = _I
         c.velox_skinny_gemm_glu_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _I, _P, _P]
         c.velox_skinny_gemm_glu_bf16.restype = _I
+        c.velox_skinny_glu_rows_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
+        c.velox_skinny_glu_rows_bf16.restype = _I
         c.velox_skinny_gemm_splitk_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P]
         c.velox_skinny_gemm_splitk_bf16.restype = _I
         c.velox_argmax.argtypes = [_P, _P, _P, _I, _I, _I, _P]
@@ -422,6 +424,24 @@ class HipOps:
         two_n = gate_up_weight.shape[0]
         fused = (self.use_skinny_gemm and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16 and out_dtype == torch.bfloat16
                  and m <= 16 and k % 64 == 0 and two_n % 2 == 0 and x.dim() == 2 and gate_up_weight.shape[1] == k)
+        if (not fused and deferred is None and self.use_skinny_gemm and x.dim() == 2 and 16 < m <= 64 and k % 64 == 0 and two_n % 2 == 0
+                and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16 and out_dtype == torch.bfloat16
+                and gate_up_weight.shape[1] == k and (packed is not None or self.packed_weight(gate_up_weight, 2) is not None)):
+            # 17 .. 64 rows: the kernel that streams the packed weight once with the activation as its epilogue
+            packed = packed if packed is not None else self.packed_weight(gate_up_weight, 2)
+            n = two_n // 2
+            if packed.dtype != torch.bfloat16 or packed.numel() != 2 * ((n + 15) // 16) * 16 * k:
+                raise KernelError("linear_silu_mul: the packed weight does not match N and K")
+            self._check("x", x, torch.bfloat16, align=16)
+            out = torch.empty((m, n), dtype=torch.bfloat16, device=self.device)
+            # pairs of tiles per workgroup: a compute unit holds one such workgroup at a time, so the launch takes
+            # rounds x pairs; the fewest wins, then the larger workgroup (measured on MI355X at 64 rows: 37888 x 3584
+            # with 5 pairs 51 us, the library's product + SiLU kernel 58; 55296 x 5120 with 4 pairs 106 us against 114)
+            tiles = (n + 15) // 16
+            per_group = min(range(2, 7), key=lambda p: (-(-(-(-tiles // p)) // self.num_cus) * p, -p))
+            self._launched(self._core.velox_skinny_glu_rows_bf16(_ptr(x), _ptr(packed), _ptr(out), m, n, k, per_group if pairs is None else int(pairs), self._stream()),
+                           "skinny_glu_rows")
+            return out
         if not fused:
             return self.silu_mul(self.linear(deferred if deferred is not None else x, gate_up_weight, None, out_dtype))
         if packed is None:
