@@ -416,7 +416,10 @@ class HipOps:
 
     def linear_silu_mul(self, x: torch.Tensor, gate_up_weight: torch.Tensor, out_dtype: torch.dtype, waves: Optional[int] = None, pairs: Optional[int] = None, packed: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``silu(x Wgate^T) * (x Wup^T)`` for ``W = [Wgate; Wup]``.  Decode-sized bfloat16 batches run as one kernel that
-        never writes the [M, 2I] product; everything else is the product followed by the SiLU kernel."""
+        never writes the [M, 2I] product (up to 16 rows on any weight, 17 .. 64 rows on a registered one); everything else
+        is the product followed by the SiLU kernel.  ``waves`` and ``pairs`` override the launch shape the wrapper would
+        pick (up to 16 rows: waves per workgroup and gate/up tile pairs per wave; 17 .. 64 rows: ``pairs`` = tile pairs per
+        workgroup)."""
         deferred = x if isinstance(x, DeferredNorm) else None
         if deferred is not None:
             x = deferred.x
