@@ -449,6 +449,35 @@ def test_paged_attention_mixed_batch(ops, ref, dtype, nh, nkv, d, page):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,page", ATTN_SHAPES)
+@pytest.mark.parametrize("window", [None, 200])
+def test_paged_attention_decoded_tokens_before_portions(ops, ref, dtype, nh, nkv, d, page, window):
+    """A mixed step as the engine lays it out: single decoded tokens first (one of them behind a long context), then
+    portions of prompts.  Told how many sequences lead with one token, the wrapper sends those through the streaming
+    kernel with split keys and the rest through the general kernel; every row agrees with the plain reference, and
+    the decoded rows with the same rows in a step of their own, to the bit."""
+    from velox_amd.engine.batch import Workspace
+
+    seqs = [(1, 2300), (1, 97), (1, 1), (1, 640), (33, 141), (2, 66), (70, 70), (1, 30)]
+    case = _attention_case(dtype, nh, nkv, d, page, seqs, seed=d + nh + 2)
+    workspace = Workspace(torch.device("cuda"))
+    tolerance = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    want = _run_attention(ref, case, nh, nkv, d, page, window=window)
+    one_launch = _run_attention(ops, case, nh, nkv, d, page, window=window, workspace=workspace)
+    got = ops.paged_attention(case["qkv"], nh, nkv, d, case["k_cache"], case["v_cache"], page, case["tables"], case["cu"], case["kv"],
+                              case["max_q"], case["max_kv"], 1.0 / math.sqrt(d), window, False, workspace, decode_prefix=4).float()
+    torch.testing.assert_close(got, want, **tolerance)
+    torch.testing.assert_close(one_launch, want, **tolerance)
+    assert torch.equal(got[4:], one_launch[4:])  # the general kernel's rows do not depend on who else is in the launch
+    alone = dict(case)
+    alone["qkv"], alone["tables"], alone["kv"] = case["qkv"][:4].contiguous(), case["tables"][:4].contiguous(), case["kv"][:4].contiguous()
+    alone["cu"] = torch.arange(5, dtype=torch.int32, device="cuda")
+    alone["max_q"] = 1
+    decoded = _run_attention(ops, alone, nh, nkv, d, page, window=window, all_decode=True, workspace=workspace)
+    assert torch.equal(got[:4], decoded)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,d,page", [(28, 4, 128, 16), (32, 16, 64, 64), (16, 8, 32, 8), (24, 12, 48, 4)])
 @pytest.mark.parametrize("window", [None, 300])
 def test_paged_attention_long_portions(ops, ref, dtype, nh, nkv, d, page, window):

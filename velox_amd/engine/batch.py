@@ -71,6 +71,7 @@ class StepContext:
     groups: List[GroupBatch]
     workspace: Workspace
     cache: CacheManager = field(repr=False, default=None)
+    decode_prefix: int = 0  # how many of the first sequences bring exactly one token
 
     def cache_view(self, entry: int):
         return self.cache.view(entry, self.groups)
@@ -232,4 +233,5 @@ class BatchBuilder:
             rows=view("rows") if r else None,
             q_lens=q_lens, starts=starts, max_q_len=max(q_lens), all_decode=max(q_lens) == 1,
             groups=groups, workspace=workspace, cache=cache,
+            decode_prefix=next((i for i, n in enumerate(q_lens) if n != 1), len(q_lens)),
         )

@@ -637,7 +637,12 @@ class HipOps:
         return splits
 
     def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens,
-                        max_q_len, max_kv_len, scale, window, all_decode, workspace, splits: Optional[int] = None):
+                        max_q_len, max_kv_len, scale, window, all_decode, workspace, splits: Optional[int] = None, decode_prefix: int = 0):
+        """Attention of every token of the step over its sequence's keys in the cache.  ``decode_prefix``: how many of the
+        first sequences bring exactly one token (the engine puts decoded tokens before portions of prompts).  In a mixed
+        step those run through the streaming kernel with their keys split over workgroups, the others through the
+        general kernel: a single token behind many keys would otherwise be one workgroup's long walk that the
+        whole step waits for."""
         tokens = qkv.shape[0]
         width = qkv.shape[1] if qkv.dim() == 2 else -1  # rows may carry keys and values after the queries
         if width not in (num_heads * head_dim, (num_heads + 2 * num_kv_heads) * head_dim):
@@ -664,23 +669,36 @@ class HipOps:
             raise KernelError(f"max_q_len={max_q_len} outside [1, {tokens}]")
         lib = self.attention_library(head_dim)
         group = num_heads // num_kv_heads
-        row_tiles = (max_q_len * group + 63) // 64
-        if splits is None:
-            splits = self.choose_splits(num_seqs, num_kv_heads, row_tiles, max_kv_len, all_decode)
-        if num_seqs * splits > 65535:
-            raise KernelError(f"{num_seqs} sequences x {splits} splits exceed the launch grid")
         out = torch.empty((tokens, num_heads * head_dim), dtype=qkv.dtype, device=self.device)
-        part_o = part_lse = None
-        if splits > 1:
-            if workspace is None:
-                raise KernelError("split attention needs a workspace")
-            part_o = workspace.get("attention_partial_out", splits * tokens * num_heads * head_dim)
-            part_lse = workspace.get("attention_partial_lse", splits * tokens * num_heads)
-        status = lib.velox_paged_attention(
-            _ptr(qkv), width, _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), block_tables.shape[1], _ptr(cu_q), _ptr(kv_lens),
-            _ptr(out), _ptr(part_o), _ptr(part_lse), num_seqs, tokens, max_q_len, int(max_kv_len), num_heads, num_kv_heads,
-            block_size.bit_length() - 1, float(scale), int(window or 0), splits, _code(qkv.dtype), self._stream())
-        self._launched(status, "paged_attention")
+
+        def launch(first_seq: int, count: int, first_token: int, num_tokens: int, longest: int, decode_only: bool, splits: Optional[int]) -> None:
+            # sequences [first_seq, first_seq + count); their tokens are rows [first_token, first_token + num_tokens) of qkv
+            # and out.  cu_q holds absolute rows, so the general kernel takes qkv and out whole; the streaming kernel
+            # counts rows from its first sequence and takes the slices.
+            row_tiles = (longest * group + 63) // 64
+            if splits is None:
+                splits = self.choose_splits(count, num_kv_heads, row_tiles, max_kv_len, decode_only)
+            if count * splits > 65535:
+                raise KernelError(f"{count} sequences x {splits} splits exceed the launch grid")
+            part_o = part_lse = None
+            if splits > 1:
+                if workspace is None:
+                    raise KernelError("split attention needs a workspace")
+                part_o = workspace.get("attention_partial_out", splits * tokens * num_heads * head_dim)
+                part_lse = workspace.get("attention_partial_lse", splits * tokens * num_heads)
+            rows_in, rows_out = (qkv[first_token:first_token + num_tokens], out[first_token:first_token + num_tokens]) if decode_only else (qkv, out)
+            status = lib.velox_paged_attention(
+                _ptr(rows_in), width, _ptr(k_cache), _ptr(v_cache), _ptr(block_tables[first_seq:]), block_tables.shape[1],
+                _ptr(cu_q[first_seq:]), _ptr(kv_lens[first_seq:]), _ptr(rows_out), _ptr(part_o), _ptr(part_lse), count,
+                num_tokens if decode_only else tokens, longest, int(max_kv_len), num_heads, num_kv_heads,
+                block_size.bit_length() - 1, float(scale), int(window or 0), splits, _code(qkv.dtype), self._stream())
+            self._launched(status, "paged_attention")
+
+        if not all_decode and splits is None and 0 < decode_prefix < num_seqs and group <= 16:
+            launch(0, decode_prefix, 0, decode_prefix, 1, True, None)
+            launch(decode_prefix, num_seqs - decode_prefix, decode_prefix, tokens - decode_prefix, max_q_len, False, 1)
+        else:
+            launch(0, num_seqs, 0, tokens, max_q_len, bool(all_decode), splits)
         return out
 
     # -- sampling -------------------------------------------------------------------------------
