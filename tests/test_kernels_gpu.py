@@ -478,6 +478,27 @@ def test_paged_attention_decoded_tokens_before_portions(ops, ref, dtype, nh, nkv
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,page", [(28, 4, 128, 16), (4, 2, 16, 4), (2, 1, 256, 16), (12, 2, 128, 32)])
+def test_paged_attention_portions_behind_many_keys_split_them(ops, ref, dtype, nh, nkv, d, page):
+    """Few prompt tokens behind thousands of keys: the wrapper splits the keys over workgroups (and merges), alone and
+    behind decoded tokens that lead the step (whose rows the second launch's merge must leave alone)."""
+    from velox_amd.engine.batch import Workspace
+
+    seqs = [(1, 4500), (1, 10), (150, 4400), (40, 40), (2, 4200)]
+    case = _attention_case(dtype, nh, nkv, d, page, seqs, seed=d + nh + 3)
+    workspace = Workspace(torch.device("cuda"))
+    tolerance = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    assert ops.choose_portion_splits(192, nh // nkv, nkv, 4500) > 1
+    want = _run_attention(ref, case, nh, nkv, d, page)
+    for prefix in (0, 2):
+        got = ops.paged_attention(case["qkv"], nh, nkv, d, case["k_cache"], case["v_cache"], page, case["tables"], case["cu"], case["kv"],
+                                  case["max_q"], case["max_kv"], 1.0 / math.sqrt(d), None, False, workspace, decode_prefix=prefix).float()
+        torch.testing.assert_close(got, want, **tolerance)
+    one_pass = _run_attention(ops, case, nh, nkv, d, page, splits=1, workspace=workspace)
+    torch.testing.assert_close(one_pass, want, **tolerance)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,d,page", [(28, 4, 128, 16), (32, 16, 64, 64), (16, 8, 32, 8), (24, 12, 48, 4)])
 @pytest.mark.parametrize("window", [None, 300])
 def test_paged_attention_long_portions(ops, ref, dtype, nh, nkv, d, page, window):

@@ -137,7 +137,7 @@ class TorchOps:
             v_cache[pages, :, :, offsets] = v.to(v_cache.dtype)
 
     # -- attention over the paged cache -------------------------------------------------
-    def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens, max_q_len, max_kv_len, scale, window, all_decode, workspace, splits=None, decode_prefix=0):
+    def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens, max_q_len, max_kv_len, scale, window, all_decode, workspace, splits=None, decode_prefix=0, portions_max_kv_len=None):
         t = qkv.shape[0]
         group = num_heads // num_kv_heads
         q_all = qkv[:, : num_heads * head_dim].view(t, num_heads, head_dim)

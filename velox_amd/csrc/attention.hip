@@ -772,8 +772,8 @@ __global__ void __launch_bounds__(64 * WAVES) decode_attention_kernel(
 // out[token, head, :] = sum_s w_s * o_s / sum_s w_s,  w_s = exp(lse_s - max_s lse_s)
 template <typename T>
 __global__ void merge_splits_kernel(const float* __restrict__ part_o, const float* __restrict__ part_lse, T* __restrict__ out,
-                                    int nh, int splits, int total_tokens) {
-  const size_t token = blockIdx.x;
+                                    int nh, int splits, int total_tokens, int first_token) {
+  const size_t token = (size_t)blockIdx.x + first_token;  // (the launch covers tokens [first_token, total_tokens))
   const int head = blockIdx.y;
   const size_t stride = (size_t)total_tokens * nh;  // slots per split
   const size_t slot0 = token * nh + head;
@@ -811,13 +811,14 @@ template <typename T> constexpr int tile_keys() { return (sizeof(T) * D > 512) ?
 template <typename T>
 static int launch(const void* qkv, int qkv_stride, const void* k_cache, const void* v_cache, const int* block_tables, int table_width,
                   const int* cu_q, const int* kv_lens, void* out, float* part_o, float* part_lse, int num_seqs, int total_tokens,
-                  int max_q_len, int max_kv_len, int nh, int nkv, int page_shift, float scale, int window, int splits, hipStream_t stream) {
+                  int max_q_len, int max_kv_len, int nh, int nkv, int page_shift, float scale, int window, int splits, int first_token,
+                  hipStream_t stream) {
   constexpr int BN = tile_keys<T>();
   const int group = nh / nkv;
   // the streaming kernel keeps the page ids of a split's keys in LDS: they have to fit
   const int keys_per_split = (((max_kv_len + 15) / 16 + splits - 1) / splits) * 16;
   const bool ids_fit = (keys_per_split >> page_shift) + 2 <= DECODE_PAGE_IDS;
-  if (max_q_len == 1 && total_tokens == num_seqs && group <= 16 && page_shift >= 2 && sizeof(T) * D <= 512 && ids_fit) {
+  if (max_q_len == 1 && total_tokens == num_seqs && first_token == 0 && group <= 16 && page_shift >= 2 && sizeof(T) * D <= 512 && ids_fit) {
     // every sequence decodes one token: the streaming kernel.  Register sets per wave: one being computed, the others
     // in flight.  (For steps with one workgroup per compute unit, twice as many sets and eight waves per workgroup
     // were both measured slower on MI355X.)
@@ -827,7 +828,7 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
         nh, nkv, page_shift, scale, window, splits, total_tokens);
     int status = (int)hipGetLastError();
     if (status != 0 || splits == 1) return status;
-    merge_splits_kernel<T><<<dim3(total_tokens, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens);
+    merge_splits_kernel<T><<<dim3(total_tokens, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens, 0);
     return (int)hipGetLastError();
   }
   // Eight waves per workgroup when bfloat16 portions are long enough to fill their rows and the step brings enough rows
@@ -838,7 +839,7 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
   // keys 315 us against 426 the other way round; the two meet where an average row reads about 1,300 keys.
   constexpr int WIDE = (sizeof(T) == 2 && D <= 128) ? 2 : 1;
   const int rows = max_q_len * group;
-  if (WIDE == 2 && rows > 64 && (long long)total_tokens * group / 128 * nkv >= compute_units()) {
+  if (WIDE == 2 && rows > 64 && (long long)total_tokens * group / 128 * nkv * splits >= compute_units()) {
     if (max_kv_len - max_q_len / 2 <= 1280 || rows < 192) {  // (keys an average row reads)
       dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
       paged_attention_kernel<T, BN, 1, 1, 8><<<grid, 512, 0, stream>>>(
@@ -864,22 +865,26 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
   }
   int status = (int)hipGetLastError();
   if (status != 0 || splits == 1) return status;
-  merge_splits_kernel<T><<<dim3(total_tokens, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens);
+  merge_splits_kernel<T><<<dim3(total_tokens - first_token, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens,
+                                                                                               first_token);
   return (int)hipGetLastError();
 }
 
 extern "C" int velox_attention_head_dim() { return D; }
 
 // part_o: float32 [splits, total_tokens, nh, D]; part_lse: float32 [splits, total_tokens, nh]; both unused when splits == 1.
+// first_token: the sequences given (cu_q holds rows of qkv and out) cover rows [first_token, total_tokens); a launch for
+// the later sequences of a step passes its first row here so that only those rows are merged.
 extern "C" int velox_paged_attention(const void* qkv, int qkv_stride, const void* k_cache, const void* v_cache,
                                      const int* block_tables, int table_width, const int* cu_q, const int* kv_lens, void* out,
                                      float* part_o, float* part_lse, int num_seqs, int total_tokens, int max_q_len, int max_kv_len,
-                                     int nh, int nkv, int page_shift, float scale, int window, int splits, int dtype, hipStream_t stream) {
+                                     int nh, int nkv, int page_shift, float scale, int window, int splits, int first_token, int dtype,
+                                     hipStream_t stream) {
   if (num_seqs <= 0 || total_tokens <= 0) return 0;
-  if (nh % nkv != 0 || splits < 1 || page_shift < 0 || max_kv_len < 1) return -1;
+  if (nh % nkv != 0 || splits < 1 || page_shift < 0 || max_kv_len < 1 || first_token < 0 || first_token >= total_tokens) return -1;
   if (dtype == VELOX_BF16)
     return launch<bf16_t>(qkv, qkv_stride, k_cache, v_cache, block_tables, table_width, cu_q, kv_lens, out, part_o, part_lse, num_seqs,
-                          total_tokens, max_q_len, max_kv_len, nh, nkv, page_shift, scale, window, splits, stream);
+                          total_tokens, max_q_len, max_kv_len, nh, nkv, page_shift, scale, window, splits, first_token, stream);
   return launch<float>(qkv, qkv_stride, k_cache, v_cache, block_tables, table_width, cu_q, kv_lens, out, part_o, part_lse, num_seqs,
-                       total_tokens, max_q_len, max_kv_len, nh, nkv, page_shift, scale, window, splits, stream);
+                       total_tokens, max_q_len, max_kv_len, nh, nkv, page_shift, scale, window, splits, first_token, stream);
 }

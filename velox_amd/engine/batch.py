@@ -35,6 +35,7 @@ class GroupBatch:
     slot_mapping: torch.Tensor  # int32 [T]: page * page_size + offset of every token's key
     kv_lens: torch.Tensor  # int32 [B]: keys in the cache once this step's are written
     max_kv_len: int
+    max_kv_len_of_portions: int = 0  # the same over the sequences behind the leading one-token sequences (0: there are none)
 
 
 class Workspace:
@@ -181,6 +182,8 @@ class BatchBuilder:
             source[:b_real] = np.asarray(ids_on_device[1], dtype=np.int32)
         put("source", source, b)
         max_kv: List[int] = []
+        max_kv_portions: List[int] = []
+        decode_prefix = next((i for i, n in enumerate(q_lens) if n != 1), len(q_lens))
         for g, group in enumerate(cache.groups):
             kv = np.ones(b, dtype=np.int32)
             slot_map = np.zeros(t, dtype=np.int32)
@@ -202,6 +205,7 @@ class BatchBuilder:
             put(f"slot{g}", slot_map, t)
             put(f"bt{g}", tables, b * width)
             max_kv.append(int(kv.max()))
+            max_kv_portions.append(int(kv[decode_prefix:].max()) if decode_prefix < b else 0)
 
         device[:offset].copy_(self._host[index][:offset], non_blocking=True)
         if self._events[index] is not None:
@@ -224,6 +228,7 @@ class BatchBuilder:
                 slot_mapping=view(f"slot{g}"),
                 kv_lens=view(f"kv{g}"),
                 max_kv_len=max_kv[g],
+                max_kv_len_of_portions=max_kv_portions[g],
             )
             for g in range(len(cache.groups))
         ]
@@ -233,5 +238,5 @@ class BatchBuilder:
             rows=view("rows") if r else None,
             q_lens=q_lens, starts=starts, max_q_len=max(q_lens), all_decode=max(q_lens) == 1,
             groups=groups, workspace=workspace, cache=cache,
-            decode_prefix=next((i for i, n in enumerate(q_lens) if n != 1), len(q_lens)),
+            decode_prefix=decode_prefix,
         )

@@ -101,7 +101,7 @@ class HipOps:
         lib = self._attention.get(head_dim)
         if lib is None:
             lib = ctypes.CDLL(build.ensure_attention(head_dim))
-            lib.velox_paged_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P]
+            lib.velox_paged_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P]
             lib.velox_paged_attention.restype = _I
             lib.velox_attention_head_dim.restype = _I
             if lib.velox_attention_head_dim() != head_dim:
@@ -636,13 +636,26 @@ class HipOps:
             splits = 1
         return splits
 
+    def choose_portion_splits(self, num_tokens: int, group: int, num_kv_heads: int, max_kv_len: int) -> int:
+        """Splits of the key range for portions of prompts.  Few tokens behind many keys are few workgroups that each walk
+        all the keys: with the keys split the step fills the GPU with the large workgroups (measured on MI355X, 512
+        tokens behind 8,192 keys: 157 us in one pass, 104 us in four splits and their merge; behind 32,768: 611 and 331).
+        At least 1,024 keys per split, and none below 4,096 keys, where one pass is as quick."""
+        if max_kv_len < 4096:
+            return 1
+        blocks = max(1, num_tokens * group // 128 * num_kv_heads)  # workgroups of 128 rows, as the launch counts them
+        if blocks >= self.num_cus:
+            return 1
+        return max(1, min(-(-self.num_cus // blocks), max_kv_len // 1024, 16))
+
     def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens,
-                        max_q_len, max_kv_len, scale, window, all_decode, workspace, splits: Optional[int] = None, decode_prefix: int = 0):
+                        max_q_len, max_kv_len, scale, window, all_decode, workspace, splits: Optional[int] = None, decode_prefix: int = 0,
+                        portions_max_kv_len: Optional[int] = None):
         """Attention of every token of the step over its sequence's keys in the cache.  ``decode_prefix``: how many of the
         first sequences bring exactly one token (the engine puts decoded tokens before portions of prompts).  In a mixed
         step those run through the streaming kernel with their keys split over workgroups, the others through the
         general kernel: a single token behind many keys would otherwise be one workgroup's long walk that the
-        whole step waits for."""
+        whole step waits for.  ``portions_max_kv_len``: the most keys any sequence behind that prefix holds (default: ``max_kv_len``)."""
         tokens = qkv.shape[0]
         width = qkv.shape[1] if qkv.dim() == 2 else -1  # rows may carry keys and values after the queries
         if width not in (num_heads * head_dim, (num_heads + 2 * num_kv_heads) * head_dim):
@@ -678,6 +691,8 @@ class HipOps:
             row_tiles = (longest * group + 63) // 64
             if splits is None:
                 splits = self.choose_splits(count, num_kv_heads, row_tiles, max_kv_len, decode_only)
+                if not decode_only:
+                    splits = self.choose_portion_splits(num_tokens, group, num_kv_heads, min(max_kv_len, portions_max_kv_len or max_kv_len))
             if count * splits > 65535:
                 raise KernelError(f"{count} sequences x {splits} splits exceed the launch grid")
             part_o = part_lse = None
@@ -691,12 +706,13 @@ class HipOps:
                 _ptr(rows_in), width, _ptr(k_cache), _ptr(v_cache), _ptr(block_tables[first_seq:]), block_tables.shape[1],
                 _ptr(cu_q[first_seq:]), _ptr(kv_lens[first_seq:]), _ptr(rows_out), _ptr(part_o), _ptr(part_lse), count,
                 num_tokens if decode_only else tokens, longest, int(max_kv_len), num_heads, num_kv_heads,
-                block_size.bit_length() - 1, float(scale), int(window or 0), splits, _code(qkv.dtype), self._stream())
+                block_size.bit_length() - 1, float(scale), int(window or 0), splits, 0 if decode_only else first_token, _code(qkv.dtype),
+                self._stream())
             self._launched(status, "paged_attention")
 
         if not all_decode and splits is None and 0 < decode_prefix < num_seqs and group <= 16:
             launch(0, decode_prefix, 0, decode_prefix, 1, True, None)
-            launch(decode_prefix, num_seqs - decode_prefix, decode_prefix, tokens - decode_prefix, max_q_len, False, 1)
+            launch(decode_prefix, num_seqs - decode_prefix, decode_prefix, tokens - decode_prefix, max_q_len, False, None)
         else:
             launch(0, num_seqs, 0, tokens, max_q_len, bool(all_decode), splits)
         return out

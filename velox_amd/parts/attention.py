@@ -102,7 +102,7 @@ class AttentionMixer(Mixer):
             meta.block_tables, ctx.cu_q, meta.kv_lens,
             ctx.max_q_len, meta.max_kv_len, self.scale, self.window,
             ctx.all_decode, ctx.workspace,
-            decode_prefix=getattr(ctx, "decode_prefix", 0),
+            decode_prefix=getattr(ctx, "decode_prefix", 0), portions_max_kv_len=getattr(meta, "max_kv_len_of_portions", 0) or None,
         )
         return ops.linear(attn, self.o_weight, None, ctx.dtype, partials_ok=True, residual_norm=sink)
 
