@@ -502,28 +502,30 @@ extern "C" int velox_skinny_qkv_rotary_bf16(const void* a, const void* w, const 
 // bfloat16(residual * norm_weight), and sums[m][block] = the sum of squares of the block's 16 new residual values of
 // row m.  Whoever multiplies `next` scales its rows with the sums (RowScale above): the norm costs no kernel.
 // ---------------------------------------------------------------------------------------------------------------
-template <int WAVES>
+template <int WAVES, int RT = 1>
 __global__ void __launch_bounds__(WAVES * 64) skinny_residual_norm_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
                                                                           float* __restrict__ residual, const float* __restrict__ norm_weight,
                                                                           bf16_t* __restrict__ next, float* __restrict__ sums, int m, int n, int k,
                                                                           int a_packed, bf16_t* __restrict__ next_packed) {
-  __shared__ float4_t partial[WAVES][1][64];
-  // what the epilogue reads is fetched before the main loop (by the 64 threads that will need it)
-  const int l = threadIdx.x;
+  __shared__ float4_t partial[WAVES][RT][64];
+  // what the epilogue reads is fetched before the main loop (by the 64 threads per tile that will need it)
+  const int l = threadIdx.x & 63, tile = threadIdx.x >> 6;  // (in the epilogue: wave t finishes tile t)
   const int row = l & 15;
-  const int col = blockIdx.x * 16 + 4 * (l >> 4);  // first of this lane's four columns
+  const int tiles_total = (n + 15) / 16;
+  const int tile_n = blockIdx.x * RT + tile;
+  const int col = tile_n * 16 + 4 * (l >> 4);  // first of this lane's four columns
   float old_residual[4], weight[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const bool inside = l < 64 && row < m && col + j < n;
+    const bool inside = tile < RT && row < m && col + j < n;
     old_residual[j] = inside ? residual[(size_t)row * n + col + j] : 0.f;
     weight[j] = inside ? norm_weight[col + j] : 0.f;
   }
-  skinny_partial_sums<1, 1, WAVES, false, true>(a, a_packed, w, m, n, k, partial);
-  if (l >= 64) return;
-  float4_t sum = partial[0][0][l];
+  skinny_partial_sums<RT, 1, WAVES, false, true>(a, a_packed, w, m, n, k, partial);
+  if (tile >= RT || tile_n >= tiles_total) return;
+  float4_t sum = partial[0][tile][l];
 #pragma unroll
-  for (int wv = 1; wv < WAVES; ++wv) sum += partial[wv][0][l];
+  for (int wv = 1; wv < WAVES; ++wv) sum += partial[wv][tile][l];
   float squares = 0.f;
   if (row < m) {
     __attribute__((aligned(8))) bf16_t four[4];
@@ -545,23 +547,27 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_residual_norm_kernel(const 
   // the four lane groups hold four columns each of the same rows: added in a fixed order
   squares += __shfl_xor(squares, 16, VELOX_WAVE);
   squares += __shfl_xor(squares, 32, VELOX_WAVE);
-  if (l < 16) sums[(size_t)l * gridDim.x + blockIdx.x] = squares;
+  if (l < 16) sums[(size_t)l * tiles_total + tile_n] = squares;
 }
 
 // a [M, K] bfloat16 (M <= 16; a_packed != 0: in the lanes' order, see packed_row_offset), w packed [N, K]; sums: float32
 // [16][ceil(N / 16)].  next_packed (or null; needs N % 64 == 0): room for N / 64 * 1024 elements, `next` once more in the
-// lanes' order.  waves: 4, 8 or 16.
+// lanes' order.  waves: 4, 8 or 16.  row_tiles: 16-row tiles of W per workgroup, 1 or 2 (with 2 every activation
+// fragment a wave loads feeds two tiles: half the activations' bytes, half as many workgroups; eight waves).
 extern "C" int velox_skinny_residual_norm_bf16(const void* a, const void* w, float* residual, const float* norm_weight, void* next,
-                                               float* sums, int m, int n, int k, int waves, int a_packed, void* next_packed, hipStream_t stream) {
+                                               float* sums, int m, int n, int k, int waves, int row_tiles, int a_packed, void* next_packed,
+                                               hipStream_t stream) {
   if (m <= 0 || n <= 0) return 0;
   if (m > 16 || k % 64 != 0 || (next_packed != nullptr && n % 64 != 0)) return -1;
-  const int blocks = (n + 15) / 16;
-  if (waves >= 16)
-    skinny_residual_norm_kernel<16><<<blocks, 16 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, residual, norm_weight, (bf16_t*)next, sums, m, n, k, a_packed, (bf16_t*)next_packed);
-  else if (waves >= 8)
-    skinny_residual_norm_kernel<8><<<blocks, 8 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, residual, norm_weight, (bf16_t*)next, sums, m, n, k, a_packed, (bf16_t*)next_packed);
-  else
-    skinny_residual_norm_kernel<4><<<blocks, 4 * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, residual, norm_weight, (bf16_t*)next, sums, m, n, k, a_packed, (bf16_t*)next_packed);
+  const int tiles = (n + 15) / 16;
+#define RESIDUAL_NORM(W, RT) \
+  skinny_residual_norm_kernel<W, RT><<<(tiles + RT - 1) / RT, W * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, residual, norm_weight, (bf16_t*)next, \
+                                                                                    sums, m, n, k, a_packed, (bf16_t*)next_packed)
+  if (row_tiles >= 2) RESIDUAL_NORM(8, 2);
+  else if (waves >= 16) RESIDUAL_NORM(16, 1);
+  else if (waves >= 8) RESIDUAL_NORM(8, 1);
+  else RESIDUAL_NORM(4, 1);
+#undef RESIDUAL_NORM
   return (int)hipGetLastError();
 }
 

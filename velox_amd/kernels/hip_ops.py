@@ -76,7 +76,7 @@ class HipOps:
         c.velox_rope_kv_write_partial_bf16.restype = _I
         c.velox_gemm_fma.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
         c.velox_skinny_gemm_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _I, _P]
-        c.velox_skinny_residual_norm_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P]
+        c.velox_skinny_residual_norm_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P]
         c.velox_skinny_residual_norm_bf16.restype = _I
         c.velox_row_scale_apply.argtypes = [_P, _P, _I, _F, _F, _P, _I, _I, _P]
         c.velox_skinny_gemm_bf16.restype = _I
@@ -337,7 +337,7 @@ class HipOps:
                     self._mm_out_dtype_ok = False
         return self.gemm_fma(x, weight, bias, out_dtype)
 
-    def _linear_into_residual(self, x: torch.Tensor, weight: torch.Tensor, sink: ResidualSink, waves: Optional[int] = None) -> Optional[DeferredNorm]:
+    def _linear_into_residual(self, x: torch.Tensor, weight: torch.Tensor, sink: ResidualSink, waves: Optional[int] = None, row_tiles: Optional[int] = None) -> Optional[DeferredNorm]:
         """``sink.residual += x @ weight^T`` with the first half of ``sink.norm`` in the same kernel, if this product
         qualifies (bfloat16, at most 16 rows, registered weight, a norm that can be split); None otherwise."""
         form = sink.norm.deferred_form()
@@ -352,12 +352,16 @@ class HipOps:
         self._check("residual", residual, torch.float32, (m, n), align=16)
         self._check("norm weight", norm_weight, torch.float32, (n,))
         blocks = (n + 15) // 16
+        if row_tiles is None:
+            # one 16-row tile of the weight per workgroup while that is at most one workgroup per compute unit; a wider
+            # weight takes two (measured on MI355X at 8 rows: 5120 x 27648 65.8 -> 58.5 us, 3584 x 18944 27.8 -> 41.4)
+            row_tiles = 2 if blocks > self.num_cus else 1
         out = torch.empty((m, n), dtype=torch.bfloat16, device=self.device)
         sums = torch.empty((16, blocks), dtype=torch.float32, device=self.device)
         x_packed = self._packed_rows_of(x, k)
         out_packed = self._room_for_packed_rows(m, n)
         status = self._core.velox_skinny_residual_norm_bf16(_ptr(x if x_packed is None else x_packed), _ptr(packed), _ptr(residual), _ptr(norm_weight),
-                                                            _ptr(out), _ptr(sums), m, n, k, int(waves or 8), int(x_packed is not None), _ptr(out_packed),
+                                                            _ptr(out), _ptr(sums), m, n, k, int(waves or 8), int(row_tiles), int(x_packed is not None), _ptr(out_packed),
                                                             self._stream())
         self._launched(status, "skinny_residual_norm")
         if out_packed is not None:
