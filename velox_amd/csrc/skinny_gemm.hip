@@ -90,12 +90,15 @@ struct NoHooks {
 // a_packed != 0: the activations come in the lanes' order (see packed_row_offset; only with CT = 1).
 template <int RT, int CT, int WAVES, bool GLU, bool PACKED, typename Hooks = NoHooks>
 __device__ __forceinline__ void skinny_partial_sums(const bf16_t* __restrict__ a, int a_packed, const bf16_t* __restrict__ w, int m, int n, int k,
-                                                    float4_t (&partial)[WAVES][RT * CT][64], Hooks hooks = Hooks()) {
+                                                    float4_t (&partial)[WAVES][RT * CT][64], Hooks hooks = Hooks(), int tile0 = -1, int w_half = -1) {
   constexpr int UNROLL = 4;  // blocks of 64 indices whose loads are issued together
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int g = lane >> 4, i = lane & 15;
   constexpr int RTO = GLU ? RT / 2 : RT;  // row tiles that become output columns
-  const int n0 = blockIdx.x * 16 * RTO;
+  // tile0 >= 0: the workgroup's first row tile is given (else blockIdx.x counts groups of RTO tiles); w_half = 0 or 1 with
+  // a packed W: only rows 8 w_half .. 8 w_half + 7 of the tile are read, the others count as zeros (two workgroups can
+  // then share a tile, each with half the bytes to fetch)
+  const int n0 = (tile0 >= 0 ? tile0 : blockIdx.x * RTO) * 16;
 
   // this wave's share of K, in blocks of 64
   const int blocks_total = k / 64;
@@ -115,6 +118,7 @@ __device__ __forceinline__ void skinny_partial_sums(const bf16_t* __restrict__ a
       const size_t tile = (size_t)(n0 / 16 + rt % RTO) + (rt >= RTO ? tiles_per_matrix : 0);
       w_ok[rt] = n0 + 16 * (rt % RTO) < n;  // padded rows are zeros in memory
       w_ptr[rt] = w + (w_ok[rt] ? tile : 0) * (size_t)(k / 64) * 1024 + lane * 8;
+      w_ok[rt] = w_ok[rt] && (w_half < 0 || (i >> 3) == w_half);
     } else {
       const size_t row = (size_t)col + (rt >= RTO ? n : 0);  // its row in W
       w_ptr[rt] = w + (w_ok[rt] ? row : 0) * k + 16 * g;
@@ -502,32 +506,38 @@ extern "C" int velox_skinny_qkv_rotary_bf16(const void* a, const void* w, const 
 // bfloat16(residual * norm_weight), and sums[m][block] = the sum of squares of the block's 16 new residual values of
 // row m.  Whoever multiplies `next` scales its rows with the sums (RowScale above): the norm costs no kernel.
 // ---------------------------------------------------------------------------------------------------------------
-template <int WAVES, int RT = 1>
+// HALF: two workgroups share a 16-row tile of W, each reading eight of its rows (a narrow W then still gives every compute
+// unit a workgroup); the sums of squares are then per block of 8 columns.
+template <int WAVES, int RT = 1, bool HALF = false>
 __global__ void __launch_bounds__(WAVES * 64) skinny_residual_norm_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
                                                                           float* __restrict__ residual, const float* __restrict__ norm_weight,
                                                                           bf16_t* __restrict__ next, float* __restrict__ sums, int m, int n, int k,
                                                                           int a_packed, bf16_t* __restrict__ next_packed) {
+  static_assert(!HALF || RT == 1, "half tiles come one to a workgroup");
   __shared__ float4_t partial[WAVES][RT][64];
   // what the epilogue reads is fetched before the main loop (by the 64 threads per tile that will need it)
   const int l = threadIdx.x & 63, tile = threadIdx.x >> 6;  // (in the epilogue: wave t finishes tile t)
   const int row = l & 15;
   const int tiles_total = (n + 15) / 16;
-  const int tile_n = blockIdx.x * RT + tile;
+  const int tile_n = HALF ? blockIdx.x >> 1 : blockIdx.x * RT + tile;
+  const int half = HALF ? blockIdx.x & 1 : -1;
+  const bool mine = !HALF || (l >> 5) == half;  // (lane group g holds rows 4g .. 4g + 3 of the tile)
   const int col = tile_n * 16 + 4 * (l >> 4);  // first of this lane's four columns
   float old_residual[4], weight[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const bool inside = tile < RT && row < m && col + j < n;
+    const bool inside = tile < RT && mine && row < m && col + j < n;
     old_residual[j] = inside ? residual[(size_t)row * n + col + j] : 0.f;
     weight[j] = inside ? norm_weight[col + j] : 0.f;
   }
-  skinny_partial_sums<RT, 1, WAVES, false, true>(a, a_packed, w, m, n, k, partial);
+  if constexpr (HALF) skinny_partial_sums<1, 1, WAVES, false, true>(a, a_packed, w, m, n, k, partial, NoHooks(), tile_n, half);
+  else skinny_partial_sums<RT, 1, WAVES, false, true>(a, a_packed, w, m, n, k, partial);
   if (tile >= RT || tile_n >= tiles_total) return;
   float4_t sum = partial[0][tile][l];
 #pragma unroll
   for (int wv = 1; wv < WAVES; ++wv) sum += partial[wv][tile][l];
   float squares = 0.f;
-  if (row < m) {
+  if (row < m && mine) {
     __attribute__((aligned(8))) bf16_t four[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -544,29 +554,35 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_residual_norm_kernel(const 
     typedef float float2_t __attribute__((ext_vector_type(2)));
     if (next_packed) *reinterpret_cast<float2_t*>(next_packed + packed_row_offset(row, col)) = *reinterpret_cast<const float2_t*>(four);
   }
-  // the four lane groups hold four columns each of the same rows: added in a fixed order
+  // the lane groups hold four columns each of the same rows: added in a fixed order
   squares += __shfl_xor(squares, 16, VELOX_WAVE);
-  squares += __shfl_xor(squares, 32, VELOX_WAVE);
-  if (l < 16) sums[(size_t)l * tiles_total + tile_n] = squares;
+  if constexpr (HALF) {
+    if ((l >> 4) == 2 * half) sums[(size_t)row * (2 * tiles_total) + blockIdx.x] = squares;
+  } else {
+    squares += __shfl_xor(squares, 32, VELOX_WAVE);
+    if (l < 16) sums[(size_t)l * tiles_total + tile_n] = squares;
+  }
 }
 
 // a [M, K] bfloat16 (M <= 16; a_packed != 0: in the lanes' order, see packed_row_offset), w packed [N, K]; sums: float32
-// [16][ceil(N / 16)].  next_packed (or null; needs N % 64 == 0): room for N / 64 * 1024 elements, `next` once more in the
-// lanes' order.  waves: 4, 8 or 16.  row_tiles: 16-row tiles of W per workgroup, 1 or 2 (with 2 every activation
-// fragment a wave loads feeds two tiles: half the activations' bytes, half as many workgroups; eight waves).
+// [16][blocks], blocks = ceil(N / 16), or twice that with row_tiles = 0.  next_packed (or null; needs N % 64 == 0): room
+// for N / 64 * 1024 elements, `next` once more in the lanes' order.  waves: 4, 8 or 16.  row_tiles: 16-row tiles of W per
+// workgroup: 1; 2 (every activation fragment a wave loads feeds two tiles: half the activations' bytes, half as many
+// workgroups; eight waves); or 0 for half a tile (twice as many workgroups; eight waves).
 extern "C" int velox_skinny_residual_norm_bf16(const void* a, const void* w, float* residual, const float* norm_weight, void* next,
                                                float* sums, int m, int n, int k, int waves, int row_tiles, int a_packed, void* next_packed,
                                                hipStream_t stream) {
   if (m <= 0 || n <= 0) return 0;
   if (m > 16 || k % 64 != 0 || (next_packed != nullptr && n % 64 != 0)) return -1;
   const int tiles = (n + 15) / 16;
-#define RESIDUAL_NORM(W, RT) \
-  skinny_residual_norm_kernel<W, RT><<<(tiles + RT - 1) / RT, W * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, residual, norm_weight, (bf16_t*)next, \
-                                                                                    sums, m, n, k, a_packed, (bf16_t*)next_packed)
-  if (row_tiles >= 2) RESIDUAL_NORM(8, 2);
-  else if (waves >= 16) RESIDUAL_NORM(16, 1);
-  else if (waves >= 8) RESIDUAL_NORM(8, 1);
-  else RESIDUAL_NORM(4, 1);
+#define RESIDUAL_NORM(W, RT, HALF, GRID) \
+  skinny_residual_norm_kernel<W, RT, HALF><<<GRID, W * 64, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, residual, norm_weight, (bf16_t*)next, sums, \
+                                                                         m, n, k, a_packed, (bf16_t*)next_packed)
+  if (row_tiles == 0) RESIDUAL_NORM(8, 1, true, 2 * tiles);
+  else if (row_tiles >= 2) RESIDUAL_NORM(8, 2, false, (tiles + 1) / 2);
+  else if (waves >= 16) RESIDUAL_NORM(16, 1, false, tiles);
+  else if (waves >= 8) RESIDUAL_NORM(8, 1, false, tiles);
+  else RESIDUAL_NORM(4, 1, false, tiles);
 #undef RESIDUAL_NORM
   return (int)hipGetLastError();
 }
