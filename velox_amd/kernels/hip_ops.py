@@ -687,6 +687,8 @@ class HipOps:
             raise KernelError(f"paged_attention: the scale must be positive, got {scale}")
         if max_q_len < 1 or max_q_len > tokens:
             raise KernelError(f"max_q_len={max_q_len} outside [1, {tokens}]")
+        if not 0 <= decode_prefix <= num_seqs or num_seqs > tokens:
+            raise KernelError(f"decode_prefix={decode_prefix} does not fit {num_seqs} sequences with {tokens} tokens")
         lib = self.attention_library(head_dim)
         group = num_heads // num_kv_heads
         out = torch.empty((tokens, num_heads * head_dim), dtype=qkv.dtype, device=self.device)
