@@ -165,6 +165,19 @@ class ModelRunner:
         ctx.rows = ctx.rows[:bucket]
         return ctx
 
+    @torch.no_grad()
+    def warm_prefill(self, num_tokens: int) -> None:
+        """Runs one prompt portion of ``num_tokens`` tokens on the null page and drops the result, so that whatever a
+        first portion pays once (the matrix library loads its kernels for a data type at first use, tens of
+        milliseconds, and picks a kernel per shape) is paid before the first request."""
+        from ..cache.manager import SequenceCache
+
+        num_tokens = max(2, min(int(num_tokens), self.builder.max_num_tokens, self.cache.max_model_len))
+        pages = (num_tokens + self.cache.page_size - 1) // self.cache.page_size
+        null_seq = SequenceCache(slot=self.cache.state.pad_slot, tables=[[0] * pages for _ in self.cache.groups], released=[0 for _ in self.cache.groups])
+        ctx = self.builder.build([StepEntry(null_seq, [0] * num_tokens, 0, [num_tokens - 1])], self.ops, self.dtype, self.workspace)
+        self._forward(ctx)
+
     def _replay(self, bucket: int, entries: Sequence[StepEntry], ids_on_device: Optional[tuple] = None) -> torch.Tensor:
         graph, logits, _ = self._graphs[bucket]
         if bucket in self._short_graphs and all(e.start < SHORT_CONTEXT_KEYS for e in entries):
