@@ -149,7 +149,8 @@ class Engine:
         self.runner.capture_decode_graphs()
         # one prompt portion of the usual size on the null page: the first request does not pay for the matrix library's
         # first use of a data type and of these shapes (about 50 ms for the first portion otherwise)
-        self.runner.warm_prefill(self.config.max_prefill_chunk_size)
+        for count in sorted({self.config.max_prefill_chunk_size, self.config.max_num_batched_tokens}):
+            self.runner.warm_prefill(count)  # (a step's portions together may reach the token budget)
         torch.cuda.synchronize()
 
     def tune_matrix_products(self, token_counts: Sequence[int]) -> int:
