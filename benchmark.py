@@ -214,7 +214,7 @@ def main(argv=None) -> int:
         if args.tune_library:
             from velox_amd.engine.runner import decode_buckets
 
-            engine.tune_matrix_products([args.max_prefill_chunk_size] + [b for b in decode_buckets(max_num_seqs) if b > 16])
+            engine.tune_matrix_products([args.max_prefill_chunk_size, max(args.max_num_batched_tokens, max_num_seqs)] + [b for b in decode_buckets(max_num_seqs) if b > 16])
         vocab = engine.model.spec.vocab_size
         limit = engine.max_model_len - args.max_tokens - 1
         if limit < 1:
