@@ -3,6 +3,9 @@
 // One workgroup per row; every reduction runs in a fixed order, so a row's result depends on that
 // row alone.
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 #define SAMPLE_THREADS 1024
 
@@ -100,6 +103,62 @@ extern "C" int velox_argmax(const float* logits, int* out, void* partial, int ro
   argmax_kernel<<<dim3(rows, chunks), SAMPLE_THREADS, 0, stream>>>(logits, out, (Best*)partial, vocab, chunk);
   if (chunks > 1) argmax_merge_kernel<<<rows, 64, 0, stream>>>((const Best*)partial, out, chunks);
   VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---- the entry point that allocates nothing (declared in no_alloc.h) ----------------------------------------------
+// The chunks' best pairs of velox_argmax_static.  In host code this name is only a stand-in for the symbol: each GPU
+// holds its own copy at its own address, which hipGetSymbolAddress gives with that GPU current; host code passes
+// that address on, never the name.
+static __device__ __align__(256) unsigned char argmax_static_scratch[VELOX_ARGMAX_STATIC_BYTES];
+
+#define VELOX_MAX_DEVICES 64
+static void* argmax_scratch_of_device[VELOX_MAX_DEVICES];  // the address of each GPU's copy, looked up once
+static std::mutex argmax_scratch_lock;
+
+static int argmax_scratch_of_current_device(void** address) {
+  int device = -1;
+  hipError_t status = hipGetDevice(&device);
+  if (status != hipSuccess) return (int)status;
+  if (device < 0 || device >= VELOX_MAX_DEVICES) return VELOX_NO_ALLOC_NO_SCRATCH;
+  std::lock_guard<std::mutex> guard(argmax_scratch_lock);
+  if (argmax_scratch_of_device[device] == nullptr) {
+    void* found = nullptr;
+    status = hipGetSymbolAddress(&found, HIP_SYMBOL(argmax_static_scratch));
+    if (status != hipSuccess) return (int)status;
+    if (found == nullptr) return VELOX_NO_ALLOC_NO_SCRATCH;
+    argmax_scratch_of_device[device] = found;
+  }
+  *address = argmax_scratch_of_device[device];
+  return 0;
+}
+
+extern "C" int velox_argmax_static_init(void) {
+  void* address = nullptr;
+  return argmax_scratch_of_current_device(&address);
+}
+
+extern "C" int velox_argmax_static(const float* logits, int* out, int rows, int vocab, int chunks, hipStream_t stream) {
+  if (rows < 0 || vocab < 1 || chunks < 1 || chunks > vocab || logits == nullptr || out == nullptr) return VELOX_NO_ALLOC_BAD_ARGUMENT;
+  if (rows == 0) return 0;
+  if (rows > 65535 || chunks > 65535 || (long long)rows * chunks > VELOX_ARGMAX_STATIC_MAX_PAIRS) return VELOX_NO_ALLOC_TOO_LARGE;
+  void* scratch = nullptr;
+  const int found = argmax_scratch_of_current_device(&scratch);
+  if (found != 0) return found;
+  const int chunk = (vocab + chunks - 1) / chunks;
+  // every pair that the merge reads is written by this launch first: what an earlier call left is never read
+  argmax_kernel<<<dim3(rows, chunks), SAMPLE_THREADS, 0, stream>>>(logits, out, (Best*)scratch, vocab, chunk);
+  if (chunks > 1) argmax_merge_kernel<<<rows, 64, 0, stream>>>((const Best*)scratch, out, chunks);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" const char* velox_no_alloc_error_text(int code) {
+  switch (code) {
+    case 0: return "success";
+    case VELOX_NO_ALLOC_BAD_ARGUMENT: return "bad argument: rows >= 0, vocab >= 1, 1 <= chunks <= vocab and non-null pointers are required";
+    case VELOX_NO_ALLOC_TOO_LARGE: return "rows * chunks exceeds VELOX_ARGMAX_STATIC_MAX_PAIRS (65536), the size of the static scratch array";
+    case VELOX_NO_ALLOC_NO_SCRATCH: return "the static scratch array of this GPU could not be found";
+    default: return hipGetErrorString((hipError_t)code);
+  }
 }
 
 // Philox 4x32 with 10 rounds.

@@ -25,7 +25,7 @@ ARCH = "gfx950"
 FLAGS = ["-O3", f"--offload-arch={ARCH}", "-shared", "-fPIC", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 CORE_SOURCES = ["elementwise.hip", "gemm.hip", "skinny_gemm.hip", "sampling.hip", "probe.hip"]
 ATTENTION_SOURCES = ["attention.hip"]
-HEADERS = ["common.h"]
+HEADERS = ["common.h", "no_alloc.h"]
 # head sizes built ahead of time by build_all(); any other multiple of 16 up to 256 is built at first use
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 96, 128, 256)
 
