@@ -50,3 +50,24 @@ def test_mixed_batch_with_page_reuse(tmp_path):
         torch.testing.assert_close(torch.cat(got[rid]), expected[rid], rtol=1e-4, atol=1e-5)
     h.cache.assert_consistent([])
     assert h.cache.num_used_pages() == 0
+
+
+def test_a_fixed_workspace_refuses_to_replace_a_buffer():
+    import pytest
+    import torch
+
+    from velox_amd.engine.batch import Workspace, WorkspaceError
+
+    workspace = Workspace(torch.device("cpu"))
+    first = workspace.get("a", 10)
+    assert workspace.get("a", 4).data_ptr() == first.data_ptr()
+    grown = workspace.get("a", 100)  # not fixed: grows on demand
+    assert grown.numel() == 100
+    workspace.reserve("b", 50)
+    workspace.fix()
+    assert workspace.get("a", 100).data_ptr() == grown.data_ptr()
+    assert workspace.get("b", 50).numel() == 50
+    with pytest.raises(WorkspaceError, match="'a'"):
+        workspace.get("a", 101)
+    with pytest.raises(WorkspaceError, match="nothing"):
+        workspace.get("c", 1)

@@ -31,3 +31,36 @@ def test_whole_then_decode_matches_plain(tmp_path, ops, name, dtype):
         got.append(h.feed([("a", [tokens[i]], [0])]))
     got = torch.cat(got)
     torch.testing.assert_close(got, expected, **TOL[dtype])
+
+
+def test_workspace_addresses_never_change_once_the_runner_exists(tmp_path, ops):
+    """Captured steps hold the addresses of the attention's partial buffers: they are sized once, for the largest step the
+    limits allow, and capture, a warm-up portion, a mixed step and a portion whose keys are split all find them in place."""
+    from velox_amd.weights import write_random_model
+
+    config = dict(CONFIGS["A"], max_position_embeddings=8192)
+    folder = write_random_model(config, str(tmp_path / "long"), seed=3, dtype="bfloat16")
+    h = Harness(folder, ops, torch.bfloat16, "cuda", page_size=16, num_pages=600, max_num_seqs=8, max_num_tokens=512, enable_graphs=True)
+    before = h.runner.workspace.addresses()
+    assert before and h.runner.workspace.fixed
+    h.runner.capture_decode_graphs()
+    h.runner.warm_prefill(512)
+    tokens = random_tokens(config["vocab_size"], 4400, seed=1)
+    for lo in range(0, 4096, 512):
+        h.feed([("long", tokens[lo:lo + 512], [])])
+    h.feed([("short", tokens[:40], [39])])
+    calls = []
+    original = ops.choose_portion_splits
+    ops.choose_portion_splits = lambda *args: calls.append(original(*args)) or calls[-1]
+    try:
+        h.feed([("short", [5], [0]), ("long", tokens[4096:4200], [103])])  # a decoded token beside a portion behind 4,096 keys
+    finally:
+        ops.choose_portion_splits = original
+    assert max(calls) > 1  # the portion's keys were split: the partial buffers were used
+    for _ in range(3):
+        h.feed([("short", [7], [0]), ("long", [9], [0])])  # captured steps
+    assert h.runner.num_graph_replays == 3
+    torch.cuda.synchronize()
+    assert h.runner.workspace.addresses() == before
+    with pytest.raises(RuntimeError, match="cannot be replaced"):
+        h.runner.workspace.get("attention_partial_out", 1 << 30)

@@ -93,9 +93,87 @@ def test_dtypes_kept(tmp_path):
     assert torch.equal(bf.final_norm.weight, raw["model.norm.weight"].float())
     wide = _load(folder, torch.float32)
     assert wide.embedding.table.dtype == torch.float32 and torch.equal(wide.embedding.table, raw["model.embed_tokens.weight"].float())
-    # stored float32 stays float32 even in a bfloat16 run
+    # stored float32 takes the run dtype too (reference src/weight_loader.py:127): rounded once, to nearest even, so the
+    # tensors are those of a folder that stores the same values in bfloat16
     folder32 = make_folder(tmp_path, "B", "float32")
-    kept = _load(folder32, torch.bfloat16)
-    assert kept.blocks[0].mixer.qkv_weight.dtype == torch.float32
+    raw32 = load_file(os.path.join(folder32, "model.safetensors"))
+    narrowed = _load(folder32, torch.bfloat16)
+    assert narrowed.blocks[0].mixer.qkv_weight.dtype == torch.bfloat16 and narrowed.embedding.table.dtype == torch.bfloat16
+    assert narrowed.head.weight.dtype == torch.bfloat16 and narrowed.blocks[2].feed_forward.down_weight.dtype == torch.bfloat16
+    assert torch.equal(narrowed.blocks[0].mixer.qkv_weight, bf.blocks[0].mixer.qkv_weight)
+    assert torch.equal(narrowed.head.weight, raw32["lm_head.weight"].to(torch.bfloat16))
+    assert narrowed.final_norm.weight.dtype == torch.float32 and torch.equal(narrowed.final_norm.weight, raw32["model.norm.weight"])
+    assert held_dtype("matrix", torch.float32, torch.bfloat16) == torch.bfloat16
     assert held_dtype("matrix", torch.int64, torch.bfloat16) == torch.int32
     assert held_dtype("matrix", torch.float16, torch.bfloat16) == torch.bfloat16
+    # a part may ask for a tensor as stored: 32-bit stays 32-bit
+    assert held_dtype("stored", torch.float32, torch.bfloat16) == torch.float32
+    assert held_dtype("stored", torch.bfloat16, torch.float32) == torch.float32
+    assert held_dtype("stored", torch.bfloat16, torch.bfloat16) == torch.bfloat16
+
+
+def test_a_bfloat16_run_on_a_float32_folder_gives_the_logits_of_the_bfloat16_folder(tmp_path):
+    from helpers import PAGE_SIZE, Harness, random_tokens
+    from torch_ops import TorchOps
+
+    tokens = random_tokens(TINY_B["vocab_size"], 20, seed=3)
+    logits = []
+    for storage in ("float32", "bfloat16"):
+        folder = make_folder(tmp_path, "B", storage)
+        if storage == "float32":
+            # vectors (biases, norm weights) are held in float32 as stored: give them the values the other folder holds,
+            # so that the matrices' conversion is the only difference left
+            path = os.path.join(folder, "model.safetensors")
+            raw = load_file(path)
+            save_file({name: t.to(torch.bfloat16).float() if t.dim() == 1 else t for name, t in raw.items()}, path)
+        h = Harness(folder, TorchOps(), torch.bfloat16, "cpu", PAGE_SIZE["B"], num_pages=16)
+        assert h.model.blocks[1].feed_forward.gate_up_weight.dtype == torch.bfloat16
+        logits.append(h.feed([("a", tokens, list(range(len(tokens))))]))
+    assert torch.equal(logits[0], logits[1])
+
+
+def _shard(folder, pieces=2, drop=None):
+    """Splits the folder's model.safetensors into ``pieces`` shards with an index file (the layout of every larger
+    checkpoint, reference ``src/weight_loader.py:31-55``); ``drop`` names a tensor left out of its shard."""
+    path = os.path.join(folder, "model.safetensors")
+    raw = load_file(path)
+    os.unlink(path)
+    names = sorted(raw)
+    weight_map = {}
+    for index in range(pieces):
+        shard = f"model-{index + 1:05d}-of-{pieces:05d}.safetensors"
+        mine = names[index::pieces]  # interleaved: the q, k and v rows of one fused tensor come from different files
+        save_file({name: raw[name] for name in mine if name != drop}, os.path.join(folder, shard))
+        weight_map.update({name: shard for name in mine})
+    with open(os.path.join(folder, "model.safetensors.index.json"), "w", encoding="utf-8") as handle:
+        json.dump({"metadata": {"total_size": sum(t.numel() * t.element_size() for t in raw.values())}, "weight_map": weight_map}, handle)
+    return raw
+
+
+def test_sharded_checkpoint_with_an_index_file(tmp_path):
+    folder = make_folder(tmp_path, "B")
+    whole = _load(folder)
+    raw = _shard(folder, pieces=3)
+    assert not os.path.exists(os.path.join(folder, "model.safetensors"))
+    sharded = _load(folder)
+    for a, b in zip(whole.all_parts(), sharded.all_parts()):
+        for attr in a.params():
+            assert torch.equal(getattr(a, attr), getattr(b, attr)), (a.prefix, attr)
+    p = "model.layers.2.self_attn."
+    assert torch.equal(sharded.blocks[2].mixer.qkv_weight, torch.cat([raw[p + "q_proj.weight"], raw[p + "k_proj.weight"], raw[p + "v_proj.weight"]]))
+
+
+def test_sharded_checkpoint_with_a_tensor_missing_from_its_shard(tmp_path):
+    folder = make_folder(tmp_path, "A")
+    _shard(folder, pieces=2, drop="model.layers.1.mlp.up_proj.weight")
+    with pytest.raises(WeightsError) as err:
+        _load(folder)
+    assert err.value.missing == ["model.layers.1.mlp.up_proj.weight"] and not err.value.unexpected and not err.value.wrong_shape
+
+
+def test_index_file_that_names_a_shard_that_is_not_there(tmp_path):
+    folder = make_folder(tmp_path, "A")
+    _shard(folder, pieces=2)
+    os.unlink(os.path.join(folder, "model-00002-of-00002.safetensors"))
+    with pytest.raises(FileNotFoundError, match="model-00002-of-00002.safetensors"):
+        _load(folder)

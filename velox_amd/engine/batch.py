@@ -38,19 +38,53 @@ class GroupBatch:
     max_kv_len_of_portions: int = 0  # the same over the sequences behind the leading one-token sequences (0: there are none)
 
 
+class WorkspaceError(RuntimeError):
+    pass
+
+
 class Workspace:
-    """Scratch tensors by name, kept across steps so their addresses are stable."""
+    """Scratch tensors by name, kept across steps so their addresses are stable.
+
+    A captured step holds the addresses of the buffers it was captured with, so a buffer must never be replaced once a
+    capture may exist.  The runner therefore asks every part what it can need at most (``Part.workspace_needs``),
+    reserves that before anything runs and calls :meth:`fix`; from then on a request for more than is there is an
+    error, not a new allocation.  A workspace that was never fixed (a test's own) grows on demand.
+    """
 
     def __init__(self, device) -> None:
         self.device = device
         self._buffers: Dict[str, torch.Tensor] = {}
+        self.fixed = False
+
+    def reserve(self, name: str, numel: int, dtype: torch.dtype = torch.float32) -> None:
+        """Makes sure ``name`` holds at least ``numel`` elements."""
+        buf = self._buffers.get(name)
+        if buf is not None and buf.dtype == dtype and buf.numel() >= numel:
+            return
+        if self.fixed:
+            have = "nothing" if buf is None else f"{buf.numel()} x {buf.dtype}"
+            raise WorkspaceError(f"workspace buffer {name!r} holds {have} but {numel} x {dtype} are asked for; captured steps hold its "
+                                 "address, so it cannot be replaced (the part that uses it must state this size in workspace_needs)")
+        self._buffers[name] = torch.empty(max(int(numel), 1), dtype=dtype, device=self.device)
+
+    def fix(self) -> None:
+        self.fixed = True
 
     def get(self, name: str, numel: int, dtype: torch.dtype = torch.float32) -> torch.Tensor:
-        buf = self._buffers.get(name)
-        if buf is None or buf.numel() < numel or buf.dtype != dtype:
-            buf = torch.empty(max(numel, 1), dtype=dtype, device=self.device)
-            self._buffers[name] = buf
-        return buf[:numel]
+        self.reserve(name, numel, dtype)
+        return self._buffers[name][:numel]
+
+    def addresses(self) -> Dict[str, int]:
+        return {name: buf.data_ptr() for name, buf in self._buffers.items()}
+
+
+@dataclass(frozen=True)
+class StepLimits:
+    """The most a step can hold: what parts size their scratch for."""
+
+    max_num_tokens: int
+    max_num_seqs: int
+    max_model_len: int
 
 
 @dataclass

@@ -165,7 +165,7 @@ class Engine:
         for part in self.model.all_parts():
             for attr, param in part.params().items():
                 tensor = getattr(part, attr, None)
-                if param.role == "matrix" and tensor is not None and tensor.dim() == 2 and tensor.dtype == torch.bfloat16 and attr != "table":
+                if param.role == "matrix" and param.product and tensor is not None and tensor.dim() == 2 and tensor.dtype == torch.bfloat16:
                     shapes.add(tuple(tensor.shape))
         done = 0
         recapture = False

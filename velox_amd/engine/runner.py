@@ -22,7 +22,7 @@ import torch
 
 from ..cache.manager import CacheManager
 from ..parts.model import DecoderModel
-from .batch import BatchBuilder, StepContext, StepEntry, Workspace
+from .batch import BatchBuilder, StepContext, StepEntry, StepLimits, Workspace
 
 
 def decode_buckets(max_num_seqs: int) -> List[int]:
@@ -62,7 +62,13 @@ class ModelRunner:
         self.max_num_tokens = max(int(max_num_tokens), int(max_num_seqs))
         self.max_num_seqs = int(max_num_seqs)
         self.builder = BatchBuilder(cache, self.device, self.max_num_tokens, self.max_num_seqs)
+        # every part's scratch at its largest, before anything runs: captured steps hold these addresses
         self.workspace = Workspace(self.device)
+        limits = StepLimits(self.max_num_tokens, self.max_num_seqs, cache.max_model_len)
+        for part in model.all_parts():
+            for name, numel in part.workspace_needs(ops, limits).items():
+                self.workspace.reserve(name, numel)
+        self.workspace.fix()
         self.enable_graphs = bool(enable_graphs) and self.device.type == "cuda"
         self._graphs: Dict[int, Tuple[object, torch.Tensor, torch.Tensor]] = {}
         self._short_graphs: Dict[int, Tuple[object, torch.Tensor, torch.Tensor]] = {}  # the same buckets behind few keys

@@ -655,6 +655,19 @@ class HipOps:
             return 1
         return max(1, min(-(-self.num_cus // blocks), max_kv_len // 1024, 16))
 
+    def attention_scratch_elems(self, num_heads: int, num_kv_heads: int, head_dim: int, max_num_tokens: int, max_num_seqs: int, max_model_len: int) -> Tuple[int, int]:
+        """The most float32 elements ``paged_attention`` asks its workspace for (partial outputs, partial log-sums) in
+        any step of at most ``max_num_tokens`` tokens and ``max_num_seqs`` sequences behind at most ``max_model_len`` keys,
+        with the splits that ``choose_splits`` and ``choose_portion_splits`` pick."""
+        group = num_heads // num_kv_heads
+        rows = 0  # splits x the rows the partial results are counted by
+        for count in range(1, max_num_seqs + 1):  # single tokens, alone or before portions
+            rows = max(rows, count * self.choose_splits(count, num_kv_heads, 1, max_model_len, True))
+        for portion in range(1, max_num_tokens + 1):  # portions of prompts, behind up to max_num_seqs - 1 single tokens
+            whole = min(max_num_tokens, portion + max_num_seqs - 1)
+            rows = max(rows, whole * self.choose_portion_splits(portion, group, num_kv_heads, max_model_len))
+        return rows * num_heads * head_dim, rows * num_heads
+
     def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens,
                         max_q_len, max_kv_len, scale, window, all_decode, workspace, splits: Optional[int] = None, decode_prefix: int = 0,
                         portions_max_kv_len: Optional[int] = None):
@@ -708,8 +721,9 @@ class HipOps:
             if splits > 1:
                 if workspace is None:
                     raise KernelError("split attention needs a workspace")
-                part_o = workspace.get("attention_partial_out", splits * tokens * num_heads * head_dim)
-                part_lse = workspace.get("attention_partial_lse", splits * tokens * num_heads)
+                span = num_tokens if decode_only else tokens  # the rows the kernels count partial results by
+                part_o = workspace.get("attention_partial_out", splits * span * num_heads * head_dim)
+                part_lse = workspace.get("attention_partial_lse", splits * span * num_heads)
             rows_in, rows_out = (qkv[first_token:first_token + num_tokens], out[first_token:first_token + num_tokens]) if decode_only else (qkv, out)
             status = lib.velox_paged_attention(
                 _ptr(rows_in), width, _ptr(k_cache), _ptr(v_cache), _ptr(block_tables[first_seq:]), block_tables.shape[1],

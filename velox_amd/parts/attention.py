@@ -81,6 +81,13 @@ class AttentionMixer(Mixer):
         ops.register_weight(self.qkv_weight, rotary_heads=(self.num_heads, self.num_kv_heads, self.head_dim) if whole_heads else None)
         ops.register_weight(self.o_weight)
 
+    def workspace_needs(self, ops, limits):
+        sizes = getattr(ops, "attention_scratch_elems", None)
+        if sizes is None:
+            return {}
+        partial_out, partial_lse = sizes(self.num_heads, self.num_kv_heads, self.head_dim, limits.max_num_tokens, limits.max_num_seqs, limits.max_model_len)
+        return {"attention_partial_out": partial_out, "attention_partial_lse": partial_lse}
+
     accepts_sink = True  # its last product may add itself to the residual (ResidualSink)
     accepts_deferred = True  # its first product can read a DeferredNorm
 

@@ -37,9 +37,11 @@ class Param:
     ``sources`` are checkpoint tensor names relative to the part's prefix; more
     than one means "concatenate along dim 0" (the reference fuses q/k/v and
     gate/up the same way, ``src/weight_loader.py:91-98``).  ``role`` decides the
-    dtype it is held in: a ``matrix`` follows the run's dtype (a checkpoint tensor
-    stored in 32-bit stays 32-bit), a ``vector`` (norm weights, biases) is always
-    held in float32.  ``init`` names the random-weights law: ``normal`` is
+    dtype it is held in: a ``matrix`` takes the run's dtype whatever the checkpoint
+    stores, a ``vector`` (norm weights, biases) is always held in float32, a
+    ``stored`` tensor stays in 32-bit when the checkpoint holds it so (a router's
+    weights, say) and takes the run dtype otherwise.  ``product`` = False marks a
+    matrix that no matrix product reads (a table that is only looked up).  ``init`` names the random-weights law: ``normal`` is
     N(0, 0.02), ``one_plus_normal`` is 1 + N(0, 0.02).
     """
 
@@ -49,10 +51,11 @@ class Param:
     role: str = "matrix"
     init: str = "normal"
     alias_of: Optional[str] = None  # absolute checkpoint name this falls back to (tied head)
+    product: bool = True
 
 
-def single(name: str, shape: Tuple[int, ...], role: str = "matrix", init: str = "normal") -> Param:
-    return Param(shape=tuple(shape), sources=(name,), source_shapes=(tuple(shape),), role=role, init=init)
+def single(name: str, shape: Tuple[int, ...], role: str = "matrix", init: str = "normal", product: bool = True) -> Param:
+    return Param(shape=tuple(shape), sources=(name,), source_shapes=(tuple(shape),), role=role, init=init, product=product)
 
 
 def fused_rows(names: Tuple[str, ...], shapes: Tuple[Tuple[int, ...], ...], role: str = "matrix") -> Param:
@@ -79,6 +82,12 @@ class Part:
     def prepare_kernels(self, ops) -> None:
         """Called once with the kernels' handle: a part may register the weights its decode-sized products read
         (``ops.register_weight``).  Nothing has to be done here."""
+
+    def workspace_needs(self, ops, limits) -> Dict[str, int]:
+        """Scratch this part may ask ``ctx.workspace`` for: buffer name -> the most float32 elements, for any step within
+        ``limits`` (``max_num_tokens``, ``max_num_seqs``, ``max_model_len``).  The step function reserves these before it
+        runs or captures anything and refuses to grow them later, because captured steps hold their addresses."""
+        return {}
 
 
 # ----------------------------------------------------------------------------------------

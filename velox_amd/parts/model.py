@@ -82,7 +82,7 @@ class Embedding(Part):
         self.table: Optional[torch.Tensor] = None
 
     def params(self) -> Dict[str, Param]:
-        return {"table": single(self.name, (self.vocab_size, self.hidden_size))}
+        return {"table": single(self.name, (self.vocab_size, self.hidden_size), product=False)}
 
     def forward(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
         return ctx.ops.embed(token_ids, self.table)

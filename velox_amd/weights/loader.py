@@ -8,9 +8,12 @@ shapes ``:123-126``.  Differences: tensors are read one at a time straight into 
 memory (no whole-checkpoint copy on the host), and every problem (missing tensors,
 unexpected tensors, wrong shapes) is collected and raised as ONE ``WeightsError``.
 
-Dtypes: a ``matrix`` stored in bfloat16 stays bfloat16 in a bfloat16 run and is widened
-(exactly) in a float32 run; a tensor stored in 32-bit stays 32-bit; ``vector`` tensors
-(norm weights, biases) are always held in float32; integer tensors become int32.
+Dtypes: a ``matrix`` is held in the run dtype whatever the checkpoint stores (bfloat16 is
+widened exactly in a float32 run; float32 is rounded once, to nearest even, in a bfloat16
+run, as the reference's ``param.copy_(src.to(device, dtype))`` does, ``src/weight_loader.py:127``);
+``vector`` tensors (norm weights, biases) are always held in float32; a part that needs a
+tensor exactly as stored declares it with role ``stored`` (32-bit stays 32-bit); integer
+tensors become int32.
 """
 from __future__ import annotations
 
@@ -83,12 +86,15 @@ class _Checkpoint:
 
 
 def held_dtype(role: str, stored: torch.dtype, run_dtype: torch.dtype) -> torch.dtype:
-    """The dtype a tensor is kept in, from its role, its stored dtype and the run dtype."""
+    """The dtype a tensor is kept in, from its role, its stored dtype and the run dtype.  A ``matrix`` takes the run
+    dtype whatever it is stored in (reference ``src/weight_loader.py:127`` converts while it copies); a ``vector`` is
+    float32; a ``stored`` tensor that the checkpoint holds in 32-bit (or wider) stays float32 and otherwise takes the
+    run dtype; integers become int32."""
     if not stored.is_floating_point:
         return torch.int32
     if role == "vector":
         return torch.float32
-    if stored == torch.float32 or stored == torch.float64:
+    if role == "stored" and stored in (torch.float32, torch.float64):
         return torch.float32
     return run_dtype
 
