@@ -1,8 +1,9 @@
 """A plain, slow Qwen2.5 forward written from the reference's formulas.
 
 Whole sequences, no cache, no batching, one function per part, float32 (or float64) on
-the CPU, sharing no code with ``velox_amd``.  Every function cites the reference lines
-(under ``/root/reference``) it was written from.  The reference was read, not run.
+the CPU, sharing no code with ``velox_amd``.  Every function cites the lines of the
+reference's files (paths from the reference's root) it was written from.  The reference
+was read, not run.
 """
 from __future__ import annotations
 

@@ -50,13 +50,16 @@ def changing_portions(requests, sizes=(7, 2, 5, 3, 11, 2, 16, 1, 2, 9)) -> List[
     return steps
 
 
-def mixed(requests, seed: int, max_live: int = 4) -> List[dict]:
+def mixed(requests, seed: int, max_live: int = 4, preempt: Tuple[str, ...] = ()) -> List[dict]:
     """Up to ``max_live`` requests at a time; every step gives each live request (sometimes leaving one out) a
     portion of 1..16 tokens, so portions of some sit beside single tokens of others; a request that is done
-    ends and the next one starts in its pages."""
+    ends and the next one starts in its pages.  A request named in ``preempt`` is ended once when it is about half
+    way (what it holds goes back), waits while the others go on in its pages, and is then fed again from its first
+    token under the same id: what a scheduler does to a preempted request (reference ``engine/scheduler.py:136-146``)."""
     rng = random.Random(seed)
     waiting = list(requests)
     live: Dict[str, int] = {}
+    to_preempt = set(preempt)
     steps = []
     while waiting or live:
         while waiting and len(live) < max_live:
@@ -72,11 +75,16 @@ def mixed(requests, seed: int, max_live: int = 4) -> List[dict]:
             live[rid] = at + n
             if at + n == len(requests[rid]):
                 end.append(rid)
+            elif rid in to_preempt and 2 * (at + n) >= len(requests[rid]):
+                to_preempt.discard(rid)
+                end.append(rid)
+                waiting.insert(min(1, len(waiting)), rid)  # behind the next newcomer, which takes over its pages first
         if not entries:
             continue
         for rid in end:
             del live[rid]
         steps.append({"step": len(steps), "entries": entries, "end": end})
+    assert not to_preempt, "a request to preempt never got half way"
     return steps
 
 
@@ -95,23 +103,41 @@ def tokens_needed(trace: List[dict], round_to: int) -> int:
 
 def collect(trace: List[dict], outputs: Dict[int, np.ndarray], requests) -> Dict[str, torch.Tensor]:
     """Puts the logits of every step back in order per request: {id: [len, vocab]}."""
-    rows: Dict[str, List[Tuple[int, np.ndarray]]] = {rid: [] for rid in requests}
+    rows: Dict[str, Dict[int, np.ndarray]] = {rid: {} for rid in requests}
     at: Dict[str, int] = {rid: 0 for rid in requests}
     for record in trace:
         out = outputs.get(record["step"])
         row = 0
         for entry in record["entries"]:
             for w in entry["want"]:
-                rows[entry["id"]].append((at[entry["id"]] + w, out[row]))
+                rows[entry["id"]][at[entry["id"]] + w] = out[row]  # (a request that starts over overwrites its first run)
                 row += 1
             at[entry["id"]] += len(entry["tokens"])
         assert out is None or row == out.shape[0]
+        for rid in record["end"]:
+            at[rid] = 0  # ended: if it comes again it starts from its first token
     result = {}
-    for rid, items in rows.items():
-        items.sort(key=lambda item: item[0])
-        assert [p for p, _ in items] == list(range(len(requests[rid]))), f"{rid}: positions {[p for p, _ in items][:5]}..."
-        result[rid] = torch.from_numpy(np.stack([r for _, r in items]))
+    for rid, found in rows.items():
+        assert sorted(found) == list(range(len(requests[rid]))), f"{rid}: positions {sorted(found)[:5]}..."
+        result[rid] = torch.from_numpy(np.stack([found[p] for p in range(len(requests[rid]))]))
     return result
+
+
+def first_runs(trace: List[dict], outputs: Dict[int, np.ndarray], requests) -> Dict[str, Dict[int, np.ndarray]]:
+    """For requests that a trace ends half way and feeds again: the logits of the first run, {id: {position: row}}."""
+    rows: Dict[str, Dict[int, np.ndarray]] = {}
+    at: Dict[str, int] = {rid: 0 for rid in requests}
+    for record in trace:
+        out = outputs.get(record["step"])
+        row = 0
+        for entry in record["entries"]:
+            for w in entry["want"]:
+                rows.setdefault(entry["id"], {}).setdefault(at[entry["id"]] + w, out[row])
+                row += 1
+            at[entry["id"]] += len(entry["tokens"])
+        for rid in record["end"]:
+            at[rid] = 0
+    return rows
 
 
 def run_trace(replayer, trace: List[dict]) -> Dict[int, np.ndarray]:

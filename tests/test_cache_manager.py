@@ -4,33 +4,33 @@ import random
 import pytest
 import torch
 
-from velox_amd.cache import NULL_PAGE, CacheManager, OutOfPagesError, PageAllocator
+from velox_amd.cache import NULL_PAGE, CacheManager, PoolExhausted, PageAllocator
 from velox_amd.parts.base import PagedNeed, StateNeed
 
 
 def test_allocator_order_and_errors():
     a = PageAllocator(6)
-    assert [a.allocate() for _ in range(3)] == [1, 2, 3]  # page 0 is never handed out
-    a.free(2)
-    assert a.allocate() == 2  # the page freed last is used again first
-    assert a.allocate_many(2) == [4, 5]
-    with pytest.raises(OutOfPagesError):
-        a.allocate()
-    with pytest.raises(OutOfPagesError):
-        a.allocate_many(1)
-    a.free(4)
+    assert [a.take() for _ in range(3)] == [1, 2, 3]  # page 0 is never handed out
+    a.drop(2)
+    assert a.take() == 2  # the page freed last is used again first
+    assert a.take_many(2) == [4, 5]
+    with pytest.raises(PoolExhausted):
+        a.take()
+    with pytest.raises(PoolExhausted):
+        a.take_many(1)
+    a.drop(4)
     with pytest.raises(RuntimeError):
-        a.free(4)  # freed twice
+        a.drop(4)  # freed twice
     with pytest.raises(RuntimeError):
-        a.incref(4)  # free page
-    a.incref(1)
-    assert a.free(1) == 1 and a.num_free == 1
-    assert a.free(NULL_PAGE) == 1  # the reserved page stays
+        a.share(4)  # free page
+    a.share(1)
+    assert a.drop(1) == 1 and a.num_free == 1
+    assert a.drop(NULL_PAGE) == 1  # the reserved page stays
     with pytest.raises(IndexError):
-        a.free(6)
+        a.drop(6)
     with pytest.raises(ValueError):
         PageAllocator(1)
-    a.assert_consistent()
+    a.verify()
 
 
 @pytest.mark.parametrize("num_pages", [2, 3, 4, 5, 17, 64, 1000, 7201])
@@ -39,20 +39,20 @@ def test_scattered_first_hand_outs(num_pages):
     first, the order is the same every time, and pages handed out 256 hand-outs apart (the same place of two sequences
     filled one after the other) lie at no regular distance."""
     a = PageAllocator(num_pages, scatter=True)
-    order = a.allocate_many(num_pages - 1)
+    order = a.take_many(num_pages - 1)
     assert sorted(order) == list(range(1, num_pages))
-    with pytest.raises(OutOfPagesError):
-        a.allocate()
+    with pytest.raises(PoolExhausted):
+        a.take()
     if num_pages > 2:
-        a.free(order[0])
-        a.free(order[-1])
-        assert a.allocate() == order[-1] and a.allocate() == order[0]
-    a.assert_consistent()
-    assert PageAllocator(num_pages, scatter=True).allocate_many(num_pages - 1) == order
+        a.drop(order[0])
+        a.drop(order[-1])
+        assert a.take() == order[-1] and a.take() == order[0]
+    a.verify()
+    assert PageAllocator(num_pages, scatter=True).take_many(num_pages - 1) == order
     if num_pages >= 1000:
         far = {(order[i + 256] - order[i]) % (num_pages - 1) for i in range(len(order) - 256)}
         assert len(far) > (len(order) - 256) // 2
-    assert PageAllocator(num_pages).allocate_many(num_pages - 1) == list(range(1, num_pages))
+    assert PageAllocator(num_pages).take_many(num_pages - 1) == list(range(1, num_pages))
 
 
 def _manager(needs, pages=9, page=4, seqs=4, max_len=None):

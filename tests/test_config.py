@@ -4,7 +4,8 @@ import json
 import pytest
 
 from helpers import TINY_A, TINY_B, TINY_C
-from velox_amd.config import ConfigError, Qwen2Config, config_from_dict, known_architectures, load_config
+from velox_amd.config import ConfigError, config_from_dict, known_architectures, load_config
+from velox_amd.models.qwen2 import Qwen2Config
 from velox_amd.config.engine_config import EngineConfig, resolve_dtype
 from velox_amd.config.registry import get_architecture
 

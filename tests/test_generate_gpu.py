@@ -283,8 +283,29 @@ def test_sampling_through_the_engine(tmp_path):
     assert mixed[1].output_token_ids == greedy_alone.output_token_ids
     top1 = engine.generate([Request("k1", prompts[1], SamplingParams(temperature=1.5, top_k=1, max_tokens=6, ignore_eos=True))])[0]
     assert top1.output_token_ids == greedy_alone.output_token_ids
-    penalised = engine.generate([Request("pen", prompts[1], SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True, repetition_penalty=1.3, frequency_penalty=0.4))])[0]
-    assert len(penalised.output_token_ids) == 6
+    # penalties over prompt plus output: the tokens that the plain model's logits give under the reference's formula; a
+    # prompt that repeats few tokens makes the penalties decide (without them the tokens differ), beside a neighbour
+    # with another history and other coefficients
+    from torch_ops import TorchOps
+
+    config, weights = read_model_folder(folder)
+    histories = [[5, 9, 5, 9, 5, 9, 5, 9, 12, 5, 9], prompts[2]]
+    coefficients = [dict(repetition_penalty=1.6, frequency_penalty=0.05, presence_penalty=0.02), dict(repetition_penalty=1.2, presence_penalty=0.03)]
+
+    def plain_penalised(prompt, steps, repetition_penalty=1.0, presence_penalty=0.0, frequency_penalty=0.0):
+        tokens = list(prompt)
+        for _ in range(steps):
+            logits = qwen2_logits(config, weights, tokens)[-1:].clone()
+            TorchOps().apply_penalties(logits, torch.tensor([tokens]), torch.tensor([len(tokens)]),
+                                       torch.tensor([[repetition_penalty, presence_penalty, frequency_penalty]]))
+            tokens.append(int(logits[0].argmax()))
+        return tokens[len(prompt):]
+
+    penalised = engine.generate([Request(f"pen{i}", h, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True, **c))
+                                 for i, (h, c) in enumerate(zip(histories, coefficients))])
+    for request, history, c in zip(penalised, histories, coefficients):
+        assert request.output_token_ids == plain_penalised(history, 10, **c), request.request_id
+    assert penalised[0].output_token_ids != plain_penalised(histories[0], 10)  # the penalties changed what is chosen
 
 
 def test_command_line(tmp_path):

@@ -189,8 +189,8 @@ def test_qkv_projection_with_rotation_and_cache_write_in_one_kernel(ops, ref, m,
     slots = (torch.randperm((pages - 1) * page, generator=torch.Generator().manual_seed(74))[:m] + page).to(torch.int32).cuda()
     angles = torch.outer(torch.arange(512, dtype=torch.float32), 1.0 / (10000.0 ** (torch.arange(half, dtype=torch.float32) / half)))
     cos, sin = angles.cos().cuda(), angles.sin().cuda()
-    ops.register_weight(w, rotary_heads=(nh, nkv, d))
-    assert ops.packed_weight(w, "rotary") is not None
+    pw = ops.prepare_weight(w, rotary_heads=(nh, nkv, d))
+    assert pw.copy("rotary") is not None
     for use_bias in (bias, None):
         # float32 reference: exact product of the bfloat16 operands, then everything in float32
         k32 = torch.full((pages, nkv, page, d), 7.0, dtype=torch.float32, device="cuda")
@@ -202,7 +202,7 @@ def test_qkv_projection_with_rotation_and_cache_write_in_one_kernel(ops, ref, m,
             k_cache = torch.full((pages, nkv, page, d), 7.0, dtype=torch.bfloat16, device="cuda")
             v_cache = torch.full((pages, nkv, d, page), 7.0, dtype=torch.bfloat16, device="cuda")
             for waves in ((8, 16) if fused else (None,)):
-                q = ops.qkv_rope_write(x, w, use_bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, waves=waves, fused=fused)
+                q = ops.qkv_rope_write(x, pw, use_bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, waves=waves, fused=fused)
                 results[(fused, waves)] = (q[:, : nh * d].float(), k_cache.float(), v_cache.float())
         scale = float(wide.abs().max())
         for key, (q, kc, vc) in results.items():
@@ -215,9 +215,9 @@ def test_qkv_projection_with_rotation_and_cache_write_in_one_kernel(ops, ref, m,
         torch.testing.assert_close(results[(True, 8)][0], results[(False, None)][0], rtol=2e-2, atol=2e-2 * scale)
     # a layer that reads another layer's cache writes nothing: not a case for the fused kernel
     with pytest.raises(Exception):
-        ops.qkv_rope_write(x, w, bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, write_kv=False, fused=True)
+        ops.qkv_rope_write(x, pw, bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, write_kv=False, fused=True)
     before = k_cache.clone()
-    ops.qkv_rope_write(x, w, bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, write_kv=False)
+    ops.qkv_rope_write(x, pw, bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, write_kv=False)
     assert torch.equal(before, k_cache)
 
 
@@ -238,7 +238,7 @@ def test_qkv_projection_at_17_to_64_rows_with_partial_sums_added_by_the_rotation
     consecutive = torch.arange(m) + page + 3
     angles = torch.outer(torch.arange(512, dtype=torch.float32), 1.0 / (10000.0 ** (torch.arange(half, dtype=torch.float32) / half)))
     cos, sin = (angles.cos().cuda(), angles.sin().cuda()) if rotate else (None, None)
-    ops.register_weight(w, rotary_heads=(nh, nkv, d))
+    pw = ops.prepare_weight(w, rotary_heads=(nh, nkv, d))
     scale = float(ref.linear(x, w, None, torch.float32).abs().max())
     for slots in (scattered, consecutive):
         slots = slots.to(torch.int32).cuda()
@@ -250,7 +250,7 @@ def test_qkv_projection_at_17_to_64_rows_with_partial_sums_added_by_the_rotation
             k_cache = torch.full((pages, nkv, page, d), 7.0, dtype=torch.bfloat16, device="cuda")
             v_cache = torch.full((pages, nkv, d, page), 7.0, dtype=torch.bfloat16, device="cuda")
             for splits in (None, 1, 3):
-                partial = ops.skinny_gemm_splitk(x, w, splits=splits, packed=ops.packed_weight(w))
+                partial = ops.skinny_gemm_splitk(x, w, splits=splits, packed=pw.copy(1))
                 q = ops.rope_kv_write_partial(partial, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, bias=use_bias)
                 bound = dict(rtol=1e-2, atol=1e-2 * scale)
                 torch.testing.assert_close(q[:, : nh * d].float(), wide[:, : nh * d], **bound)
@@ -258,12 +258,12 @@ def test_qkv_projection_at_17_to_64_rows_with_partial_sums_added_by_the_rotation
                 torch.testing.assert_close(v_cache.float(), v32, **bound)
             # the route the engine takes for this many rows is this one
             k2, v2 = torch.full_like(k_cache, 7.0), torch.full_like(v_cache, 7.0)
-            q2 = ops.qkv_rope_write(x, w, use_bias, nh, nkv, d, positions, cos, sin, slots, k2, v2, page)
+            q2 = ops.qkv_rope_write(x, pw, use_bias, nh, nkv, d, positions, cos, sin, slots, k2, v2, page)
             torch.testing.assert_close(q2[:, : nh * d].float(), wide[:, : nh * d], rtol=1e-2, atol=1e-2 * scale)
             torch.testing.assert_close(k2.float(), k32, rtol=1e-2, atol=1e-2 * scale)
     # a layer that reads another layer's cache writes nothing
     before = k_cache.clone()
-    ops.qkv_rope_write(x, w, bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, write_kv=False)
+    ops.qkv_rope_write(x, pw, bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, write_kv=False)
     assert torch.equal(before, k_cache)
 
 
@@ -281,7 +281,7 @@ def test_residual_add_and_norm_split_between_two_products(ops, ref, m, hidden, i
     residual0 = rand((m, hidden), torch.float32, 82, 2.0)
     norm = RMSNorm("", hidden, 1e-5)
     norm.weight = (1.0 + rand((hidden,), torch.float32, 83, 0.1))
-    ops.register_weight(w_out)
+    p_out = ops.prepare_weight(w_out)
     if hidden % 64 != 0:
         # the next product cannot stream this width: it gets the materialised rows
         pass
@@ -290,7 +290,7 @@ def test_residual_add_and_norm_split_between_two_products(ops, ref, m, hidden, i
     want_residual = residual0 + delta
     want_normed = ref.add_rmsnorm(residual0.clone(), delta, norm.weight, norm.eps, torch.float32)
     residual = residual0.clone()
-    deferred = ops.linear(x, w_out, None, torch.bfloat16, partials_ok=True, residual_norm=ResidualSink(residual, norm))
+    deferred = ops.linear(x, p_out, None, torch.bfloat16, partials_ok=True, residual_norm=ResidualSink(residual, norm))
     assert isinstance(deferred, DeferredNorm) and deferred.norm is norm
     torch.testing.assert_close(residual, want_residual, rtol=1e-5, atol=1e-4 * float(want_residual.abs().max()))
     torch.testing.assert_close(ops.materialize(deferred).float(), want_normed, rtol=2e-2, atol=2e-2)
@@ -314,19 +314,19 @@ def test_residual_add_and_norm_split_between_two_products(ops, ref, m, hidden, i
     scale = float(ref.linear(normed_bf16, w_next, None, torch.float32).abs().max())
     tol = dict(rtol=2e-2, atol=2e-2 * scale)
     torch.testing.assert_close(ops.linear(deferred, w_next, bias, torch.float32), ref.linear(normed_bf16, w_next, bias, torch.float32), **tol)  # unregistered: materialised
-    ops.register_weight(w_next)
-    torch.testing.assert_close(ops.linear(deferred, w_next, bias, torch.float32), ref.linear(normed_bf16, w_next, bias, torch.float32), **tol)
+    p_next = ops.prepare_weight(w_next)
+    torch.testing.assert_close(ops.linear(deferred, p_next, bias, torch.float32), ref.linear(normed_bf16, w_next, bias, torch.float32), **tol)
     # 64 rows of the weight per wave (the variant for very tall weights), four and eight waves
     for waves in (4, 8):
         if hidden // 16 <= 64 * waves:
-            got = ops.skinny_gemm(deferred.x, w_next, bias, torch.float32, waves=waves, row_tiles=4, packed=ops.packed_weight(w_next), row_scale=deferred)
+            got = ops.skinny_gemm(deferred.x, w_next, bias, torch.float32, waves=waves, row_tiles=4, packed=p_next.copy(1), row_scale=deferred)
             torch.testing.assert_close(got, ref.linear(normed_bf16, w_next, bias, torch.float32), **tol)
-    ops.register_weight(w_next, stacked=2)
+    p_next = ops.prepare_weight(w_next, stacked=2, handle=p_next)
     want_glu = ref.linear_silu_mul(normed_bf16, w_next, torch.bfloat16).float()
-    torch.testing.assert_close(ops.linear_silu_mul(deferred, w_next, torch.bfloat16).float(), want_glu, rtol=3e-2, atol=3e-2 * float(want_glu.abs().max()))
+    torch.testing.assert_close(ops.linear_silu_mul(deferred, p_next, torch.bfloat16).float(), want_glu, rtol=3e-2, atol=3e-2 * float(want_glu.abs().max()))
     # q/k/v with rotation: 2 heads, 1 kv head, head size 80 -> 320 rows
     nh, nkv, d, page, pages = 2, 1, 80, 8, 12
-    ops.register_weight(w_next, rotary_heads=(nh, nkv, d))
+    p_next = ops.prepare_weight(w_next, rotary_heads=(nh, nkv, d), handle=p_next)
     positions = torch.randint(0, 300, (m,), generator=torch.Generator().manual_seed(86)).to(torch.int32).cuda()
     slots = (torch.randperm((pages - 1) * page, generator=torch.Generator().manual_seed(87))[:m] + page).to(torch.int32).cuda()
     angles = torch.outer(torch.arange(512, dtype=torch.float32), 1.0 / (10000.0 ** (torch.arange(d // 2, dtype=torch.float32) / (d // 2))))
@@ -335,7 +335,7 @@ def test_residual_add_and_norm_split_between_two_products(ops, ref, m, hidden, i
     for source in (deferred, normed_bf16):
         k_cache = torch.zeros((pages, nkv, page, d), dtype=torch.bfloat16, device="cuda")
         v_cache = torch.zeros((pages, nkv, d, page), dtype=torch.bfloat16, device="cuda")
-        q = ops.qkv_rope_write(source, w_next, bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page)
+        q = ops.qkv_rope_write(source, p_next, bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page)
         outs.append((q[:, : nh * d].float(), k_cache.float(), v_cache.float()))
     for got, want in zip(*outs):
         torch.testing.assert_close(got, want, rtol=3e-2, atol=3e-2 * max(1.0, float(want.abs().max())))
@@ -359,9 +359,9 @@ def test_decode_activations_handed_on_in_the_lanes_order(ops, ref, m, monkeypatc
     x = rand((m, hidden), torch.bfloat16, 90)
     w_gu = rand((2 * inner, hidden), torch.bfloat16, 91, 0.05)
     w_down = rand((hidden, inner), torch.bfloat16, 92, 0.05)
-    ops.register_weight(w_gu, stacked=2)
-    ops.register_weight(w_down)
-    act = ops.linear_silu_mul(x, w_gu, torch.bfloat16)
+    p_gu = ops.prepare_weight(w_gu, stacked=2)
+    p_down = ops.prepare_weight(w_down)
+    act = ops.linear_silu_mul(x, p_gu, torch.bfloat16)
     twin, version = act._velox_packed_rows
     assert version == act._version and torch.equal(_rows_from_lanes_order(twin, inner)[:m], act)
     norm = RMSNorm("", hidden, 1e-6)
@@ -371,7 +371,7 @@ def test_decode_activations_handed_on_in_the_lanes_order(ops, ref, m, monkeypatc
         source = act if use_twin else act.clone()  # (a clone is another tensor object: no copy hangs on it)
         assert (ops._packed_rows_of(source, inner) is not None) == use_twin
         residual = rand((m, hidden), torch.float32, 94)
-        deferred = ops.linear(source, w_down, None, torch.bfloat16, partials_ok=True, residual_norm=ResidualSink(residual, norm))
+        deferred = ops.linear(source, p_down, None, torch.bfloat16, partials_ok=True, residual_norm=ResidualSink(residual, norm))
         assert isinstance(deferred, DeferredNorm)
         next_twin = ops._packed_rows_of(deferred.x, hidden)
         assert torch.equal(_rows_from_lanes_order(next_twin, hidden)[:m], deferred.x)
@@ -382,10 +382,10 @@ def test_decode_activations_handed_on_in_the_lanes_order(ops, ref, m, monkeypatc
     deferred = results[0][3]
     plain = DeferredNorm(deferred.x.clone(), deferred.sums, deferred.width, deferred.eps, deferred.norm)
     bias = rand((2 * inner,), torch.float32, 95)
-    assert torch.equal(ops.linear(deferred, w_gu, bias, torch.float32), ops.linear(plain, w_gu, bias, torch.float32))
-    assert torch.equal(ops.linear_silu_mul(deferred, w_gu, torch.bfloat16), ops.linear_silu_mul(plain, w_gu, torch.bfloat16))
+    assert torch.equal(ops.linear(deferred, p_gu, bias, torch.float32), ops.linear(plain, p_gu, bias, torch.float32))
+    assert torch.equal(ops.linear_silu_mul(deferred, p_gu, torch.bfloat16), ops.linear_silu_mul(plain, p_gu, torch.bfloat16))
     nh, nkv, d, page, pages = 3, 2, 128, 16, 6  # (3 + 2 * 2) * 128 = 896 = 2 * inner rows
-    ops.register_weight(w_gu, rotary_heads=(nh, nkv, d))
+    p_gu = ops.prepare_weight(w_gu, rotary_heads=(nh, nkv, d), handle=p_gu)
     positions = torch.arange(m, dtype=torch.int32, device="cuda") * 7
     slots = (torch.randperm((pages - 1) * page, generator=torch.Generator().manual_seed(96))[:m] + page).to(torch.int32).cuda()
     angles = torch.outer(torch.arange(128, dtype=torch.float32), 1.0 / (10000.0 ** (torch.arange(d // 2, dtype=torch.float32) / (d // 2))))
@@ -394,7 +394,7 @@ def test_decode_activations_handed_on_in_the_lanes_order(ops, ref, m, monkeypatc
     for source in (deferred, plain):
         k_cache = torch.zeros((pages, nkv, page, d), dtype=torch.bfloat16, device="cuda")
         v_cache = torch.zeros((pages, nkv, d, page), dtype=torch.bfloat16, device="cuda")
-        q = ops.qkv_rope_write(source, w_gu, bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, fused=True)
+        q = ops.qkv_rope_write(source, p_gu, bias, nh, nkv, d, positions, cos, sin, slots, k_cache, v_cache, page, fused=True)
         outs.append((q, k_cache, v_cache))
     for a, b in zip(*outs):
         assert torch.equal(a, b)
@@ -704,27 +704,48 @@ def test_skinny_gemm(ops, ref, out_dtype, m, n, k):
         torch.testing.assert_close(ops.skinny_gemm(x, w, None, out_dtype)[:fewer], part, rtol=0, atol=0)
 
 
-def test_registered_weight_copies_die_with_their_weight(ops, ref):
-    """The lane-ordered copy belongs to one tensor object: another weight that later lands on the same address, or the
-    same weight after a change in place, must not be multiplied with the old copy."""
+def test_prepared_copies_belong_to_one_weight_and_one_version(ops, ref):
+    """What ``prepare_weight`` returns is held by the caller and stands in the weight's place; a plain tensor is multiplied
+    as it is (no copy is ever found through an address), and a weight changed in place behind its copies is an error, not a
+    product with stale values."""
+    from velox_amd.kernels.hip_ops import KernelError
+
     x = rand((4, 128), torch.bfloat16, 60)
     first = rand((96, 128), torch.bfloat16, 61, 0.05)
-    ops.register_weight(first)
-    assert ops.packed_weight(first) is not None
-    address = first.data_ptr()
-    del first
-    for seed in range(62, 70):
-        other = rand((96, 128), torch.bfloat16, seed, 0.05)
-        assert ops.packed_weight(other) is None
-        torch.testing.assert_close(ops.linear(x, other, None, torch.float32), ref.linear(x, other, None, torch.float32), rtol=1e-4, atol=1e-4)
-        if other.data_ptr() == address:
-            break
-    ops.register_weight(other)
-    other.mul_(2.0)
-    assert ops.packed_weight(other) is None
-    torch.testing.assert_close(ops.linear(x, other, None, torch.float32), ref.linear(x, other, None, torch.float32), rtol=1e-4, atol=1e-4)
-    ops.register_weight(other, stacked=2)
-    assert ops.packed_weight(other, 2) is not None and ops.packed_weight(other, 1) is None
+    prepared = ops.prepare_weight(first)
+    assert prepared.weight is first and prepared.copy(1) is not None and prepared.copy(2) is None
+    want = ref.linear(x, first, None, torch.float32)
+    torch.testing.assert_close(ops.linear(x, prepared, None, torch.float32), want, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(ops.linear(x, first, None, torch.float32), want, rtol=1e-4, atol=1e-4)
+    other = rand((96, 128), torch.bfloat16, 62, 0.05)
+    assert ops.prepare_weight(other, stacked=2, handle=prepared).weight is other  # another weight: a new handle, not an extended one
+    first.mul_(2.0)
+    with pytest.raises(KernelError, match="changed in place"):
+        ops.linear(x, prepared, None, torch.float32)
+    again = ops.prepare_weight(first, handle=prepared)
+    assert again is not prepared
+    torch.testing.assert_close(ops.linear(x, again, None, torch.float32), 2 * want, rtol=1e-4, atol=1e-4)
+    stacked = ops.prepare_weight(other, stacked=2)
+    assert stacked.copy(2) is not None and stacked.copy(1) is None
+    # what the kernels cannot read in their lanes' order stays as it is
+    assert ops.prepare_weight(rand((96, 100), torch.bfloat16, 63)) is None
+    assert ops.prepare_weight(rand((96, 128), torch.float32, 64)) is None
+
+
+def test_a_part_refuses_a_weight_bound_again_behind_prepared_copies(ops):
+    from velox_amd.parts import make_part
+
+    ff = make_part("feed_forward", "gated_mlp", prefix="m.", hidden_size=128, intermediate_size=192)
+    ff.gate_up_weight = rand((384, 128), torch.bfloat16, 65, 0.05)
+    ff.down_weight = rand((128, 192), torch.bfloat16, 66, 0.05)
+    assert ff.operand("down_weight") is ff.down_weight  # nothing prepared yet: the tensor itself
+    ff.prepare_kernels(ops)
+    assert ff.operand("down_weight").weight is ff.down_weight and ff.operand("gate_up_weight").copy(2) is not None
+    ff.down_weight = ff.down_weight.clone()
+    with pytest.raises(RuntimeError, match="bound again"):
+        ff.operand("down_weight")
+    ff.prepare_kernels(ops)
+    assert ff.operand("down_weight").weight is ff.down_weight
 
 
 @pytest.mark.parametrize("m,inter,k", [(1, 128, 64), (8, 18944, 3584), (16, 150, 128), (7, 1000, 192), (3, 16, 64)])
@@ -757,12 +778,12 @@ def test_gate_up_product_with_silu_epilogue_at_17_to_64_rows(ops, ref, m, inter,
     want = (torch.nn.functional.silu(gate_up[:, :inter]) * gate_up[:, inter:])
     scale = float(want.abs().max())
     unregistered = ops.linear_silu_mul(x, w, torch.bfloat16).float()  # (product + SiLU kernel)
-    ops.register_weight(w, stacked=2)
-    got = ops.linear_silu_mul(x, w, torch.bfloat16).float()
+    pw = ops.prepare_weight(w, stacked=2)
+    got = ops.linear_silu_mul(x, pw, torch.bfloat16).float()
     torch.testing.assert_close(got, want, rtol=1e-2, atol=1e-2 * scale)
     torch.testing.assert_close(got, unregistered, rtol=2e-2, atol=2e-2 * scale)
     # rows of a batch do not depend on one another: the first rows alone give the same bits
-    few = ops.linear_silu_mul(x[:17].contiguous(), w, torch.bfloat16).float()
+    few = ops.linear_silu_mul(x[:17].contiguous(), pw, torch.bfloat16).float()
     assert torch.equal(few, got[:17])
 
 

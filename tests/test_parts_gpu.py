@@ -9,8 +9,8 @@ import torch
 
 from plain_qwen2 import apply_rope, causal_attention, gated_mlp, rms_norm, rope_tables
 from velox_amd.cache import CacheManager
-from velox_amd.config.model_config import ModelConfig, architecture_name
-from velox_amd.config.registry import config_from_dict, get_architecture, register_architecture
+from velox_amd.config.model_config import ModelConfig
+from velox_amd.config.registry import architecture_name, config_from_dict, get_architecture, register_architecture
 from velox_amd.engine.batch import StepEntry
 from velox_amd.engine.engine import build_model
 from velox_amd.engine.runner import ModelRunner
@@ -136,8 +136,15 @@ def test_attention_part_alone(ops, nh, nkv, d, hidden, bias, window):
 # a toy architecture defined here: a mixer with per-request state, then an attention layer that runs twice,
 # the second time beside an entry that reads the first run's cache
 # ----------------------------------------------------------------------------------------------------
+# where the toy architectures keep their tensors in a checkpoint (an architecture chooses its own names)
+HF_NAMES = dict(mixer_prefix="self_attn.", feed_forward_prefix="mlp.", mixer_norm_prefix="input_layernorm.", ff_norm_prefix="post_attention_layernorm.")
+HF_ENDS = dict(embed_name="model.embed_tokens.weight", head_name="lm_head.weight", final_norm_prefix="model.norm.")
+
+
 class DecayingSumMixer(Mixer):
     """y_t = W s_t,  s_t = decay * s_{t-1} + x_t, with s kept per request in the cache manager's state slots."""
+
+    graph_safe = False  # forward reads the step's slots and lengths on the host
 
     def __init__(self, prefix: str, hidden_size: int, decay: float) -> None:
         super().__init__(prefix)
@@ -171,12 +178,12 @@ def toy_spec(config, max_position=None) -> ModelSpec:
     ff = PartSpec.of("gated_mlp", hidden_size=h, intermediate_size=raw["inter"])
     attention = PartSpec.of("attention", hidden_size=h, num_heads=4, num_kv_heads=2, head_dim=16, qkv_bias=False)
     layers = [
-        LayerSpec("layers.0.", PartSpec.of("toy_decaying_sum", hidden_size=h, decay=raw["decay"]), ff, norm, norm, mixer_prefix="mixer."),
-        LayerSpec("layers.1.", attention, ff, norm, norm, position="rope"),
+        LayerSpec("layers.0.", PartSpec.of("toy_decaying_sum", hidden_size=h, decay=raw["decay"]), ff, norm, norm, **dict(HF_NAMES, mixer_prefix="mixer.")),
+        LayerSpec("layers.1.", attention, ff, norm, norm, position="rope", **HF_NAMES),
     ]
     schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(1, cache_from=1)]
     return ModelSpec(vocab_size=raw["vocab_size"], hidden_size=h, max_position=256, layers=layers, schedule=schedule, final_norm=norm,
-                     positions={"rope": PartSpec.of("rotary", rotary_dim=16, theta=10000.0, max_position=256)}, tie_head=True)
+                     positions={"rope": PartSpec.of("rotary", rotary_dim=16, theta=10000.0, max_position=256)}, tie_head=True, **HF_ENDS)
 
 
 def plain_toy(tensors: Dict[str, torch.Tensor], raw, tokens):
@@ -275,8 +282,8 @@ class RoutedFeedForward(FeedForward):
 
     def prepare_kernels(self, ops) -> None:
         for e in range(self.num_experts):
-            ops.register_weight(getattr(self, f"gate_up_{e}"), stacked=2)
-            ops.register_weight(getattr(self, f"down_{e}"))
+            self.prepare_weight(ops, f"gate_up_{e}", stacked=2)
+            self.prepare_weight(ops, f"down_{e}")
 
     def forward(self, x, ctx):
         ops = ctx.ops
@@ -288,8 +295,8 @@ class RoutedFeedForward(FeedForward):
             rows = torch.nonzero(choice == e).flatten()
             if rows.numel() == 0:
                 continue
-            act = ops.linear_silu_mul(x[rows].contiguous(), getattr(self, f"gate_up_{e}"), ctx.dtype)
-            y = ops.linear(act, getattr(self, f"down_{e}"), None, torch.float32)
+            act = ops.linear_silu_mul(x[rows].contiguous(), self.operand(f"gate_up_{e}"), ctx.dtype)
+            y = ops.linear(act, self.operand(f"down_{e}"), None, torch.float32)
             out[rows] = y * probs[rows, e].unsqueeze(1)
         return out.to(ctx.dtype)
 
@@ -314,13 +321,13 @@ def routed_spec(config, max_position=None) -> ModelSpec:
     norm = PartSpec.of("rmsnorm", hidden_size=h, eps=raw["eps"])
     attention = PartSpec.of("attention", hidden_size=h, num_heads=2, num_kv_heads=1, head_dim=32, qkv_bias=True)
     layers = [
-        LayerSpec("layers.0.", attention, PartSpec.of("toy_routed", hidden_size=h, intermediate_size=raw["inter"], num_experts=3), norm, norm),
-        LayerSpec("layers.1.", attention, PartSpec.of("gated_mlp", hidden_size=h, intermediate_size=raw["inter"]), norm, norm),
-        LayerSpec("layers.2.", attention, PartSpec.of("toy_routed", hidden_size=h, intermediate_size=raw["inter"], num_experts=3), norm, norm),
+        LayerSpec("layers.0.", attention, PartSpec.of("toy_routed", hidden_size=h, intermediate_size=raw["inter"], num_experts=3), norm, norm, **HF_NAMES),
+        LayerSpec("layers.1.", attention, PartSpec.of("gated_mlp", hidden_size=h, intermediate_size=raw["inter"]), norm, norm, **HF_NAMES),
+        LayerSpec("layers.2.", attention, PartSpec.of("toy_routed", hidden_size=h, intermediate_size=raw["inter"], num_experts=3), norm, norm, **HF_NAMES),
     ]
     return ModelSpec(vocab_size=raw["vocab_size"], hidden_size=h, max_position=128, layers=layers, schedule=[ScheduleEntry(i) for i in range(3)],
                      final_norm=norm, positions={"learned": PartSpec.of("toy_learned", max_position=128, hidden_size=h)},
-                     embedding_position="learned", tie_head=False)
+                     embedding_position="learned", tie_head=False, **HF_ENDS)
 
 
 def plain_routed(tensors: Dict[str, torch.Tensor], raw, tokens):
@@ -396,3 +403,180 @@ def test_toy_architecture_with_routed_experts_and_learned_positions(ops, dtype):
             assert close.float().mean() > 0.9, f"{k}: only {int(close.sum())} of {len(close)} rows match"
         else:
             torch.testing.assert_close(have, want, **bound)
+
+
+# ----------------------------------------------------------------------------------------------------
+# a third toy architecture: what stands at the two ends and how a layer is arranged are parts like the others.
+# An embedding with a scale, a head with a bias and a soft cap on its logits, and a block whose mixer and feed-forward
+# read the same normalised input side by side; all defined and registered here.
+# ----------------------------------------------------------------------------------------------------
+from velox_amd.parts import Block, Embedding, OutputHead, register_arrangement  # noqa: E402
+from velox_amd.parts.base import Param  # noqa: E402
+
+
+class ScaledEmbedding(Embedding):
+    def __init__(self, name, vocab_size, hidden_size, scale):
+        super().__init__("")
+        self.name, self.vocab_size, self.hidden_size, self.scale = name, vocab_size, hidden_size, scale
+        self.table = None
+
+    def params(self):
+        return {"table": single(self.name, (self.vocab_size, self.hidden_size), product=False)}
+
+    def forward(self, token_ids, ctx):
+        return ctx.ops.embed(token_ids, self.table).mul_(self.scale)
+
+
+class SoftcapHead(OutputHead):
+    def __init__(self, name, vocab_size, hidden_size, tied_to, cap):
+        super().__init__("")
+        self.name, self.vocab_size, self.hidden_size, self.tied_to, self.cap = name, vocab_size, hidden_size, tied_to, cap
+        self.weight = self.bias = None
+
+    def params(self):
+        weight = single(self.name, (self.vocab_size, self.hidden_size))
+        if self.tied_to is not None:
+            weight = Param(weight.shape, weight.sources, weight.source_shapes, weight.role, weight.init, alias_of=self.tied_to)
+        return {"weight": weight, "bias": single("head.bias", (self.vocab_size,), role="vector")}
+
+    def prepare_kernels(self, ops):
+        self.prepare_weight(ops, "weight")
+
+    def forward(self, hidden_rows, ctx):
+        logits = ctx.ops.linear(hidden_rows, self.operand("weight"), self.bias, torch.float32)
+        return self.cap * torch.tanh(logits / self.cap)
+
+
+class ParallelBlock(Block):
+    """h = h + mixer(norm(h)) + ff(norm(h)): one norm, both sub-layers read it."""
+
+    def __init__(self, prefix, mixer, feed_forward, mixer_norm, ff_norm):
+        super().__init__(prefix)
+        self.mixer, self.feed_forward, self.norm = mixer, feed_forward, mixer_norm  # (ff_norm is not used and owns no tensors here)
+
+    def children(self):
+        return (self.norm, self.mixer, self.feed_forward)
+
+    def input_norm(self):
+        return self.norm
+
+    def forward(self, residual, pending, ctx, cache, owns_cache, next_norm=None):
+        normed = ctx.ops.materialize(self.norm.forward(residual, pending, ctx))
+        mixed = self.mixer.forward(normed, ctx, cache, owns_cache)
+        residual.add_((mixed.sum(0) if mixed.dim() == 3 else mixed).float())  # (a product may hand back partial sums)
+        return self.feed_forward.forward(normed, ctx)  # added by whoever normalises next
+
+
+def ends_spec(config, max_position=None) -> ModelSpec:
+    raw = config.raw
+    h = raw["hidden_size"]
+    norm = PartSpec.of("rmsnorm", hidden_size=h, eps=raw["eps"])
+    attention = PartSpec.of("attention", hidden_size=h, num_heads=3, num_kv_heads=3, head_dim=32, qkv_bias=False)
+    ff = PartSpec.of("gated_mlp", hidden_size=h, intermediate_size=raw["inter"])
+    layers = [LayerSpec("blocks.0.", attention, ff, norm, norm, position="rope", arrangement="toy_parallel"),
+              LayerSpec("blocks.1.", attention, ff, norm, norm, position="rope")]  # (the framework's own names for the tensors)
+    return ModelSpec(vocab_size=raw["vocab_size"], hidden_size=h, max_position=128, layers=layers, schedule=[ScheduleEntry(0), ScheduleEntry(1)],
+                     final_norm=norm, positions={"rope": PartSpec.of("rotary", rotary_dim=32, theta=10000.0, max_position=128)},
+                     tie_head=raw["tied"], embedding=PartSpec.of("toy_scaled", scale=raw["embedding_scale"]), head=PartSpec.of("toy_softcap", cap=raw["cap"]))
+
+
+def plain_ends(tensors, raw, tokens):
+    eps, n = raw["eps"], len(tokens)
+    cos, sin = rope_tables(32, 10000.0, n)
+    table = tensors["embedding.weight"]
+    x = table[torch.tensor(tokens)] * raw["embedding_scale"]
+
+    def attend(p, a):
+        q = apply_rope((a @ tensors[p + "mixer.q_proj.weight"].T).reshape(n, 3, 32), cos, sin, torch.arange(n))
+        k = apply_rope((a @ tensors[p + "mixer.k_proj.weight"].T).reshape(n, 3, 32), cos, sin, torch.arange(n))
+        v = (a @ tensors[p + "mixer.v_proj.weight"].T).reshape(n, 3, 32)
+        return causal_attention(q, k, v, 1.0 / math.sqrt(32)).reshape(n, 96) @ tensors[p + "mixer.o_proj.weight"].T
+
+    def ff(p, m):
+        return gated_mlp(m, tensors[p + "feed_forward.gate_proj.weight"], tensors[p + "feed_forward.up_proj.weight"], tensors[p + "feed_forward.down_proj.weight"])
+
+    a = rms_norm(x, tensors["blocks.0.mixer_norm.weight"], eps)
+    x = x + attend("blocks.0.", a) + ff("blocks.0.", a)
+    x = x + attend("blocks.1.", rms_norm(x, tensors["blocks.1.mixer_norm.weight"], eps))
+    x = x + ff("blocks.1.", rms_norm(x, tensors["blocks.1.feed_forward_norm.weight"], eps))
+    head = table if raw["tied"] else tensors["head.weight"]
+    logits = rms_norm(x, tensors["final_norm.weight"], eps) @ head.T + tensors["head.bias"]
+    return raw["cap"] * torch.tanh(logits / raw["cap"])
+
+
+def _step_through(runner, cache, prompts, plan):
+    seqs = {k: cache.new_sequence() for k in prompts}
+    done = {k: 0 for k in prompts}
+    got = {k: [] for k in prompts}
+    for cuts in plan:
+        entries = []
+        for k, n in cuts.items():
+            assert cache.append(seqs[k], done[k], n)
+            entries.append(StepEntry(seqs[k], prompts[k][done[k]:done[k] + n], done[k], list(range(n))))
+        logits = runner.step(entries).cpu()
+        at = 0
+        for k, n in cuts.items():
+            got[k].append(logits[at:at + n])
+            at += n
+            done[k] += n
+    return {k: torch.cat(v) for k, v in got.items()}
+
+
+@pytest.mark.parametrize("tied", [True, False])
+def test_toy_architecture_with_its_own_embedding_head_and_arrangement(ops, tied):
+    register_part("embedding", "toy_scaled", ScaledEmbedding)
+    register_part("head", "toy_softcap", SoftcapHead)
+    register_arrangement("toy_parallel", ParallelBlock)
+    register_architecture("EndsToyForCausalLM", lambda raw: ModelConfig(architecture_name(raw), dict(raw)), ends_spec)
+    raw = {"architectures": ["EndsToyForCausalLM"], "hidden_size": 96, "inter": 160, "vocab_size": 77, "eps": 1e-5, "embedding_scale": 9.5, "cap": 0.3, "tied": tied}
+    model = build_model(config_from_dict(raw), torch.float32, "cuda")
+    assert type(model.embedding) is ScaledEmbedding and type(model.head) is SoftcapHead and type(model.blocks[0]) is ParallelBlock
+    bind_random(model, 11, torch.float32, "cuda", storage_dtype=torch.float32)
+    tensors = dict(random_tensors(model, 11))
+    assert ("head.weight" in tensors) == (not tied) and "blocks.0.feed_forward_norm.weight" not in tensors
+    ops.prepare(model, torch.float32)
+    cache = CacheManager(model.cache_needs(), 8, 30, 3, torch.float32, "cuda")
+    runner = ModelRunner(model, cache, ops, torch.float32, "cuda", 128, 3)
+    g = torch.Generator().manual_seed(2)
+    prompts = {k: torch.randint(0, 77, (n,), generator=g).tolist() for k, n in (("p", 19), ("q", 8), ("r", 33))}
+    got = _step_through(runner, cache, prompts, [{"p": 4, "q": 8}, {"p": 1, "r": 20}, {"p": 14, "r": 1}, {"r": 12}])
+    for k, tokens in prompts.items():
+        want = plain_ends(tensors, raw, tokens)
+        assert float(want.abs().max()) > 0.2  # the cap bites: a head without it would fail
+        torch.testing.assert_close(got[k], want, rtol=2e-4, atol=2e-5)
+
+
+def test_stateful_toy_architecture_through_the_engine_with_preemption(tmp_path, ops):
+    """The mixer with state of its own meets the scheduler: admission takes a zeroed slot, preemption gives slot and pages
+    back and recomputes from a zeroed slot, decoding goes through the engine's loop with graphs asked for (and not
+    captured, because the mixer says it reads the host).  Greedy tokens against the plain implementation."""
+    from velox_amd import Engine, EngineConfig, Request, SamplingParams
+    from velox_amd.weights import write_random_model
+
+    register_part("mixer", "toy_decaying_sum", DecayingSumMixer)
+    register_architecture("ToyForCausalLM", lambda raw: ModelConfig(architecture_name(raw), dict(raw)), toy_spec)
+    raw = {"architectures": ["ToyForCausalLM"], "hidden_size": 64, "inter": 96, "vocab_size": 101, "eps": 1e-5, "decay": 0.8}
+    folder = write_random_model(raw, str(tmp_path / "toy"), seed=4, dtype="float32")
+    from safetensors.torch import load_file
+
+    tensors = load_file(f"{folder}/model.safetensors")
+    g = torch.Generator().manual_seed(5)
+    prompts = [torch.randint(0, 101, (n,), generator=g).tolist() for n in (18, 7, 25, 11)]
+    steps = 14
+
+    def plain_greedy(prompt):
+        tokens = list(prompt)
+        for _ in range(steps):
+            tokens.append(int(plain_toy(tensors, raw, tokens)[-1].argmax()))
+        return tokens[len(prompt):]
+
+    want = [plain_greedy(p) for p in prompts]
+    for pages, expect_preemption in ((64, False), (16, True)):
+        engine = Engine.from_pretrained(EngineConfig(model=folder, dtype="float32", device="cuda", max_model_len=64, max_num_seqs=4, max_num_batched_tokens=24,
+                                                     max_prefill_chunk_size=6, block_size=4, num_gpu_blocks=pages, enable_cuda_graphs=True, seed=0), ops=ops)
+        assert not engine.runner.uses_graphs and engine.cache.prefix is None  # (a state stands for tokens a sharer would skip)
+        requests = [Request(f"r{i}", p, SamplingParams(temperature=0.0, max_tokens=steps, ignore_eos=True)) for i, p in enumerate(prompts)]
+        engine.generate(requests)
+        assert (engine.scheduler.num_preemptions > 0) == expect_preemption
+        assert [r.output_token_ids for r in requests] == want
+        assert engine.cache.num_used_pages() == 0 and engine.cache.state.num_free == 4

@@ -23,36 +23,36 @@ def test_publish_match_and_eviction_order():
     allocator = PageAllocator(12)
     trie = PrefixCache([allocator], page_size=2)
     tokens_a = [1, 2, 3, 4, 5, 6, 7]
-    pages_a = allocator.allocate_many(4)  # the fourth page is not full
+    pages_a = allocator.take_many(4)  # the fourth page is not full
     assert trie.publish(tokens_a, [pages_a], 0, 3) == (3, True) and trie.num_nodes == 3 and trie.num_reclaimable == 0
-    assert [allocator.ref_count(p) for p in pages_a] == [2, 2, 2, 1]
+    assert [allocator.holders(p) for p in pages_a] == [2, 2, 2, 1]
     # a second request with the same first two pages and another third
     tokens_b = [1, 2, 3, 4, 9, 9, 9]
     found = trie.match(tokens_b, max_pages=3)
     assert [n.pages for n in found] == [(pages_a[0],), (pages_a[1],)]
     for node in found:
-        allocator.incref(node.pages[0])
+        allocator.share(node.pages[0])
         trie.page_taken(node.pages[0])
-    own = allocator.allocate()
+    own = allocator.take()
     assert trie.publish(tokens_b, [[pages_a[0], pages_a[1], own]], 2, 3) == (3, True) and trie.num_nodes == 4
     trie.assert_consistent()
     # the first request ends: its third page is held by nobody any more, the first two still by the second request
     for page in pages_a:
-        allocator.free(page)
+        allocator.drop(page)
         trie.page_dropped(page)
-    assert trie.num_reclaimable == 1 and allocator.ref_count(pages_a[2]) == 1 and allocator.ref_count(pages_a[3]) == 0
+    assert trie.num_reclaimable == 1 and allocator.holders(pages_a[2]) == 1 and allocator.holders(pages_a[3]) == 0
     trie.assert_consistent()
-    assert trie.evict(5) == 1 and allocator.ref_count(pages_a[2]) == 0 and trie.num_nodes == 3
+    assert trie.evict(5) == 1 and allocator.holders(pages_a[2]) == 0 and trie.num_nodes == 3
     # the second ends too: leaves go before their parents, the least recently used leaf first
     for page in (pages_a[0], pages_a[1], own):
-        allocator.free(page)
+        allocator.drop(page)
         trie.page_dropped(page)
     assert trie.num_reclaimable == 3
-    assert trie.evict(1) == 1 and allocator.ref_count(own) == 0 and allocator.ref_count(pages_a[1]) == 1
+    assert trie.evict(1) == 1 and allocator.holders(own) == 0 and allocator.holders(pages_a[1]) == 1
     assert trie.match([1, 2, 3, 4, 9, 9], max_pages=3)[-1].pages == (pages_a[1],)
     assert trie.evict(10) == 2 and trie.num_nodes == 0 and allocator.num_used == 0 and trie.num_reclaimable == 0
     trie.assert_consistent()
-    allocator.assert_consistent()
+    allocator.verify()
     assert trie.hit_rate == pytest.approx((4 + 4) / (6 + 6))
 
 
@@ -61,19 +61,19 @@ def test_least_recently_used_leaf_goes_first_and_a_held_leaf_stays():
     trie = PrefixCache([allocator], page_size=1)
     pages = {}
     for token in (10, 20, 30):
-        pages[token] = allocator.allocate()
+        pages[token] = allocator.take()
         trie.publish([token], [[pages[token]]], 0, 1)
-        allocator.free(pages[token])
+        allocator.drop(pages[token])
         trie.page_dropped(pages[token])
     assert trie.num_reclaimable == 3
     trie.match([10], max_pages=1)  # 10 is the most recently used now, 20 the least
     holder = trie.match([20], max_pages=1)[0]  # ... but 20 is taken by a request
-    allocator.incref(holder.pages[0])
+    allocator.share(holder.pages[0])
     trie.page_taken(holder.pages[0])
     assert trie.num_reclaimable == 2
     assert trie.evict(1) == 1 and not trie.holds(pages[30]) and trie.holds(pages[10]) and trie.holds(pages[20])
     assert trie.evict(5) == 1 and trie.holds(pages[20]) and trie.num_nodes == 1  # the held one cannot go
-    allocator.free(pages[20])
+    allocator.drop(pages[20])
     trie.page_dropped(pages[20])
     assert trie.evict(5) == 1 and trie.num_nodes == 0
     trie.assert_consistent()
@@ -82,26 +82,26 @@ def test_least_recently_used_leaf_goes_first_and_a_held_leaf_stays():
 def test_a_request_stops_publishing_where_another_request_page_stands():
     allocator = PageAllocator(10)
     trie = PrefixCache([allocator], page_size=2)
-    first = allocator.allocate_many(2)
-    second = allocator.allocate_many(3)
+    first = allocator.take_many(2)
+    second = allocator.take_many(3)
     assert trie.publish([1, 2, 3, 4], [first], 0, 2) == (2, True)
     # the same tokens computed by another request at the same time, with pages of its own: nothing of it is published,
     # not even its third page, which would hang below a node whose page it does not hold
     assert trie.publish([1, 2, 3, 4, 5, 6], [second], 0, 3) == (0, False)
-    assert trie.num_nodes == 2 and [allocator.ref_count(p) for p in second] == [1, 1, 1]
+    assert trie.num_nodes == 2 and [allocator.holders(p) for p in second] == [1, 1, 1]
     trie.assert_consistent()
 
 
 def test_nodes_hold_one_page_per_group():
     a, b = PageAllocator(6), PageAllocator(6)
     trie = PrefixCache([a, b], page_size=2)
-    pa, pb = a.allocate_many(2), b.allocate_many(2)
+    pa, pb = a.take_many(2), b.take_many(2)
     pb.reverse()
     assert trie.publish([7, 7, 8, 8], [pa, pb], 0, 2) == (2, True)
     for page in pa:
-        a.free(page)
+        a.drop(page)
     for page in pb:
-        b.free(page)
+        b.drop(page)
     for page in pa:
         trie.page_dropped(page)
     assert trie.num_reclaimable == 2 and a.num_used == 2 and b.num_used == 2
@@ -139,7 +139,7 @@ def test_matched_pages_enter_the_table_and_one_token_is_left_to_compute():
     d = m.new_sequence()
     assert m.match_prefix(d, tokens[:4] + [0] + tokens[5:]) == 4
     m.assert_consistent([a, b, c, d])
-    assert [m.groups[0].allocator.ref_count(p) for p in a.tables[0]] == [5, 4, 3]
+    assert [m.groups[0].allocator.holders(p) for p in a.tables[0]] == [5, 4, 3]
     for seq in (a, b, c, d):
         m.free_sequence(seq)
     m.assert_consistent([])
@@ -219,19 +219,16 @@ def scheduler(pages=33, page=4, seqs=4, budget=16, chunk=8, max_len=128, waterma
 
 
 def run_step(s, out):
-    for r in out.decode_batch:
+    sampled = list(out.decodes)
+    for r in out.decodes:
         s.advance(r, 1)
-    sampled = list(out.decode_batch)
-    for r in out.prefill_batch:
-        completes = r.num_computed_tokens + r.current_chunk_size >= len(r.all_token_ids)
-        s.advance(r, r.current_chunk_size)
-        r.refresh_status()
-        if completes:
-            sampled.append(r)
+    for portion in out.portions:
+        s.advance(portion.request, portion.count)
+        if portion.completes:
+            sampled.append(portion.request)
     for r in sampled:
-        r.append_token(1000 + len(r.output_token_ids))
-        r.refresh_status()
-        reason = r.should_stop(r.output_token_ids[-1], frozenset())
+        r.record_token(1000 + len(r.output_token_ids))
+        reason = r.stop_reason(r.output_token_ids[-1], frozenset())
         if reason:
             r.finish(reason)
 
@@ -254,14 +251,14 @@ def test_admission_takes_over_a_published_prefix():
     second = Request("second", prompt + [77, 78], SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True))
     s.add_request(second)
     out = s.schedule()
-    assert out.prefill_batch == [second] and second.num_cached_tokens == 20 and second.num_computed_tokens == 20 and second.current_chunk_size == 4
-    assert out.num_batched_tokens == 4
+    assert [p.request for p in out.portions] == [second] and second.num_cached_tokens == 20 and second.num_computed_tokens == 20
+    assert out.count_of(second) == 4 and out.portions[0].start == 20 and out.num_tokens == 4
     run_to_end(s)
     # the same prompt again: all of it is known, but its last page is computed again so that there is a row to sample from
     third = Request("third", prompt[:20], SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True))
     s.add_request(third)
     out = s.schedule()
-    assert third.num_cached_tokens == 16 and third.current_chunk_size == 4
+    assert third.num_cached_tokens == 16 and out.count_of(third) == 4
     run_to_end(s)
     s.cache.assert_consistent([])
     assert s.stats()["prefix_hit_rate"] > 0 and s.stats()["evictable_blocks"] == s.cache.prefix.num_nodes
@@ -292,7 +289,7 @@ def test_pages_that_only_the_trie_holds_count_as_room_for_admission():
     other = Request("other", list(range(201, 225)), SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True))
     s.add_request(other)
     out = s.schedule()
-    assert out.prefill_batch == [other] and other.current_chunk_size == 24 and other.status is RequestStatus.RUNNING_PREFILL
+    assert [p.request for p in out.portions] == [other] and out.count_of(other) == 24 and other.status is RequestStatus.RUNNING_PREFILL
     assert s.cache.prefix.num_nodes == 2  # four of the first request's pages had to go
     run_to_end(s)
     s.cache.assert_consistent([])

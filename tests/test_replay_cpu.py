@@ -20,13 +20,22 @@ def test_all_ways_of_cutting_agree_with_the_plain_model(tmp_path, name):
     expected = rc.expected_logits(config, weights, requests)
     page = PAGE_SIZE[name]
     for label, trace in (("whole", rc.whole(requests)), ("tail", rc.tail_one_by_one(requests)),
-                         ("portions", rc.changing_portions(requests)), ("mixed", rc.mixed(requests, seed=5))):
+                         ("portions", rc.changing_portions(requests)), ("mixed", rc.mixed(requests, seed=5)),
+                         ("recompute", rc.mixed(requests, seed=6, preempt=("r0", "r2", "r4")))):
         pool = rc.tokens_needed(trace, page)
         replayer = Replayer(folder, "float32", pool, block_size=page, device="cpu", ops=TorchOps())
-        got = rc.collect(trace, rc.run_trace(replayer, trace), requests)
+        outputs = rc.run_trace(replayer, trace)
+        got = rc.collect(trace, outputs, requests)
         for rid in requests:
             torch.testing.assert_close(got[rid], expected[rid], msg=lambda m: f"{name} {label} {rid}: {m}", **TOL)
-        if label == "mixed":
+        if label == "recompute":
+            # the requests that were ended half way and fed again from their first token: both runs gave the plain logits
+            first = rc.first_runs(trace, outputs, requests)
+            for rid in ("r0", "r2", "r4"):
+                assert sum(1 for r in trace if rid in r["end"]) == 2
+                for position, row in first[rid].items():
+                    torch.testing.assert_close(torch.from_numpy(row), expected[rid][position], **TOL)
+        if label in ("mixed", "recompute"):
             # the pool is so small that pages were handed out more than once
             total_pages = sum((len(t) + page - 1) // page for t in requests.values())
             assert total_pages > replayer.cache.num_total_pages

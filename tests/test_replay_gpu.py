@@ -39,16 +39,26 @@ def test_four_ways_of_cutting(tmp_path, name, dtype):
     page = PAGE_SIZE[name]
     results = {}
     for label, trace in (("whole", rc.whole(requests)), ("tail", rc.tail_one_by_one(requests)),
-                         ("portions", rc.changing_portions(requests)), ("mixed", rc.mixed(requests, seed=5))):
+                         ("portions", rc.changing_portions(requests)), ("mixed", rc.mixed(requests, seed=5)),
+                         ("recompute", rc.mixed(requests, seed=8, preempt=("r0", "r2", "r6")))):
         replayer = Replayer(folder, dtype, rc.tokens_needed(trace, page), block_size=page)
-        results[label] = rc.collect(trace, rc.run_trace(replayer, trace), requests)
+        outputs = rc.run_trace(replayer, trace)
+        results[label] = rc.collect(trace, outputs, requests)
         for rid in requests:
             torch.testing.assert_close(results[label][rid], expected[rid], msg=lambda m: f"{name} {dtype} {label} {rid}: {m}", **TOL[dtype])
-        if label == "mixed":
+        if label in ("mixed", "recompute"):
             assert sum((len(t) + page - 1) // page for t in requests.values()) > replayer.cache.num_total_pages
+        if label == "recompute":
+            # requests ended half way, their pages taken by others, then fed again from their first token under the same
+            # id (what preemption does): the first run's logits were right too, and the second run's match them
+            first = rc.first_runs(trace, outputs, requests)
+            for rid in ("r0", "r2", "r6"):
+                assert sum(1 for r in trace if rid in r["end"]) == 2 and len(first[rid]) >= len(requests[rid]) // 2
+                for position, row in first[rid].items():
+                    torch.testing.assert_close(torch.from_numpy(row.copy()), expected[rid][position], **TOL[dtype])
     if dtype == "float32":
         # the ways of cutting agree with each other much closer than any of them must with the plain model
-        for label in ("tail", "portions", "mixed"):
+        for label in ("tail", "portions", "mixed", "recompute"):
             for rid in requests:
                 torch.testing.assert_close(results[label][rid], results["whole"][rid], rtol=5e-5, atol=5e-6)
 
@@ -174,6 +184,45 @@ def test_layers_of_the_real_size_in_four_ways_of_cutting(tmp_path, dtype):
         for label in ("tail", "portions", "mixed"):
             for rid in requests:
                 torch.testing.assert_close(results[label][rid], results["whole"][rid], **tol)
+
+
+@pytest.mark.parametrize("live", [40, 12])
+def test_captured_decode_steps_of_many_requests_at_the_real_size(tmp_path, live):
+    """40 and 12 requests decode together through the captured steps of 64 and 16 rows, at the widths of Qwen2.5-7B:
+    the products of 17 to 64 rows (split sums, the library's kernels), the decode attention with many sequences and rows
+    padded onto the null page.  Logits of every decoded position against the plain model, to the bound of the test above."""
+    from velox_amd.weights import write_random_model
+
+    folder = write_random_model(QWEN25_7B_TWO_LAYERS, str(tmp_path / "real_size"), 3, dtype="bfloat16")
+    config, weights = read_model_folder(folder)
+    decoded = 6
+    lengths = [20 + (7 * i) % 23 for i in range(live)]
+    requests = rc.request_set(config["vocab_size"], lengths, seed=61)
+    trace = []
+    names = list(requests)
+    for lo in range(0, live, 8):  # prompts, eight requests a step, all but the last `decoded` tokens
+        trace.append({"step": len(trace), "end": [],
+                      "entries": [{"id": rid, "tokens": requests[rid][:len(requests[rid]) - decoded], "want": []} for rid in names[lo:lo + 8]]})
+    for i in range(decoded):
+        trace.append({"step": len(trace), "end": names if i == decoded - 1 else [],
+                      "entries": [{"id": rid, "tokens": [requests[rid][len(requests[rid]) - decoded + i]], "want": [0]} for rid in names]})
+    replayer = Replayer(folder, "bfloat16", rc.tokens_needed(trace, 16), block_size=16, max_live=64, enable_graphs=True)
+    assert replayer.runner.uses_graphs
+    outputs = rc.run_trace(replayer, trace)
+    assert replayer.runner.num_graph_replays == decoded
+    eager = Replayer(folder, "bfloat16", rc.tokens_needed(trace, 16), block_size=16, max_live=64, enable_graphs=False, ops=replayer.ops)
+    eager_outputs = rc.run_trace(eager, trace)
+    for index, rid in enumerate(names):
+        expected = qwen2_logits(config, weights, requests[rid])[-decoded:]
+        got = torch.stack([torch.from_numpy(outputs[len(trace) - decoded + i][index].copy()) for i in range(decoded)])
+        spread = float(expected.std())
+        error = got - expected
+        assert float(error.pow(2).mean().sqrt()) < 0.0175 * spread, (rid, float(error.pow(2).mean().sqrt()), spread)
+        assert float(error.abs().max()) < 8 * 0.0175 * spread, (rid, float(error.abs().max()), spread)
+        # a captured step pads to 16 or 64 rows and may take other kernels than the same step uncaptured (the rows decide):
+        # the two agree as two bfloat16 runs do
+        same = torch.stack([torch.from_numpy(eager_outputs[len(trace) - decoded + i][index].copy()) for i in range(decoded)])
+        assert float((got - same).pow(2).mean().sqrt()) < 0.0175 * spread
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

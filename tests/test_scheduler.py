@@ -20,25 +20,27 @@ def request(rid, prompt_len, max_tokens=4):
 
 def run_step(s, out):
     """What the engine does after a forward: advance, append a token to rows that completed their tokens."""
-    scheduled = out.decode_batch + out.prefill_batch
+    scheduled = out.requests()
     assert len({id(r) for r in scheduled}) == len(scheduled), "a request is in a step twice"
     assert all(r.cache is not None and r in s.running for r in scheduled), "a scheduled request has no pages"
     assert not any(r in scheduled for r in out.preempted if r.cache is None)
-    for r in out.decode_batch:
+    sampled = list(out.decodes)
+    for r in out.decodes:
         s.advance(r, 1)
-    for r in out.prefill_batch:
-        completes = r.num_computed_tokens + r.current_chunk_size >= len(r.all_token_ids)
-        s.advance(r, r.current_chunk_size)
-        r.refresh_status()
-        if not completes:
-            continue
-        out.decode_batch.append(r)  # sampled below
-    for r in out.decode_batch:
-        r.append_token(1000 + len(r.output_token_ids))
-        r.refresh_status()
-        reason = r.should_stop(r.output_token_ids[-1], frozenset())
+    for portion in out.portions:
+        assert portion.start == portion.request.num_computed_tokens
+        s.advance(portion.request, portion.count)
+        if portion.completes:
+            sampled.append(portion.request)
+    for r in sampled:
+        r.record_token(1000 + len(r.output_token_ids))
+        reason = r.stop_reason(r.output_token_ids[-1], frozenset())
         if reason:
             r.finish(reason)
+
+
+def portions(out):
+    return [(p.request.request_id, p.count) for p in out.portions]
 
 
 def test_prompt_is_cut_under_budget_and_chunk_then_decodes_first():
@@ -47,15 +49,15 @@ def test_prompt_is_cut_under_budget_and_chunk_then_decodes_first():
     s.add_request(a)
     s.add_request(b)
     out = s.schedule()
-    assert [r.request_id for r in out.prefill_batch] == ["a", "b"] and (a.current_chunk_size, b.current_chunk_size) == (8, 5)
-    assert out.num_batched_tokens == 13 and not out.decode_batch
+    assert portions(out) == [("a", 8), ("b", 5)] and (out.count_of(a), out.count_of(b)) == (8, 5)
+    assert out.num_tokens == 13 and not out.decodes
     run_step(s, out)
     assert a.status is RequestStatus.RUNNING_PREFILL and b.status is RequestStatus.RUNNING_DECODE and b.output_token_ids == [1000]
     out = s.schedule()
-    assert [r.request_id for r in out.decode_batch] == ["b"] and [r.request_id for r in out.prefill_batch] == ["a"] and a.current_chunk_size == 8
+    assert [r.request_id for r in out.decodes] == ["b"] and portions(out) == [("a", 8)] and out.count_of(b) == 1
     run_step(s, out)
     out = s.schedule()
-    assert a.current_chunk_size == 3 and a.num_computed_tokens == 16
+    assert out.count_of(a) == 3 and a.num_computed_tokens == 16 and out.portions[0].start == 16 and out.portions[0].completes
     run_step(s, out)
     assert a.status is RequestStatus.RUNNING_DECODE and a.output_token_ids == [1000]
 
@@ -67,7 +69,7 @@ def test_budget_counts_decodes_before_prompts():
     run_step(s, s.schedule())
     s.add_request(request("p", 30))
     out = s.schedule()
-    assert len(out.decode_batch) == 3 and out.prefill_batch[0].current_chunk_size == 3  # 6 - 3 decodes
+    assert len(out.decodes) == 3 and portions(out) == [("p", 3)]  # 6 - 3 decodes
 
 
 def test_finish_frees_pages_at_the_next_schedule_and_reasons():
@@ -82,8 +84,9 @@ def test_finish_frees_pages_at_the_next_schedule_and_reasons():
     assert out.is_empty() and s.cache.num_used_pages() == 0 and not s.has_work() and s.num_finished == 1
     s.cache.assert_consistent([])
     stop = Request("s", [1, 2, 3], SamplingParams(max_tokens=9, stop_token_ids=[77]))
-    assert stop.should_stop(77, frozenset()) is FinishReason.STOP and stop.should_stop(5, frozenset({5})) is FinishReason.STOP
-    assert Request("i", [1], SamplingParams(max_tokens=9, ignore_eos=True)).should_stop(5, frozenset({5})) is None
+    assert stop.stop_reason(77, frozenset()) is FinishReason.STOP and stop.stop_reason(5, frozenset({5})) is FinishReason.STOP
+    assert stop.stop_reason(6, frozenset({5})) is None
+    assert Request("i", [1], SamplingParams(max_tokens=9, ignore_eos=True)).stop_reason(5, frozenset({5})) is None
 
 
 def test_limits_are_refused_at_add():
@@ -108,14 +111,14 @@ def test_admission_waits_for_slots_and_keeps_a_watermark_first_come_first_served
         s.add_request(request(rid, n, max_tokens=2))
     out = s.schedule()
     # a takes 3 pages; b wants 5 of the 7 left, headroom 7 - 2 = 5: fits; c finds no slot
-    assert [r.request_id for r in out.prefill_batch] == ["a", "b"] and s.num_waiting == 1
+    assert portions(out) == [("a", 12), ("b", 20)] and s.num_waiting == 1
     run_step(s, out)
     s2 = make(pages=11, seqs=4, budget=64, chunk=64, watermark=0.2)
     for rid, n in (("a", 12), ("b", 28), ("c", 4)):
         s2.add_request(request(rid, n, max_tokens=2))
     out = s2.schedule()
     # b needs 7 pages, headroom is 5: it gets a 20-token portion (5 pages); c then sees headroom 0 and waits behind it
-    assert [(r.request_id, r.current_chunk_size) for r in out.prefill_batch] == [("a", 12), ("b", 20)]
+    assert portions(out) == [("a", 12), ("b", 20)]
     assert [r.request_id for r in s2.waiting] == ["c"]
 
 
@@ -131,11 +134,11 @@ def test_decode_out_of_pages_preempts_the_newest_and_recomputes_it():
     for _ in range(3):
         run_step(s, s.schedule())  # positions 9, 10, 11 fit
     out = s.schedule()  # position 12: a needs a 4th page, none free: b (the newest) is preempted
-    assert [r.request_id for r in out.preempted] == ["b"] and [r.request_id for r in out.decode_batch] == ["a"]
+    assert [r.request_id for r in out.preempted] == ["b"] and [r.request_id for r in out.decodes] == ["a"]
     assert b.num_preemptions == 1 and s.num_preemptions == 1 and len(b.output_token_ids) == 5  # its tokens are kept
     # the same scheduling decision admits it again from the front of the queue, from position 0, with what fits
-    assert [r.request_id for r in out.prefill_batch] == ["b"] and b.num_computed_tokens == 0
-    assert b.status is RequestStatus.RUNNING_PREFILL and b.current_chunk_size == 4  # 2 pages free, 1 held back
+    assert b.status is RequestStatus.RUNNING_PREFILL and b.num_computed_tokens == 0
+    assert portions(out) == [("b", 4)] and out.portions[0].start == 0  # 2 pages free, 1 held back
     run_step(s, out)
     s.cache.assert_consistent([a.cache, b.cache])
     # its recomputation covers prompt and generated tokens (13), then it decodes on: no token is lost or sampled twice
@@ -158,14 +161,14 @@ def test_oldest_prefill_may_evict_newer_requests_but_a_newer_prefill_waits():
     s.add_request(a)
     s.add_request(b)
     out = s.schedule()  # a: 8 tokens, 2 pages; b: the 4 tokens the budget leaves, 1 page
-    assert [(r.request_id, r.current_chunk_size) for r in out.prefill_batch] == [("a", 8), ("b", 4)]
+    assert portions(out) == [("a", 8), ("b", 4)]
     run_step(s, out)
     out = s.schedule()  # a takes the last 2 free pages; b finds none and, not being the oldest, just waits
-    assert [(r.request_id, r.current_chunk_size) for r in out.prefill_batch] == [("a", 8)] and not out.preempted
+    assert portions(out) == [("a", 8)] and not out.preempted
     run_step(s, out)
     out = s.schedule()  # a needs one more page: as the oldest prefill it evicts b, the newest request
-    assert [r.request_id for r in out.preempted] == ["b"] and out.prefill_batch[0] is a and a.current_chunk_size == 2
-    assert b.num_preemptions == 1 and b.num_computed_tokens == 0
+    assert [r.request_id for r in out.preempted] == ["b"] and portions(out) == [("a", 2)]
+    assert b.num_preemptions == 1 and b.num_computed_tokens == 0 and b.status is RequestStatus.PREEMPTED and s.waiting[0] is b
     run_step(s, out)
     while s.has_work():
         run_step(s, s.schedule())
@@ -212,7 +215,7 @@ def test_a_victim_leaves_the_step_it_was_already_given_a_token_in():
     run_step(s, s.schedule())  # b decodes; a: 8 more (4 pages)
     assert s.cache.num_free_pages() == 1
     out = s.schedule()  # b decodes (position 4: takes the last page); a then needs a 5th page and evicts b
-    assert [r.request_id for r in out.preempted] == ["b"] and b not in out.decode_batch
+    assert [r.request_id for r in out.preempted] == ["b"] and b not in out.decodes and out.count_of(b) == 0
     run_step(s, out)
     while s.has_work():
         run_step(s, s.schedule())
@@ -233,9 +236,9 @@ def test_the_next_decode_step_can_be_fixed_while_one_is_in_flight():
     s = make(pages=33, page=4, budget=16)
     requests = decoding(s, [3, 4, 7])
     out = s.schedule()  # a decode-only step: "in flight" until run_step books it
-    assert out.decode_batch == requests and not out.prefill_batch
+    assert out.decodes == requests and not out.portions
     pages_before = [len(r.cache.tables[0]) for r in requests]
-    ahead = s.schedule_ahead(out.decode_batch)
+    ahead = s.schedule_ahead(out.decodes)
     assert ahead == requests
     # every table now covers the position after the one in flight
     for r, before in zip(requests, pages_before):
@@ -245,7 +248,7 @@ def test_the_next_decode_step_can_be_fixed_while_one_is_in_flight():
     for r in ahead:
         assert len(r.cache.tables[0]) * 4 >= r.num_computed_tokens + 1
         s.advance(r, 1)
-        r.append_token(7)
+        r.record_token(7)
     s.cache.assert_consistent([r.cache for r in requests])
 
 
@@ -255,41 +258,58 @@ def test_nothing_is_fixed_ahead_when_the_next_step_could_look_different():
     requests = decoding(s, [3, 4])
     s.add_request(request("late", 5))
     out = s.schedule()  # both slots are taken: the late request waits
-    assert not out.prefill_batch and len(s.waiting) == 1
-    assert s.schedule_ahead(out.decode_batch) is None
+    assert not out.portions and len(s.waiting) == 1
+    assert s.schedule_ahead(out.decodes) is None
     # a request reaches its length limit with the token in flight
     s = make(pages=33, page=4, budget=16)
     requests = decoding(s, [3, 4], max_tokens=2)  # one token each so far
     out = s.schedule()
-    assert s.schedule_ahead(out.decode_batch) is None
+    assert s.schedule_ahead(out.decodes) is None
     # not every running request is in the step
     s = make(pages=33, page=4, budget=16)
     requests = decoding(s, [3, 4, 5])
     out = s.schedule()
-    assert s.schedule_ahead(out.decode_batch[:2]) is None
+    assert s.schedule_ahead(out.decodes[:2]) is None
     # pages are short: both requests sit at the end of a page and one page is free; nothing may be taken
     s = make(pages=4, page=4, budget=16, watermark=0.01)  # 3 usable pages
     requests = decoding(s, [3, 3])  # 4 tokens each after the first sampled one: position 4 needs a second page
     out = s.schedule()
-    assert len(out.decode_batch) == 2
+    assert len(out.decodes) == 2
     if True:
         free_before = s.cache.groups[0].allocator.num_free
         tables = [list(r.cache.tables[0]) for r in requests]
-        assert s.schedule_ahead(out.decode_batch) is None
+        assert s.schedule_ahead(out.decodes) is None
         assert s.cache.groups[0].allocator.num_free == free_before and [list(r.cache.tables[0]) for r in requests] == tables
 
 
 def test_listeners_hear_tokens_and_the_end_and_may_fail():
-    from velox_amd.engine.request import RequestEvent
-
     r = request("r", 3, max_tokens=2)
     heard = []
-    r.add_listener(lambda req, event: heard.append((req.request_id, event)))
-    r.add_listener(lambda req, event: 1 / 0)  # a failing listener is logged, the request goes on
-    r.append_token(7)
-    r.append_token(8)
-    assert r.num_output_tokens == 2 and r.max_tokens == 2 and r.tokens_for_chunk(2) == [1, 2]
-    r.finish(r.should_stop(8, frozenset()))
+    r.subscribe(on_token=lambda req, token: heard.append((req.request_id, "token", token)),
+                on_finish=lambda req, reason: heard.append((req.request_id, "finish", reason)))
+    r.subscribe(on_token=lambda req, token: 1 / 0, on_finish=lambda req, reason: 1 / 0)  # a failing listener is logged, the request goes on
+    r.record_token(7)
+    r.record_token(8)
+    assert r.num_output_tokens == 2 and r.all_token_ids == [1, 2, 3, 7, 8] and r.first_token_time is not None
+    r.finish(r.stop_reason(8, frozenset()))
     r.finish(FinishReason.ABORT)  # the second end is not heard
-    assert heard == [("r", RequestEvent("token", token_id=7)), ("r", RequestEvent("token", token_id=8)),
-                     ("r", RequestEvent("finish", finish_reason=FinishReason.LENGTH))]
+    assert heard == [("r", "token", 7), ("r", "token", 8), ("r", "finish", FinishReason.LENGTH)]
+    assert r.finished and r.status is RequestStatus.FINISHED and r.time_to_first_token >= 0
+
+
+def test_status_follows_from_what_the_request_holds():
+    s = make(pages=33, page=4, budget=8, chunk=8)
+    r = request("r", 11, max_tokens=3)
+    assert r.status is RequestStatus.WAITING
+    s.add_request(r)
+    run_step(s, s.schedule())
+    assert r.status is RequestStatus.RUNNING_PREFILL and r.num_uncomputed_tokens == 3
+    run_step(s, s.schedule())
+    assert r.status is RequestStatus.RUNNING_DECODE and r.num_uncomputed_tokens == 1 and r.output_token_ids == [1000]
+    s._preempt(r)
+    assert r.status is RequestStatus.PREEMPTED and r.cache is None and r.num_computed_tokens == 0 and r.num_uncomputed_tokens == 12
+    run_step(s, s.schedule())
+    assert r.status is RequestStatus.RUNNING_PREFILL and r.num_preemptions == 1
+    while s.has_work():
+        run_step(s, s.schedule())
+    assert r.status is RequestStatus.FINISHED and r.output_token_ids == [1000, 1001, 1002]

@@ -61,9 +61,6 @@ class TorchOps:
     def prepare(self, model, dtype) -> None:
         pass
 
-    def register_weight(self, weight, stacked=1, rotary_heads=None) -> None:
-        pass
-
     def materialize(self, x):
         return x
 

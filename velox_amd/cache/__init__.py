@@ -1,2 +1,2 @@
-from .allocator import NULL_PAGE, OutOfPagesError, PageAllocator  # noqa: F401
+from .allocator import NULL_PAGE, PoolExhausted, PageAllocator  # noqa: F401
 from .manager import CacheManager, PagedView, SequenceCache, StateSlots, StateView, pages_that_fit  # noqa: F401

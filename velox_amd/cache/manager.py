@@ -29,7 +29,7 @@ import numpy as np
 import torch
 
 from ..parts.base import PagedNeed, StateNeed
-from .allocator import NULL_PAGE, OutOfPagesError, PageAllocator
+from .allocator import NULL_PAGE, PoolExhausted, PageAllocator
 from .prefix import PrefixCache
 
 
@@ -266,7 +266,7 @@ class CacheManager:
                 return False
         for n, group, table in zip(extra, self.groups, seq.tables):
             if n:
-                table.extend(group.allocator.allocate_many(n))
+                table.extend(group.allocator.take_many(n))
                 seq.version += 1
         return True
 
@@ -280,7 +280,7 @@ class CacheManager:
         nodes = self.prefix.match(tokens, max_pages=min((len(tokens) - 1) // self.page_size, self.max_pages_per_seq))
         for node in nodes:
             for index, (group, page) in enumerate(zip(self.groups, node.pages)):
-                group.allocator.incref(page)
+                group.allocator.share(page)
                 seq.tables[index].append(page)
             self.prefix.page_taken(node.pages[0])
         if nodes:
@@ -306,7 +306,7 @@ class CacheManager:
             table = seq.tables[index]
             for position in range(seq.released[index], first):
                 if table[position] != NULL_PAGE:
-                    group.allocator.free(table[position])
+                    group.allocator.drop(table[position])
                     table[position] = NULL_PAGE
                     seq.version += 1
                     given_back += 1
@@ -318,7 +318,7 @@ class CacheManager:
             group = self.groups[index]
             for page in seq.tables[index]:  # (in table order, so that the request's last page is the next one handed out)
                 if page != NULL_PAGE:
-                    group.allocator.free(page)
+                    group.allocator.drop(page)
                     if index == 0 and self.prefix is not None:
                         self.prefix.page_dropped(page)
             seq.tables[index] = []
@@ -367,7 +367,7 @@ class CacheManager:
         if self.prefix is not None:
             self.prefix.assert_consistent()
         for index, group in enumerate(self.groups):
-            group.allocator.assert_consistent()
+            group.allocator.verify()
             holders: Dict[int, int] = {}
             for seq in live:
                 pages = [p for p in seq.tables[index] if p != NULL_PAGE]
@@ -382,8 +382,8 @@ class CacheManager:
                 raise AssertionError(f"group {index}: a page is held twice")
             for page in set(holders) | published:
                 expected = holders.get(page, 0) + (page in published)
-                if group.allocator.ref_count(page) != expected:
-                    raise AssertionError(f"group {index}: page {page} has refcount {group.allocator.ref_count(page)}, expected {expected}")
+                if group.allocator.holders(page) != expected:
+                    raise AssertionError(f"group {index}: page {page} has refcount {group.allocator.holders(page)}, expected {expected}")
             if live is not None and len(set(holders) | published) != group.allocator.num_used:
                 raise AssertionError(f"group {index}: {group.allocator.num_used} pages used but {len(set(holders) | published)} accounted for (a page was lost)")
 

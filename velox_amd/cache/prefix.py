@@ -67,7 +67,7 @@ class PrefixCache:
 
     # -- bookkeeping ----------------------------------------------------------------------
     def _held_by_requests(self, node: PrefixNode) -> bool:
-        return self.allocators[0].ref_count(node.pages[0]) > 1
+        return self.allocators[0].holders(node.pages[0]) > 1
 
     def _touch(self, node: PrefixNode) -> None:
         self._clock += 1
@@ -83,13 +83,13 @@ class PrefixCache:
     def page_taken(self, first_group_page: int) -> None:
         """A request has just added its reference to a published page (called after the increment)."""
         node = self._node_of.get(first_group_page)
-        if node is not None and self.allocators[0].ref_count(first_group_page) == 2:
+        if node is not None and self.allocators[0].holders(first_group_page) == 2:
             self.num_reclaimable -= 1
 
     def page_dropped(self, first_group_page: int) -> None:
         """A request has just given up its reference to a published page (called after the decrement)."""
         node = self._node_of.get(first_group_page)
-        if node is not None and self.allocators[0].ref_count(first_group_page) == 1:
+        if node is not None and self.allocators[0].holders(first_group_page) == 1:
             self.num_reclaimable += 1
             self._offer(node)
 
@@ -134,7 +134,7 @@ class PrefixCache:
             else:
                 child = PrefixNode(key, pages, node)
                 for allocator, page in zip(self.allocators, pages):
-                    allocator.incref(page)
+                    allocator.share(page)
                 node.children[key] = child
                 self._node_of[pages[0]] = child
             self._touch(child)
@@ -154,7 +154,7 @@ class PrefixCache:
             node.alive = False
             node.parent = None
             for allocator, page in zip(self.allocators, node.pages):
-                allocator.free(page)
+                allocator.drop(page)
             self.num_reclaimable -= 1
             freed += 1
             if parent is not self.root:
@@ -179,10 +179,10 @@ class PrefixCache:
                     raise AssertionError("prefix trie: a node of the wrong size")
                 if self._node_of.get(child.pages[0]) is not child:
                     raise AssertionError("prefix trie: a reachable node is missing from the page index")
-                counts = [allocator.ref_count(page) for allocator, page in zip(self.allocators, child.pages)]
+                counts = [allocator.holders(page) for allocator, page in zip(self.allocators, child.pages)]
                 if min(counts) < 1 or len(set(counts)) != 1:
                     raise AssertionError(f"prefix trie: pages {child.pages} have reference counts {counts}")
-                if node is not self.root and counts[0] > self.allocators[0].ref_count(node.pages[0]):
+                if node is not self.root and counts[0] > self.allocators[0].holders(node.pages[0]):
                     raise AssertionError("prefix trie: a page is held by more requests than its parent")
                 seen += 1
                 unheld += counts[0] == 1

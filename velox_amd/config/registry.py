@@ -9,7 +9,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Any, Callable, Dict
 
-from .model_config import ConfigError, ModelConfig, architecture_name, read_config_json
+from .model_config import ConfigError, ModelConfig, read_config_json
 
 
 @dataclass(frozen=True)
@@ -20,10 +20,26 @@ class Architecture:
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
+_ARCHITECTURE_OF_MODEL_TYPE: Dict[str, str] = {}
 
 
-def register_architecture(name: str, read_config, make_spec) -> None:
+def register_architecture(name: str, read_config, make_spec, model_types=()) -> None:
+    """``name`` is what ``config.json`` holds in ``architectures[0]``; ``model_types`` are values of its ``model_type``
+    key that stand for this class when ``architectures`` is left out."""
     _ARCHITECTURES[name] = Architecture(name, read_config, make_spec)
+    for model_type in model_types:
+        _ARCHITECTURE_OF_MODEL_TYPE[model_type] = name
+
+
+def architecture_name(raw: Dict[str, Any]) -> str:
+    names = raw.get("architectures")
+    if names and isinstance(names, (list, tuple)) and isinstance(names[0], str):
+        return names[0]
+    _load_builtin()
+    model_type = raw.get("model_type")
+    if isinstance(model_type, str) and model_type in _ARCHITECTURE_OF_MODEL_TYPE:
+        return _ARCHITECTURE_OF_MODEL_TYPE[model_type]
+    raise ConfigError('config.json must name its model class in "architectures" (or a known "model_type")')
 
 
 def known_architectures():

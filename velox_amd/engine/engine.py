@@ -29,14 +29,14 @@ from ..weights import bind_from_checkpoint, bind_random
 from .batch import StepEntry
 from .request import FinishReason, Request
 from .runner import ModelRunner
-from .scheduler import Scheduler, SchedulerConfig
+from .scheduler import Portion, Scheduler, SchedulerConfig
 
 @dataclass
 class _Flight:
     """A step that has been queued on the device."""
 
     decode: List[Request]
-    prefill: List[Request]
+    prefill: List[Portion]
     sampled: List[Request]  # the requests whose rows were sampled, in row order
     tokens: Optional[torch.Tensor]  # int32 [len(sampled)] on the device
     landing: Optional[tuple] = None  # (pinned host tensor the tokens are copied to, event recorded behind the copy)
@@ -255,7 +255,7 @@ class Engine:
             self.stats["scheduler_ms"].append((time.perf_counter() - step_start) * 1000)
             if scheduled.is_empty():
                 return
-            flight = self._launch(scheduled.decode_batch, scheduled.prefill_batch)
+            flight = self._launch(scheduled.decodes, scheduled.portions)
         if self.config.decode_lookahead and flight.tokens is not None and not flight.prefill:
             alive = [(row, r) for row, r in enumerate(flight.sampled) if self._alive(r)]
             if alive and not any(r.sampling_params.has_penalties for _, r in alive):
@@ -270,7 +270,7 @@ class Engine:
     def _alive(request: Request) -> bool:
         return not request.finished and request.cache is not None
 
-    def _launch(self, decode: List[Request], prefill: List[Request], ids_on_device=None) -> "_Flight":
+    def _launch(self, decode: List[Request], prefill: List[Portion], ids_on_device=None) -> "_Flight":
         """Queues one step on the device: the forward over the batch and the sampler.  With ``ids_on_device`` the step
         before this one has not been finished on the host yet: every request is one position and one generated token
         further than its fields say."""
@@ -283,13 +283,10 @@ class Engine:
             token = 0 if ahead else request.all_token_ids[start]
             entries.append(StepEntry(request.cache, [token], start, [0]))
             sampled.append(request)
-        for request in prefill:
-            start = request.num_computed_tokens
-            chunk = request.current_chunk_size
-            tokens = request.all_token_ids[start:start + chunk]
-            completes = start + chunk >= len(request.all_token_ids)
-            entries.append(StepEntry(request.cache, tokens, start, [chunk - 1] if completes else []))
-            if completes:
+        for portion in prefill:
+            request, start, count = portion.request, portion.start, portion.count
+            entries.append(StepEntry(request.cache, request.all_token_ids[start:start + count], start, [count - 1] if portion.completes else []))
+            if portion.completes:
                 sampled.append(request)
 
         t0 = time.perf_counter()
@@ -333,16 +330,14 @@ class Engine:
         for request in flight.decode:
             if self._alive(request):
                 self.scheduler.advance(request, 1)
-        for request in flight.prefill:
-            if self._alive(request):
-                self.scheduler.advance(request, request.current_chunk_size)
-                request.refresh_status()
+        for portion in flight.prefill:
+            if self._alive(portion.request):
+                self.scheduler.advance(portion.request, portion.count)
         for request, token in zip(flight.sampled, tokens):
             if not self._alive(request):
                 continue  # stopped or aborted while this step was in flight
-            request.append_token(int(token))
-            request.refresh_status()
-            reason = request.should_stop(int(token), self.eos_token_ids)
+            request.record_token(int(token))
+            reason = request.stop_reason(int(token), self.eos_token_ids)
             if reason is not None:
                 request.finish(reason)
                 self.sampler.release(request.request_id)

@@ -35,7 +35,10 @@ class TraceError(RuntimeError):
 
 
 class Replayer:
-    def __init__(self, model_dir: str, dtype: str, max_tokens: int, block_size: int = 16, max_live: int = 8, device: str = "cuda", ops=None) -> None:
+    def __init__(self, model_dir: str, dtype: str, max_tokens: int, block_size: int = 16, max_live: int = 8, device: str = "cuda", ops=None,
+                 enable_graphs: bool = False) -> None:
+        """``max_live``: the most requests that are live at a time (and so in one step).  ``enable_graphs``: steps in which
+        every entry brings one token and wants it are replayed from captured HIP graphs, as the engine decodes."""
         self.device = torch.device(device)
         self.dtype = resolve_dtype(dtype)
         if ops is None:
@@ -54,7 +57,8 @@ class Replayer:
         bind_from_checkpoint(self.model, model_dir, self.dtype, self.device)
         ops.prepare(self.model, self.dtype)
         self.cache = CacheManager(self.model.cache_needs(), block_size, pages + 1, max_live, self.dtype, self.device, max_model_len=self.max_model_len)
-        self.runner = ModelRunner(self.model, self.cache, ops, self.dtype, self.device, max_num_tokens=max(capacity, 64), max_num_seqs=max_live, enable_graphs=False)
+        self.runner = ModelRunner(self.model, self.cache, ops, self.dtype, self.device, max_num_tokens=max(capacity, 64), max_num_seqs=max_live, enable_graphs=enable_graphs)
+        self.runner.capture_decode_graphs()
         self.vocab_size = self.model.spec.vocab_size
         self.live: Dict[str, List] = {}  # id -> [SequenceCache, tokens in the cache]
 

@@ -69,7 +69,8 @@ class ModelRunner:
             for name, numel in part.workspace_needs(ops, limits).items():
                 self.workspace.reserve(name, numel)
         self.workspace.fix()
-        self.enable_graphs = bool(enable_graphs) and self.device.type == "cuda"
+        # a model with a part that reads the host while it runs (``Part.graph_safe`` False) is never captured
+        self.enable_graphs = bool(enable_graphs) and self.device.type == "cuda" and model.allows_capture()
         self._graphs: Dict[int, Tuple[object, torch.Tensor, torch.Tensor]] = {}
         self._short_graphs: Dict[int, Tuple[object, torch.Tensor, torch.Tensor]] = {}  # the same buckets behind few keys
         self._graph_buffers: Dict[int, torch.Tensor] = {}

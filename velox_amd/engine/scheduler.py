@@ -32,6 +32,8 @@ from .request import FinishReason, Request, RequestStatus
 
 @dataclass
 class SchedulerConfig:
+    """The reference's knobs under the reference's names (``engine/scheduler.py:16-23``)."""
+
     max_num_seqs: int = 32
     max_num_batched_tokens: int = 2048
     max_prefill_chunk_size: int = 512
@@ -39,15 +41,49 @@ class SchedulerConfig:
     watermark: float = 0.01
 
 
+@dataclass(frozen=True)
+class Portion:
+    """``count`` tokens of ``request.all_token_ids`` from position ``start`` on: a piece of a prompt (or of a prompt plus
+    what was generated before a preemption) that one step computes."""
+
+    request: Request
+    start: int
+    count: int
+
+    @property
+    def completes(self) -> bool:
+        """Whether the request's tokens are all in the cache after this portion, so that its last row is sampled."""
+        return self.start + self.count >= len(self.request.all_token_ids)
+
+
 @dataclass
-class SchedulerOutput:
-    prefill_batch: List[Request] = field(default_factory=list)
-    decode_batch: List[Request] = field(default_factory=list)
+class StepPlan:
+    """What one step computes: a single token for each of ``decodes``, then ``portions``.  ``preempted`` lists who lost
+    their pages while the plan was made; none of them is in the plan."""
+
+    decodes: List[Request] = field(default_factory=list)
+    portions: List[Portion] = field(default_factory=list)
     preempted: List[Request] = field(default_factory=list)
-    num_batched_tokens: int = 0
+
+    @property
+    def num_tokens(self) -> int:
+        return len(self.decodes) + sum(p.count for p in self.portions)
 
     def is_empty(self) -> bool:
-        return not self.prefill_batch and not self.decode_batch
+        return not self.decodes and not self.portions
+
+    def requests(self) -> List[Request]:
+        return self.decodes + [p.request for p in self.portions]
+
+    def count_of(self, request: Request) -> int:
+        """Tokens of ``request`` in this step (0: it is not in it)."""
+        if any(r is request for r in self.decodes):
+            return 1
+        return next((p.count for p in self.portions if p.request is request), 0)
+
+    def withdraw(self, request: Request) -> None:
+        self.decodes = [r for r in self.decodes if r is not request]
+        self.portions = [p for p in self.portions if p.request is not request]
 
 
 class Scheduler:
@@ -55,48 +91,43 @@ class Scheduler:
         self.config = config or SchedulerConfig(**overrides)
         self.cache = cache
         self.config.max_model_len = min(self.config.max_model_len, cache.max_model_len)
-        self.waiting: Deque[Request] = deque()
-        self.running: List[Request] = []
+        self.waiting: Deque[Request] = deque()  # first come first served; a preempted request goes to the front
+        self.running: List[Request] = []  # in order of admission: the last one is the newest
         self.requests: Dict[str, Request] = {}
-        self._watermark_pages = max(1, int(cache.num_total_pages * self.config.watermark))
+        # admission leaves this many pages free, so that running requests can grow for a while without preempting
+        self._pages_held_back = max(1, int(cache.num_total_pages * self.config.watermark))
         self.num_preemptions = 0
         self.num_finished = 0
 
-    # -- queue --------------------------------------------------------------------------
+    # -- requests come and go -------------------------------------------------------------------
     def add_request(self, request: Request) -> None:
+        """Queues a request; refuses one that could not run to its end even alone (reference ``engine/scheduler.py:67-82``
+        checks the same two lengths; its pool capacity counts the reserved page, so a request of exactly that size would
+        wait for ever there)."""
         limit = self.config.max_model_len
-        if request.num_prompt_tokens >= limit:
-            raise ValueError(
-                f"prompt of {request.num_prompt_tokens} tokens does not fit in max_model_len={limit} "
-                "(at least one token must remain for generation)"
-            )
-        if request.num_prompt_tokens + request.sampling_params.max_tokens > limit:
-            raise ValueError(
-                f"prompt of {request.num_prompt_tokens} tokens plus max_tokens={request.sampling_params.max_tokens} "
-                f"exceeds max_model_len={limit}"
-            )
+        prompt, generated = request.num_prompt_tokens, request.sampling_params.max_tokens
+        if prompt >= limit:
+            raise ValueError(f"request {request.request_id!r}: a prompt of {prompt} tokens leaves no room to generate under max_model_len={limit}")
+        if prompt + generated > limit:
+            raise ValueError(f"request {request.request_id!r}: {prompt} prompt tokens + max_tokens={generated} is more than max_model_len={limit}")
         if request.request_id in self.requests:
-            raise ValueError(f"request id {request.request_id!r} is already queued")
+            raise ValueError(f"there is already a request with the id {request.request_id!r}")
         self.requests[request.request_id] = request
         self.waiting.append(request)
 
     def abort_request(self, request_id: str) -> bool:
-        request = self.requests.get(request_id)
+        """Ends a queued or running request now and gives back what it holds; False if there is none to end."""
+        request = self.requests.pop(request_id, None)
         if request is None or request.finished:
             return False
         request.finish(FinishReason.ABORT)
-        self._release(request)
-        try:
-            self.waiting.remove(request)
-        except ValueError:
-            pass
-        if request in self.running:
-            self.running.remove(request)
-        self.requests.pop(request_id, None)
+        self._give_back(request)
+        self.running = [r for r in self.running if r is not request]
+        self.waiting = deque(r for r in self.waiting if r is not request)
         return True
 
     def has_work(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self.waiting) or bool(self.running)
 
     @property
     def num_waiting(self) -> int:
@@ -106,51 +137,46 @@ class Scheduler:
     def num_running(self) -> int:
         return len(self.running)
 
-    # -- cache bookkeeping --------------------------------------------------------------
-    def _release(self, request: Request) -> None:
+    def _give_back(self, request: Request) -> None:
         if request.cache is not None:
             self.cache.free_sequence(request.cache)
             request.cache = None
 
-    def _preempt(self, request: Request, output: Optional[SchedulerOutput] = None) -> None:
-        if output is not None:
-            # a victim may already have been given its token of this step (the reference leaves it in the
-            # batch, engine/scheduler.py:241-247): it must not run without its pages
-            if request in output.decode_batch:
-                output.decode_batch.remove(request)
-            if request in output.prefill_batch:
-                output.prefill_batch.remove(request)
-            output.preempted.append(request)
-        self._release(request)
-        request.num_computed_tokens = 0
-        request.status = RequestStatus.PREEMPTED
-        request.num_preemptions += 1
+    def _drop_finished(self) -> None:
+        """Requests that ended since the last decision leave ``running``; their pages and slot go back only now, so a step
+        that was still in flight when they ended wrote into pages that were still theirs."""
+        ended = [r for r in self.running if r.finished]
+        if not ended:
+            return
+        for request in ended:
+            self._give_back(request)
+            self.requests.pop(request.request_id, None)
+        self.num_finished += len(ended)
+        self.running = [r for r in self.running if not r.finished]
+
+    def _preempt(self, victim: Request, plan: Optional[StepPlan] = None) -> None:
+        """Recompute preemption: everything the victim holds goes back, it waits at the front of the queue and is later
+        computed again from its first token, generated tokens included."""
+        if plan is not None:
+            # it may have been given a place in this very plan already (the reference leaves such a request in its
+            # batch, engine/scheduler.py:241-247): it must not run without pages
+            plan.withdraw(victim)
+            plan.preempted.append(victim)
+        self._give_back(victim)
+        victim.evicted()
+        self.running = [r for r in self.running if r is not victim]
+        self.waiting.appendleft(victim)
         self.num_preemptions += 1
-        if request in self.running:
-            self.running.remove(request)
-        self.waiting.appendleft(request)
 
-    def _make_room(self, request: Request, num_tokens: int, output: SchedulerOutput) -> bool:
-        while not self.cache.can_append(request.cache, request.num_computed_tokens, num_tokens):
-            if not self.running:
-                return False
-            victim = self.running[-1]  # always the newest, even when that is the caller
-            self._preempt(victim, output)
-            if victim is request:
-                return False
-        return True
-
-    # -- one scheduling decision --------------------------------------------------------
-    def schedule(self) -> SchedulerOutput:
-        output = SchedulerOutput()
-        self._reap_finished()
+    # -- one decision ---------------------------------------------------------------------------
+    def schedule(self) -> StepPlan:
+        self._drop_finished()
+        plan = StepPlan()
         budget = self.config.max_num_batched_tokens
-        self._schedule_decodes(output, budget)
-        budget -= len(output.decode_batch)
-        budget = self._schedule_running_prefills(output, budget)
-        self._admit(output, budget)
-        output.num_batched_tokens = len(output.decode_batch) + sum(r.current_chunk_size for r in output.prefill_batch)
-        return output
+        budget = self._place_decodes(plan, budget)
+        budget = self._place_running_prompts(plan, budget)
+        self._admit_waiting(plan, budget)
+        return plan
 
     def schedule_ahead(self, in_flight: List[Request]) -> Optional[List[Request]]:
         """The decode step after the one in flight, decided before that one's tokens are known (not in the reference,
@@ -163,8 +189,8 @@ class Scheduler:
         length limit is not reached by the token in flight), and every one finds its next page without preemption.
         Then the requests' tables are grown and the list comes back (order kept); otherwise None, and nothing has
         changed.  A request that stops on the token in flight has then been given a place it does not use: the caller
-        drops its row, and its pages go back when it is reaped."""
-        self._reap_finished()
+        drops its row, and its pages go back when it leaves ``running``."""
+        self._drop_finished()
         if self.waiting or not in_flight or len(self.running) != len(in_flight) or len(in_flight) > self.config.max_num_batched_tokens:
             return None
         chosen = set(id(r) for r in in_flight)
@@ -185,80 +211,70 @@ class Scheduler:
         for request in in_flight:
             if not self.cache.append(request.cache, request.num_computed_tokens + 1, 1):
                 raise RuntimeError("pages counted as free could not be taken")  # single-threaded: cannot happen
-            request.current_chunk_size = 1
         return list(in_flight)
 
-    def _reap_finished(self) -> None:
-        still = []
-        for request in self.running:
-            if request.finished:
-                self._release(request)
-                self.requests.pop(request.request_id, None)
-                self.num_finished += 1
-            else:
-                still.append(request)
-        self.running = still
-
-    def _schedule_decodes(self, output: SchedulerOutput, budget: int) -> None:
-        for request in list(self.running):
-            if request.status is not RequestStatus.RUNNING_DECODE or request not in self.running:
-                continue
-            if budget - len(output.decode_batch) <= 0:
-                break
-            if not self._make_room(request, 1, output) or not self.cache.append(request.cache, request.num_computed_tokens, 1):
-                if request in self.running:
-                    self._preempt(request, output)
-                continue
-            request.current_chunk_size = 1
-            output.decode_batch.append(request)
-
-    def _schedule_running_prefills(self, output: SchedulerOutput, budget: int) -> int:
-        oldest_seen = False
-        for request in list(self.running):
-            if request.status is not RequestStatus.RUNNING_PREFILL or request not in self.running:
-                continue
+    def _place_decodes(self, plan: StepPlan, budget: int) -> int:
+        """One token for every decoding request, oldest first.  When the token's page cannot be had, the newest running
+        request is preempted, as often as it takes; if that comes to be the request itself, it waits."""
+        for request in [r for r in self.running if r.status is RequestStatus.RUNNING_DECODE]:
             if budget <= 0:
                 break
-            oldest = not oldest_seen
-            oldest_seen = True
-            wanted = min(request.num_uncomputed_tokens, budget, self.config.max_prefill_chunk_size)
-            chunk = min(wanted, self.cache.max_new_tokens(request.cache, request.num_computed_tokens))
-            while chunk <= 0 and oldest and self.running and self.running[-1] is not request:
-                victim = self.running[-1]
-                self._preempt(victim, output)
-                chunk = min(wanted, self.cache.max_new_tokens(request.cache, request.num_computed_tokens))
-            if chunk <= 0 or not self.cache.append(request.cache, request.num_computed_tokens, chunk):
+            if request.cache is None:
+                continue  # preempted for an older request earlier in this loop
+            while request.cache is not None and not self.cache.can_append(request.cache, request.num_computed_tokens, 1):
+                self._preempt(self.running[-1], plan)
+            if request.cache is None:
                 continue
-            request.current_chunk_size = chunk
-            output.prefill_batch.append(request)
-            budget -= chunk
+            if not self.cache.append(request.cache, request.num_computed_tokens, 1):
+                self._preempt(request, plan)  # (beyond max_model_len: cannot happen to a request that add_request let in)
+                continue
+            plan.decodes.append(request)
+            budget -= 1
         return budget
 
-    def _admit(self, output: SchedulerOutput, budget: int) -> None:
-        while self.waiting and budget > 0:
-            if len(self.running) >= self.config.max_num_seqs:
+    def _portion_that_fits(self, request: Request, sequence, computed: int, budget: int, headroom_pages: Optional[int] = None) -> int:
+        wanted = min(len(request.all_token_ids) - computed, budget, self.config.max_prefill_chunk_size)
+        return min(wanted, self.cache.max_new_tokens(sequence, computed, headroom_pages=headroom_pages))
+
+    def _place_running_prompts(self, plan: StepPlan, budget: int) -> int:
+        """The next portion of every request whose prompt is under way, cut to the budget, the portion limit and the pages
+        that can be had.  Only the oldest of them may take pages from others, and only from requests newer than itself."""
+        under_way = [r for r in self.running if r.status is RequestStatus.RUNNING_PREFILL]
+        for index, request in enumerate(under_way):
+            if budget <= 0:
                 break
+            if request.cache is None:
+                continue  # preempted for the oldest one
+            count = self._portion_that_fits(request, request.cache, request.num_computed_tokens, budget)
+            while count <= 0 and index == 0 and self.running[-1] is not request:
+                self._preempt(self.running[-1], plan)
+                count = self._portion_that_fits(request, request.cache, request.num_computed_tokens, budget)
+            if count <= 0 or not self.cache.append(request.cache, request.num_computed_tokens, count):
+                continue
+            plan.portions.append(Portion(request, request.num_computed_tokens, count))
+            budget -= count
+        return budget
+
+    def _admit_waiting(self, plan: StepPlan, budget: int) -> None:
+        """Waiting requests start in their order of arrival while tokens, slots and pages (less those held back) are left.
+        The first one that does not fit ends admission for this step: nobody overtakes it."""
+        while self.waiting and budget > 0 and len(self.running) < self.config.max_num_seqs:
             request = self.waiting[0]
             sequence = self.cache.new_sequence()
             if sequence is None:
-                break
+                return
             # pages of a prefix that an earlier request has published are taken over, not computed (reference :268-277)
             cached = self.cache.match_prefix(sequence, request.all_token_ids)
-            wanted = min(len(request.all_token_ids) - cached, budget, self.config.max_prefill_chunk_size)
-            headroom = self.cache.num_available_pages() - self._watermark_pages
-            chunk = min(wanted, self.cache.max_new_tokens(sequence, cached, headroom_pages=headroom))
-            if chunk <= 0 or not self.cache.append(sequence, cached, chunk):
-                self.cache.free_sequence(sequence)
-                break
+            headroom = self.cache.num_available_pages() - self._pages_held_back
+            count = self._portion_that_fits(request, sequence, cached, budget, headroom_pages=headroom)
+            if count <= 0 or not self.cache.append(sequence, cached, count):
+                self.cache.free_sequence(sequence)  # (the matched pages too)
+                return
             self.waiting.popleft()
-            request.cache = sequence
-            request.num_computed_tokens = cached
-            request.num_cached_tokens = cached
-            request.status = RequestStatus.RUNNING_PREFILL
-            request.current_chunk_size = chunk
+            request.admitted(sequence, cached)
             self.running.append(request)
-            output.prefill_batch.append(request)
-            budget -= chunk
+            plan.portions.append(Portion(request, cached, count))
+            budget -= count
 
     # -- after the forward --------------------------------------------------------------
     def advance(self, request: Request, num_tokens: int) -> None:

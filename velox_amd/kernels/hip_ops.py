@@ -42,6 +42,37 @@ def _ptr(t: Optional[torch.Tensor]):
     return _P(0) if t is None else _P(t.data_ptr())
 
 
+class PreparedWeight:
+    """A ``[N, K]`` weight together with the copies of it that the decode-sized products read (``HipOps.prepare_weight``).
+    The part that owns the weight owns this; it stands wherever the weight stands in ``linear``, ``linear_silu_mul`` and
+    ``qkv_rope_write``.  ``copies``: 1 and 2 = ``pack_rows`` of the weight as one matrix or as two stacked ones,
+    ``"rotary"`` = the copy in the row order of ``qkv_rope_write``."""
+
+    def __init__(self, weight: torch.Tensor) -> None:
+        self.weight = weight
+        self.version = weight._version
+        self.copies: Dict[object, torch.Tensor] = {}
+
+    @property
+    def shape(self):
+        return self.weight.shape
+
+    @property
+    def dtype(self):
+        return self.weight.dtype
+
+    def copy(self, key=1) -> Optional[torch.Tensor]:
+        if self.weight._version != self.version:
+            raise KernelError("a weight was changed in place after the kernels prepared their copies of it; prepare it again")
+        return self.copies.get(key)
+
+
+def _weight_of(weight) -> Tuple[torch.Tensor, Optional[PreparedWeight]]:
+    if isinstance(weight, PreparedWeight):
+        return weight.weight, weight
+    return weight, None
+
+
 class HipOps:
     name = "hip-gfx950"
 
@@ -118,20 +149,21 @@ class HipOps:
         for part in model.all_parts():
             part.prepare_kernels(self)
 
-    def register_weight(self, weight: torch.Tensor, stacked: int = 1, rotary_heads: Optional[Tuple[int, int, int]] = None) -> None:
-        """Keeps a second copy of a bfloat16 ``[N, K]`` weight in the order the skinny kernels' lanes read it (see
+    def prepare_weight(self, weight: torch.Tensor, stacked: int = 1, rotary_heads: Optional[Tuple[int, int, int]] = None,
+                       handle: Optional[PreparedWeight] = None) -> Optional[PreparedWeight]:
+        """A second copy of a bfloat16 ``[N, K]`` weight in the order the skinny kernels' lanes read it (see
         ``pack_rows``): decode-sized products then stream contiguous kilobytes.  ``stacked`` = 2 marks ``[Wgate; Wup]``;
         ``rotary_heads = (heads, kv_heads, head_dim)`` marks ``[Wq; Wk; Wv]`` whose product is followed by a rotation of
         whole heads and gets a further copy for ``qkv_rope_write``.  Each copy costs the weight's size again in memory;
-        ``pack_decode_weights = False`` turns them off.  The copies hang on the tensor object itself, so they live
-        exactly as long as the weight and are found only through that object."""
+        ``pack_decode_weights = False`` turns them off.  Returns what the caller keeps and passes in the weight's place
+        (``handle``: an earlier result for the same weight, which is extended), or None when the kernels read this weight
+        as it is."""
         if (not self.pack_decode_weights or weight is None or weight.dtype != torch.bfloat16 or weight.dim() != 2
                 or weight.shape[1] % 64 != 0 or weight.shape[0] % stacked != 0 or weight.device != self.device):
-            return
-        copies = getattr(weight, "_velox_packed", None)
-        if copies is None or copies["version"] != weight._version:
-            copies = {"version": weight._version}
-            weight._velox_packed = copies
+            return handle
+        if handle is None or handle.weight is not weight or handle.version != weight._version:
+            handle = PreparedWeight(weight)
+        copies = handle.copies
         if stacked not in copies:
             per_matrix = weight.shape[0] // stacked
             whole_tiles = [c for key, c in copies.items() if key in (1, 2)] if per_matrix % 16 == 0 else []
@@ -141,6 +173,7 @@ class HipOps:
             heads, kv_heads, head_dim = rotary_heads
             if head_dim % 32 == 0 and weight.shape[0] == (heads + 2 * kv_heads) * head_dim:
                 copies["rotary"] = self.pack_rows(weight[self.rotary_row_order(heads, kv_heads, head_dim, weight.device)])
+        return handle
 
     @staticmethod
     def rotary_row_order(heads: int, kv_heads: int, head_dim: int, device) -> torch.Tensor:
@@ -151,13 +184,6 @@ class HipOps:
         rotary = (torch.arange(heads + kv_heads, device=device).view(-1, 1) * head_dim + inside.reshape(1, -1)).reshape(-1)
         values = torch.arange((heads + kv_heads) * head_dim, (heads + 2 * kv_heads) * head_dim, device=device)
         return torch.cat([rotary, values])
-
-    @staticmethod
-    def packed_weight(weight: torch.Tensor, stacked=1) -> Optional[torch.Tensor]:
-        copies = getattr(weight, "_velox_packed", None)
-        if copies is None or copies["version"] != weight._version:
-            return None
-        return copies.get(stacked)
 
     def library_serves(self, m: int, n: int, k: int) -> bool:
         """Whether ``linear`` hands ``x[m, k] @ w[n, k]^T`` in bfloat16 to the matrix library, and the product is large
@@ -299,10 +325,11 @@ class HipOps:
         come back as a ``DeferredNorm``: the product has then been added to ``residual_norm.residual`` and multiplied
         with the weight of ``residual_norm.norm`` (decode-sized bfloat16 products whose weight is registered).  ``x`` may
         be a ``DeferredNorm``."""
+        weight, prepared = _weight_of(weight)
+        packed = prepared.copy(1) if prepared is not None else None
         deferred = x if isinstance(x, DeferredNorm) else None
         if deferred is not None:
             x = deferred.x
-            packed = self.packed_weight(weight)
             if not (self.use_skinny_gemm and packed is not None and x.shape[0] <= 16 and x.shape[1] % 64 == 0 and weight.dtype == torch.bfloat16):
                 x, deferred = self.materialize(deferred), None
         self._check("x", x, align=16)
@@ -314,17 +341,17 @@ class HipOps:
         if bias is not None:
             self._check("bias", bias, torch.float32, (n,))
         if deferred is not None:
-            return self.skinny_gemm(x, weight, bias, out_dtype, packed=self.packed_weight(weight), row_scale=deferred, x_packed=self._packed_rows_of(x, k))
+            return self.skinny_gemm(x, weight, bias, out_dtype, packed=packed, row_scale=deferred, x_packed=self._packed_rows_of(x, k))
         if residual_norm is not None and bias is None:
-            fused = self._linear_into_residual(x, weight, residual_norm)
+            fused = self._linear_into_residual(x, weight, residual_norm, packed=packed)
             if fused is not None:
                 return fused
         if (partials_ok and bias is None and self.use_skinny_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
                 and 16 < m <= 64 and k % 64 == 0 and n <= 8192 and n % 4 == 0):
-            return self.skinny_gemm_splitk(x, weight, packed=self.packed_weight(weight))
+            return self.skinny_gemm_splitk(x, weight, packed=packed)
         skinny_rows = 16 if n > 8192 else 32  # measured on MI355X: beyond this the library's kernels stream faster
         if self.use_skinny_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and m <= skinny_rows and k % 64 == 0:
-            return self.skinny_gemm(x, weight, bias, out_dtype, packed=self.packed_weight(weight), x_packed=self._packed_rows_of(x, k))
+            return self.skinny_gemm(x, weight, bias, out_dtype, packed=packed, x_packed=self._packed_rows_of(x, k))
         if self.use_library_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and bias is None:
             if out_dtype == torch.bfloat16:
                 return torch.nn.functional.linear(x, weight)
@@ -337,11 +364,14 @@ class HipOps:
                     self._mm_out_dtype_ok = False
         return self.gemm_fma(x, weight, bias, out_dtype)
 
-    def _linear_into_residual(self, x: torch.Tensor, weight: torch.Tensor, sink: ResidualSink, waves: Optional[int] = None, row_tiles: Optional[int] = None) -> Optional[DeferredNorm]:
+    def _linear_into_residual(self, x: torch.Tensor, weight: torch.Tensor, sink: ResidualSink, waves: Optional[int] = None, row_tiles: Optional[int] = None,
+                              packed: Optional[torch.Tensor] = None) -> Optional[DeferredNorm]:
         """``sink.residual += x @ weight^T`` with the first half of ``sink.norm`` in the same kernel, if this product
         qualifies (bfloat16, at most 16 rows, registered weight, a norm that can be split); None otherwise."""
         form = sink.norm.deferred_form()
-        packed = self.packed_weight(weight)
+        weight, prepared = _weight_of(weight)
+        if prepared is not None and packed is None:
+            packed = prepared.copy(1)
         m, k = x.shape
         n = weight.shape[0]
         residual = sink.residual
@@ -427,6 +457,10 @@ class HipOps:
         is the product followed by the SiLU kernel.  ``waves`` and ``pairs`` override the launch shape the wrapper would
         pick (up to 16 rows: waves per workgroup and gate/up tile pairs per wave; 17 .. 64 rows: ``pairs`` = tile pairs per
         workgroup)."""
+        operand = gate_up_weight  # (as given: handed on to ``linear`` when nothing here applies)
+        gate_up_weight, prepared = _weight_of(gate_up_weight)
+        if packed is None and prepared is not None:
+            packed = prepared.copy(2)
         deferred = x if isinstance(x, DeferredNorm) else None
         if deferred is not None:
             x = deferred.x
@@ -436,9 +470,8 @@ class HipOps:
                  and m <= 16 and k % 64 == 0 and two_n % 2 == 0 and x.dim() == 2 and gate_up_weight.shape[1] == k)
         if (not fused and deferred is None and self.use_skinny_gemm and x.dim() == 2 and 16 < m <= 64 and k % 64 == 0 and two_n % 2 == 0
                 and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16 and out_dtype == torch.bfloat16
-                and gate_up_weight.shape[1] == k and (packed is not None or self.packed_weight(gate_up_weight, 2) is not None)):
+                and gate_up_weight.shape[1] == k and packed is not None):
             # 17 .. 64 rows: the kernel that streams the packed weight once with the activation as its epilogue
-            packed = packed if packed is not None else self.packed_weight(gate_up_weight, 2)
             n = two_n // 2
             if packed.dtype != torch.bfloat16 or packed.numel() != 2 * ((n + 15) // 16) * 16 * k:
                 raise KernelError("linear_silu_mul: the packed weight does not match N and K")
@@ -453,9 +486,7 @@ class HipOps:
                            "skinny_glu_rows")
             return out
         if not fused:
-            return self.silu_mul(self.linear(deferred if deferred is not None else x, gate_up_weight, None, out_dtype))
-        if packed is None:
-            packed = self.packed_weight(gate_up_weight, 2)
+            return self.silu_mul(self.linear(deferred if deferred is not None else x, operand, None, out_dtype))
         if deferred is not None and packed is None:  # only the kernels of a registered weight scale rows
             x, deferred = self.materialize(deferred), None
         self._check("x", x, align=16)
@@ -578,13 +609,15 @@ class HipOps:
                        block_size, write_kv=True, waves: Optional[int] = None, fused: Optional[bool] = None) -> torch.Tensor:
         """Projects ``x`` with ``weight = [Wq; Wk; Wv]``, adds ``bias``, rotates queries and keys and writes keys and values
         into the cache.  Returns a tensor whose first ``num_heads * head_dim`` columns are the rotated queries (it may be
-        wider).  Decode-sized bfloat16 batches run as one kernel when ``register_weight(weight, rotary_heads=...)`` has
-        prepared the weight; everything else is the product followed by ``rope_kv_write``."""
+        wider).  Decode-sized bfloat16 batches run as one kernel when ``weight`` is what ``prepare_weight(w, rotary_heads=...)``
+        returned; everything else is the product followed by ``rope_kv_write``."""
+        operand = weight
+        weight, prepared = _weight_of(weight)
         deferred = x if isinstance(x, DeferredNorm) else None
         if deferred is not None:
             x = deferred.x
         m, k = x.shape
-        packed = self.packed_weight(weight, "rotary")
+        packed = prepared.copy("rotary") if prepared is not None else None
         can_fuse = (self.use_skinny_gemm and packed is not None and write_kv and x.dtype == torch.bfloat16 and m <= 16 and k % 64 == 0
                     and cos is not None and 2 * cos.shape[1] == head_dim and head_dim % 32 == 0 and k_cache.dtype == torch.bfloat16)
         if fused is None:
@@ -598,10 +631,10 @@ class HipOps:
                     and (cos is None or 2 * cos.shape[1] == head_dim)):
                 # 17 .. 64 rows: the split-K kernel streams the weight faster than the library's choice (measured on
                 # MI355X: 15 us against 21 for 4608 x 3584 at 64 rows), and the rotation adds its partial sums
-                partial = self.skinny_gemm_splitk(x, weight, packed=self.packed_weight(weight))
+                partial = self.skinny_gemm_splitk(x, weight, packed=prepared.copy(1) if prepared is not None else None)
                 return self.rope_kv_write_partial(partial, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache,
                                                   block_size, write_kv=write_kv, bias=bias)
-            qkv = self.linear(deferred if deferred is not None else x, weight, None, x.dtype)
+            qkv = self.linear(deferred if deferred is not None else x, operand, None, x.dtype)
             self.rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size,
                                write_kv=write_kv, bias=bias)
             return qkv

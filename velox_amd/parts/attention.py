@@ -78,8 +78,8 @@ class AttentionMixer(Mixer):
     def prepare_kernels(self, ops) -> None:
         cos, _ = self._rotary_tables()
         whole_heads = cos is not None and 2 * cos.shape[1] == self.head_dim
-        ops.register_weight(self.qkv_weight, rotary_heads=(self.num_heads, self.num_kv_heads, self.head_dim) if whole_heads else None)
-        ops.register_weight(self.o_weight)
+        self.prepare_weight(ops, "qkv_weight", rotary_heads=(self.num_heads, self.num_kv_heads, self.head_dim) if whole_heads else None)
+        self.prepare_weight(ops, "o_weight")
 
     def workspace_needs(self, ops, limits):
         sizes = getattr(ops, "attention_scratch_elems", None)
@@ -97,7 +97,7 @@ class AttentionMixer(Mixer):
         meta = cache.batch
         # product, bias (added in float32), rotation and the write into the cache: one kernel for decode-sized batches
         q = ops.qkv_rope_write(
-            x, self.qkv_weight, self.qkv_bias_vec if self.qkv_bias else None,
+            x, self.operand("qkv_weight"), self.qkv_bias_vec if self.qkv_bias else None,
             self.num_heads, self.num_kv_heads, self.head_dim,
             ctx.positions, cos, sin,
             meta.slot_mapping, cache.k, cache.v, cache.block_size,
@@ -111,7 +111,7 @@ class AttentionMixer(Mixer):
             ctx.all_decode, ctx.workspace,
             decode_prefix=getattr(ctx, "decode_prefix", 0), portions_max_kv_len=getattr(meta, "max_kv_len_of_portions", 0) or None,
         )
-        return ops.linear(attn, self.o_weight, None, ctx.dtype, partials_ok=True, residual_norm=sink)
+        return ops.linear(attn, self.operand("o_weight"), None, ctx.dtype, partials_ok=True, residual_norm=sink)
 
 
 register_part("mixer", "attention", AttentionMixer)

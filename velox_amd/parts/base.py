@@ -2,7 +2,7 @@
 
 A *part* owns tensors (declared as :class:`Param`) and one piece of arithmetic.
 It is given its sizes and constants at construction and never learns which
-model it sits in.  Four kinds exist, each with a registry from a kind name to a
+model it sits in.  Six families exist, each with a registry from a kind name to a
 class so that an architecture (or a test) can add its own:
 
 ``Mixer``
@@ -17,7 +17,13 @@ class so that an architecture (or a test) can add its own:
     either changes the embeddings (absolute encodings) or hands rotary tables to
     the mixer, which fuses the rotation into its cache write.
 
-``Block`` arranges one mixer, one feed-forward and their norms.
+``Embedding``
+    token ids -> the residual stream, float32 ``[T, H]``.
+``OutputHead``
+    normalised rows -> float32 logits ``[R, vocab]``.
+
+``Block`` arranges one mixer, one feed-forward and their norms; arrangements have a
+registry of their own (``register_arrangement``).
 """
 from __future__ import annotations
 
@@ -66,8 +72,14 @@ def fused_rows(names: Tuple[str, ...], shapes: Tuple[Tuple[int, ...], ...], role
 class Part:
     """Base of every part: a prefix in the checkpoint's name space plus declared tensors."""
 
+    # Whether ``forward`` may be recorded into a HIP graph and replayed: it then reads nothing on the host that changes
+    # from step to step (no ``.tolist()``, ``.item()`` or Python loop over a step's values) and launches the same kernels
+    # on the same addresses every time.  One part that says False keeps the whole model's decode steps uncaptured.
+    graph_safe = True
+
     def __init__(self, prefix: str = "") -> None:
         self.prefix = prefix
+        self._prepared: Dict[str, object] = {}
 
     def params(self) -> Dict[str, Param]:
         """attribute name -> Param; the loader sets ``self.<attribute>`` to the bound tensor."""
@@ -80,8 +92,37 @@ class Part:
         """Called once after the weights are bound (build tables, derived tensors)."""
 
     def prepare_kernels(self, ops) -> None:
-        """Called once with the kernels' handle: a part may register the weights its decode-sized products read
-        (``ops.register_weight``).  Nothing has to be done here."""
+        """Called once with the kernels' handle, after the weights are bound: a part hands the weights that its
+        decode-sized products read to ``self.prepare_weight(ops, "<attribute>", ...)`` and from then on passes
+        ``self.operand("<attribute>")`` where it passed the tensor.  Nothing has to be done here."""
+
+    def prepare_weight(self, ops, attr: str, **options) -> None:
+        """Lets the kernels make what they want of ``self.<attr>`` (copies in the order their lanes read, say); the
+        part owns the result.  ``options`` are ``ops.prepare_weight``'s; several calls for one attribute add up."""
+        prepare = getattr(ops, "prepare_weight", None)
+        tensor = getattr(self, attr, None)
+        if prepare is None or tensor is None:
+            return
+        known = self._prepared.get(attr)
+        if known is not None and getattr(known, "weight", None) is not tensor:
+            known = None  # bound again since: start over
+        handle = prepare(tensor, handle=known, **options)
+        if handle is not None:
+            self._prepared[attr] = handle
+        else:
+            self._prepared.pop(attr, None)
+
+    def operand(self, attr: str):
+        """``self.<attr>`` as the kernels take it: what ``prepare_weight`` made of it, or the tensor itself.  A tensor
+        that was bound again behind a prepared one is an error, not a silent fall to the slow path."""
+        tensor = getattr(self, attr)
+        handle = self._prepared.get(attr)
+        if handle is None:
+            return tensor
+        if handle.weight is not tensor:
+            raise RuntimeError(f"{type(self).__name__}.{attr} ({self.prefix!r}) was bound again after the kernels prepared it; "
+                               "call ops.prepare(model, dtype) again")
+        return handle
 
     def workspace_needs(self, ops, limits) -> Dict[str, int]:
         """Scratch this part may ask ``ctx.workspace`` for: buffer name -> the most float32 elements, for any step within
@@ -197,6 +238,40 @@ class PositionEncoding(Part):
         return None
 
 
+class Embedding(Part):
+    def forward(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
+        """int32 ``[T]`` -> the residual stream before the first block, float32 ``[T, H]`` (a fresh tensor: blocks
+        update it in place)."""
+        raise NotImplementedError
+
+
+class OutputHead(Part):
+    def forward(self, hidden_rows: torch.Tensor, ctx) -> torch.Tensor:
+        """``[R, H]`` in the run dtype (the final norm's output on the wanted rows) -> float32 logits ``[R, vocab]``."""
+        raise NotImplementedError
+
+
+class Block(Part):
+    """One schedule entry's arithmetic: an arrangement of a mixer, a feed-forward and their norms around the residual.
+
+    The residual stream is a float32 ``[T, H]`` tensor that blocks update in place.  What a block's last sub-layer
+    produced may be handed on instead of added: ``forward`` takes the previous block's ``pending`` and returns its own
+    (None when it has added everything itself), and whoever normalises next adds it inside the norm's kernel."""
+
+    mixer: "Mixer"
+
+    def input_norm(self) -> Optional["Norm"]:
+        """The norm that reads this block's input first, if the block begins with one that the block before may hand its
+        output to (``next_norm``); None if it does not (then it is given a plain ``pending`` and no sink is offered)."""
+        return None
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def forward(self, residual: torch.Tensor, pending, ctx, cache, owns_cache: bool, next_norm: Optional["Norm"] = None):
+        raise NotImplementedError
+
+
 # ----------------------------------------------------------------------------------------
 # registries of kinds
 # ----------------------------------------------------------------------------------------
@@ -204,12 +279,21 @@ _MIXERS: Dict[str, Callable[..., Mixer]] = {}
 _FEED_FORWARDS: Dict[str, Callable[..., FeedForward]] = {}
 _NORMS: Dict[str, Callable[..., Norm]] = {}
 _POSITIONS: Dict[str, Callable[..., PositionEncoding]] = {}
-_TABLES = {"mixer": _MIXERS, "feed_forward": _FEED_FORWARDS, "norm": _NORMS, "position": _POSITIONS}
+_EMBEDDINGS: Dict[str, Callable[..., Embedding]] = {}
+_HEADS: Dict[str, Callable[..., OutputHead]] = {}
+_ARRANGEMENTS: Dict[str, Callable[..., Block]] = {}
+_TABLES = {"mixer": _MIXERS, "feed_forward": _FEED_FORWARDS, "norm": _NORMS, "position": _POSITIONS, "embedding": _EMBEDDINGS, "head": _HEADS,
+           "arrangement": _ARRANGEMENTS}
 
 
 def register_part(family: str, kind: str, factory: Callable[..., Part]) -> None:
     table = _TABLES[family]
     table[kind] = factory
+
+
+def register_arrangement(kind: str, factory: Callable[..., Block]) -> None:
+    """``factory(prefix, mixer, feed_forward, mixer_norm, ff_norm) -> Block``."""
+    register_part("arrangement", kind, factory)
 
 
 def make_part(family: str, kind: str, **kwargs) -> Part:

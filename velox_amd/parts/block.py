@@ -11,10 +11,10 @@ from typing import Optional, Tuple
 
 import torch
 
-from .base import FeedForward, Mixer, Norm, Part, ResidualSink
+from .base import Block, FeedForward, Mixer, Norm, Part, ResidualSink, register_arrangement
 
 
-class PreNormBlock(Part):
+class PreNormBlock(Block):
     def __init__(self, prefix: str, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, ff_norm: Norm) -> None:
         super().__init__(prefix)
         self.mixer = mixer
@@ -24,6 +24,9 @@ class PreNormBlock(Part):
 
     def children(self) -> Tuple[Part, ...]:
         return (self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward)
+
+    def input_norm(self) -> Optional[Norm]:
+        return self.mixer_norm
 
     def forward(self, residual: torch.Tensor, pending, ctx, cache, owns_cache: bool, next_norm: Optional[Norm] = None):
         """``next_norm``: the norm that will read this block's output (the next block's first norm), if the caller
@@ -43,4 +46,4 @@ class PreNormBlock(Part):
         return self.feed_forward.forward(normed, ctx)
 
 
-BLOCK_ARRANGEMENTS = {"pre_norm": PreNormBlock}
+register_arrangement("pre_norm", PreNormBlock)

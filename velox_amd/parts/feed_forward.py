@@ -33,16 +33,16 @@ class GatedMLP(FeedForward):
         }
 
     def prepare_kernels(self, ops) -> None:
-        ops.register_weight(self.gate_up_weight, stacked=2)
-        ops.register_weight(self.down_weight)
+        self.prepare_weight(ops, "gate_up_weight", stacked=2)
+        self.prepare_weight(ops, "down_weight")
 
     accepts_sink = True  # its last product may add itself to the residual (ResidualSink)
     accepts_deferred = True  # its first product can read a DeferredNorm
 
     def forward(self, x, ctx, sink=None):
         ops = ctx.ops
-        act = ops.linear_silu_mul(x, self.gate_up_weight, ctx.dtype)
-        return ops.linear(act, self.down_weight, None, ctx.dtype, partials_ok=True, residual_norm=sink)
+        act = ops.linear_silu_mul(x, self.operand("gate_up_weight"), ctx.dtype)
+        return ops.linear(act, self.operand("down_weight"), None, ctx.dtype, partials_ok=True, residual_norm=sink)
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)

@@ -19,8 +19,8 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
-from .base import Param, Part, PartSpec, make_part, single
-from .block import BLOCK_ARRANGEMENTS
+from . import block as _block  # noqa: F401  (registers the built-in arrangement)
+from .base import Embedding, OutputHead, Param, Part, PartSpec, make_part, register_part, single
 
 
 @dataclass(frozen=True)
@@ -32,10 +32,11 @@ class LayerSpec:
     ff_norm: PartSpec
     position: Optional[str] = None  # key into ModelSpec.positions handed to the mixer
     arrangement: str = "pre_norm"
-    mixer_prefix: str = "self_attn."
-    feed_forward_prefix: str = "mlp."
-    mixer_norm_prefix: str = "input_layernorm."
-    ff_norm_prefix: str = "post_attention_layernorm."
+    # where each part's tensors stand in the checkpoint, below the layer's prefix (an architecture sets its own names)
+    mixer_prefix: str = "mixer."
+    feed_forward_prefix: str = "feed_forward."
+    mixer_norm_prefix: str = "mixer_norm."
+    ff_norm_prefix: str = "feed_forward_norm."
 
 
 @dataclass(frozen=True)
@@ -55,10 +56,16 @@ class ModelSpec:
     positions: Dict[str, PartSpec] = field(default_factory=dict)
     embedding_position: Optional[str] = None  # a position encoding applied to the embeddings
     tie_head: bool = False
-    embed_name: str = "model.embed_tokens.weight"
-    head_name: str = "lm_head.weight"
-    final_norm_prefix: str = "model.norm."
+    embed_name: str = "embedding.weight"
+    head_name: str = "head.weight"
+    final_norm_prefix: str = "final_norm."
     eos_token_ids: Tuple[int, ...] = ()
+    # The parts at the two ends, chosen like every other part.  None = the plain ones: a table that is looked up
+    # (``embed_name``) and a product without bias (``head_name``, or the table itself with ``tie_head``).  A kind
+    # registered under "embedding" / "head" gets its ``args`` plus ``name``, ``vocab_size``, ``hidden_size`` and, for a
+    # head, ``tied_to`` (the table's checkpoint name or None).
+    embedding: Optional[PartSpec] = None
+    head: Optional[PartSpec] = None
 
     def validate(self) -> None:
         if not self.layers:
@@ -73,7 +80,9 @@ class ModelSpec:
                     raise ValueError(f"schedule[{index}].cache_from must name an entry that owns its cache")
 
 
-class Embedding(Part):
+class TableEmbedding(Embedding):
+    """``h[t] = E[ids[t]]``, no scaling (reference ``src/transformer.py:27,44``)."""
+
     def __init__(self, name: str, vocab_size: int, hidden_size: int) -> None:
         super().__init__("")
         self.name = name
@@ -88,11 +97,11 @@ class Embedding(Part):
         return ctx.ops.embed(token_ids, self.table)
 
 
-class OutputHead(Part):
+class LinearHead(OutputHead):
     """``logits = hidden @ W^T`` without bias; ``W`` is the embedding table when tied
     (reference ``src/transformer.py:60-62``).  Logits are returned in float32."""
 
-    def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str]) -> None:
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str] = None) -> None:
         super().__init__("")
         self.name = name
         self.vocab_size = vocab_size
@@ -107,10 +116,14 @@ class OutputHead(Part):
         return {"weight": Param(base.shape, base.sources, base.source_shapes, base.role, base.init, alias_of=self.tied_to)}
 
     def prepare_kernels(self, ops) -> None:
-        ops.register_weight(self.weight)
+        self.prepare_weight(ops, "weight")
 
     def forward(self, hidden_rows: torch.Tensor, ctx) -> torch.Tensor:
-        return ctx.ops.linear(hidden_rows, self.weight, None, torch.float32)
+        return ctx.ops.linear(hidden_rows, self.operand("weight"), None, torch.float32)
+
+
+register_part("embedding", "table", TableEmbedding)
+register_part("head", "linear", LinearHead)
 
 
 class DecoderModel(Part):
@@ -119,7 +132,8 @@ class DecoderModel(Part):
         spec.validate()
         self.spec = spec
         self.positions = {key: make_part("position", ps.kind, **ps.kwargs()) for key, ps in spec.positions.items()}
-        self.embedding = Embedding(spec.embed_name, spec.vocab_size, spec.hidden_size)
+        embedding = spec.embedding or PartSpec.of("table")
+        self.embedding = make_part("embedding", embedding.kind, name=spec.embed_name, vocab_size=spec.vocab_size, hidden_size=spec.hidden_size, **embedding.kwargs())
         self.blocks = []
         for layer in spec.layers:
             mixer_kwargs = layer.mixer.kwargs()
@@ -129,9 +143,11 @@ class DecoderModel(Part):
             ff = make_part("feed_forward", layer.feed_forward.kind, prefix=layer.prefix + layer.feed_forward_prefix, **layer.feed_forward.kwargs())
             norm1 = make_part("norm", layer.mixer_norm.kind, prefix=layer.prefix + layer.mixer_norm_prefix, **layer.mixer_norm.kwargs())
             norm2 = make_part("norm", layer.ff_norm.kind, prefix=layer.prefix + layer.ff_norm_prefix, **layer.ff_norm.kwargs())
-            self.blocks.append(BLOCK_ARRANGEMENTS[layer.arrangement](layer.prefix, mixer, ff, norm1, norm2))
+            self.blocks.append(make_part("arrangement", layer.arrangement, prefix=layer.prefix, mixer=mixer, feed_forward=ff, mixer_norm=norm1, ff_norm=norm2))
         self.final_norm = make_part("norm", spec.final_norm.kind, prefix=spec.final_norm_prefix, **spec.final_norm.kwargs())
-        self.head = OutputHead(spec.head_name, spec.vocab_size, spec.hidden_size, spec.embed_name if spec.tie_head else None)
+        head = spec.head or PartSpec.of("linear")
+        self.head = make_part("head", head.kind, name=spec.head_name, vocab_size=spec.vocab_size, hidden_size=spec.hidden_size,
+                              tied_to=spec.embed_name if spec.tie_head else None, **head.kwargs())
         self.schedule = list(spec.schedule)
 
     # -- structure ----------------------------------------------------------------------
@@ -150,11 +166,15 @@ class DecoderModel(Part):
             walk(child)
         return out
 
+    def allows_capture(self) -> bool:
+        """Whether every part allows its ``forward`` to be captured into a HIP graph (``Part.graph_safe``)."""
+        return all(part.graph_safe for part in self.all_parts())
+
     def cache_needs(self) -> List[object]:
         """One entry per schedule entry: the mixer's need, or None when it reads another entry's cache."""
         needs = []
         for entry in self.schedule:
-            need = self.blocks[entry.layer].mixer.cache_need()
+            need = self.blocks[entry.layer].cache_need()
             needs.append(need if entry.cache_from is None else None)
         return needs
 
@@ -174,9 +194,9 @@ class DecoderModel(Part):
             entry = self.schedule[index]
             owner = index if entry.cache_from is None else entry.cache_from
             cache = ctx.cache_view(owner)
-            # the norm that reads this block's output: the next entry's first norm (the final norm works on chosen rows
-            # and takes its input as it is)
-            following = self.blocks[self.schedule[index + 1].layer].mixer_norm if index + 1 < len(self.schedule) else None
+            # the norm that reads this block's output: the one the next entry's block begins with, if it begins with one
+            # (the final norm works on chosen rows and takes its input as it is)
+            following = self.blocks[self.schedule[index + 1].layer].input_norm() if index + 1 < len(self.schedule) else None
             pending = self.blocks[entry.layer].forward(residual, pending, ctx, cache, entry.cache_from is None, next_norm=following)
         return pending
 
