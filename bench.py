@@ -8,7 +8,13 @@ sampling, the host's read of the sampled tokens).  The default run has the layer
 Qwen2.5-7B with random weights N(0, 0.02), a batch of 8 and a context of 4096 tokens: the
 requests are prefilled through the engine so that they reach the context length at the last
 timed step.  ``value`` is decoded tokens per second.  The same line carries the prefill of one
-2,048-token prompt, the decode step's share of the HBM roofline, and decode at batch 1 and 64.
+2,048-token prompt (mean of the repeats), the decode step's share of the HBM roofline, and under
+``points``: decode at batch 1 and 64 at the same context, a sampled decode step (temperature 0.8,
+top-p 0.9) at batch 64, and the reference's own decode workload, batches of 1, 8 and 64 requests
+with 512-token prompts that generate 256 tokens each (``decode_b<B>_p512_g256``: batch / mean step
+over the steps in which all of them decode, ``..._frac``: that step's share of the HBM roofline,
+``e2e_b<B>_p512_g256``: generated tokens / wall time with the prompts' time included, which is how
+the reference's ``benchmark.py:204`` counts).
 """
 from __future__ import annotations
 
@@ -68,7 +74,7 @@ def make_engine(model_config, dtype, batch, context, chunk, graphs, seed=0):
     )
 
 
-def time_decode(engine, vocab, batch, context, steps, warmup, seed=0):
+def time_decode(engine, vocab, batch, context, steps, warmup, seed=0, sampling=None):
     """Reads ``batch`` prompts in through the engine, then times ``steps`` steps in which every request decodes.
     Every request holds at least ``context`` tokens at the last timed step (those admitted first a few more).
     Returns (seconds per step, mean tokens in the cache per request over the timed steps)."""
@@ -82,8 +88,8 @@ def time_decode(engine, vocab, batch, context, steps, warmup, seed=0):
     rng = random.Random(seed)
     prompt_len = max(1, context - steps - warmup)
     requests = [
-        Request(f"decode-{batch}-{i}", [rng.randrange(vocab) for _ in range(prompt_len)],
-                SamplingParams(temperature=0.0, max_tokens=steps + warmup + SLACK - 1, ignore_eos=True))
+        Request(f"decode-{batch}-{i}-{bool(sampling)}", [rng.randrange(vocab) for _ in range(prompt_len)],
+                SamplingParams(max_tokens=steps + warmup + SLACK - 1, ignore_eos=True, **(sampling or {"temperature": 0.0})))
         for i in range(batch)
     ]
     for request in requests:
@@ -107,6 +113,43 @@ def time_decode(engine, vocab, batch, context, steps, warmup, seed=0):
     return elapsed / steps, mean_context
 
 
+def time_workload(engine, vocab, batch, prompt_len, generated, seed=2):
+    """The reference's decode benchmark: ``batch`` requests with prompts of ``prompt_len`` random tokens generate
+    ``generated`` tokens each.  Returns (seconds per step over the steps in which all of them decode, mean tokens in the
+    cache per request over those steps, generated tokens per second of wall time from the first add to the last token)."""
+    import random
+
+    import torch
+
+    from velox_amd import Request, SamplingParams
+    from velox_amd.engine.request import RequestStatus
+
+    rng = random.Random(seed)
+    requests = [Request(f"work-{batch}-{i}", [rng.randrange(vocab) for _ in range(prompt_len)],
+                        SamplingParams(temperature=0.0, max_tokens=generated, ignore_eos=True)) for i in range(batch)]
+    torch.cuda.synchronize()
+    wall_start = time.perf_counter()
+    for request in requests:
+        engine.add_request(request)
+    while any(r.status is not RequestStatus.RUNNING_DECODE for r in requests):
+        engine.step()
+    torch.cuda.synchronize()
+    held = sum(r.num_computed_tokens for r in requests)
+    steps = 0
+    start = time.perf_counter()
+    while not any(len(r.output_token_ids) >= generated - 1 for r in requests):  # (a step ahead may be in flight: stop one short)
+        engine.step()
+        steps += 1
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - start
+    while engine.has_work():
+        engine.step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - wall_start
+    assert all(len(r.output_token_ids) == generated for r in requests)
+    return elapsed / steps, held / batch + (steps + 1) / 2, batch * generated / wall
+
+
 def time_prefill(engine, vocab, tokens, repeats=3, seed=1):
     import random
 
@@ -115,7 +158,7 @@ def time_prefill(engine, vocab, tokens, repeats=3, seed=1):
     from velox_amd import Request, SamplingParams
 
     rng = random.Random(seed)
-    best = None
+    times = []
     for attempt in range(repeats + 1):
         request = Request(f"prefill-{attempt}", [rng.randrange(vocab) for _ in range(tokens)],
                           SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True))
@@ -128,8 +171,8 @@ def time_prefill(engine, vocab, tokens, repeats=3, seed=1):
         assert len(request.output_token_ids) == 1, "the prompt did not prefill in one step"
         engine.step()  # reaps the finished request
         if attempt > 0:
-            best = elapsed if best is None else min(best, elapsed)
-    return best
+            times.append(elapsed)
+    return sum(times) / len(times), min(times)
 
 
 def main() -> int:
@@ -171,7 +214,16 @@ def main() -> int:
     for batch in batches:
         steps = args.steps if batch == args.batch else max(8, args.steps // 2)
         step_s[batch], contexts[batch] = time_decode(engine, vocab, batch, args.context, steps, args.warmup)
-    prefill_s = time_prefill(engine, vocab, args.prefill_tokens)
+    points = {f"decode_b{b}": round(b / t, 2) for b, t in step_s.items() if b != args.batch}
+    if not args.no_points:
+        sampled_s, _ = time_decode(engine, vocab, 64, args.context, max(8, args.steps // 2), args.warmup, sampling={"temperature": 0.8, "top_p": 0.9, "seed": 7})
+        points["decode_b64_sampled"] = round(64 / sampled_s, 2)
+        for batch in (1, 8, 64):
+            each_s, mean_context, wall_rate = time_workload(engine, vocab, batch, 512, 256)
+            points[f"decode_b{batch}_p512_g256"] = round(batch / each_s, 2)
+            points[f"decode_b{batch}_p512_g256_frac"] = round(decode_bytes(model_config, layers, batch, mean_context, elem) / each_s / 1e9 / PEAK_HBM_GBS, 4)
+            points[f"e2e_b{batch}_p512_g256"] = round(wall_rate, 2)
+    prefill_s, prefill_best_s = time_prefill(engine, vocab, args.prefill_tokens)
 
     main_step = step_s[args.batch]
     bytes_read = decode_bytes(model_config, layers, args.batch, contexts[args.batch], elem)
@@ -200,13 +252,13 @@ def main() -> int:
         },
         "prefill": {
             "value": round(args.prefill_tokens / prefill_s, 1), "tokens": args.prefill_tokens,
-            "ms": round(prefill_s * 1000, 3), "frac": round(flops / prefill_s / PEAK_FLOPS[args.dtype], 4),
+            "ms": round(prefill_s * 1000, 3), "frac": round(flops / prefill_s / PEAK_FLOPS[args.dtype], 4), "ms_best": round(prefill_best_s * 1000, 3),
         },
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
             "frac": round(achieved / PEAK_HBM_GBS, 4),
         },
-        "points": {f"decode_b{b}": round(b / s, 2) for b, s in step_s.items() if b != args.batch},
+        "points": points,
     }
     if not args.no_probes:
         # what this card delivers to a kernel that only reads, and to one that only issues matrix instructions: the

@@ -297,7 +297,7 @@ def test_residual_add_and_norm_split_between_two_products(ops, ref, m, hidden, i
     assert norm.forward(residual, deferred, None) is deferred
     for row_tiles in (1, 2, 0):  # tiles of the weight per workgroup (0: half a tile): the same sums in the same order
         again = residual0.clone()
-        other = ops._linear_into_residual(x, w_out, ResidualSink(again, norm), row_tiles=row_tiles)
+        other = ops._linear_into_residual(x, p_out, ResidualSink(again, norm), row_tiles=row_tiles)
         assert torch.equal(again, residual) and torch.equal(other.x, deferred.x)
         blocks = (hidden + 15) // 16
         assert other.sums.shape[1] == (2 * blocks if row_tiles == 0 else blocks)
