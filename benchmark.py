@@ -214,7 +214,10 @@ def main(argv=None) -> int:
         if args.tune_library:
             from velox_amd.engine.runner import decode_buckets
 
-            engine.tune_matrix_products([args.max_prefill_chunk_size, max(args.max_num_batched_tokens, max_num_seqs)] + [b for b in decode_buckets(max_num_seqs) if b > 16])
+            # a ladder of step sizes up to the token budget: a step is padded up to the next one when that is close
+            budget = max(args.max_num_batched_tokens, max_num_seqs)
+            ladder = sorted({args.max_prefill_chunk_size, budget} | {n for n in range(128, budget + 1, 128) if n * 8 >= budget})
+            engine.tune_matrix_products(ladder + [b for b in decode_buckets(max_num_seqs) if b > 16])
         vocab = engine.model.spec.vocab_size
         limit = engine.max_model_len - args.max_tokens - 1
         if limit < 1:

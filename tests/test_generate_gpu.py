@@ -171,6 +171,26 @@ def test_graph_replay_gives_the_eager_logits(tmp_path, name, dtype):
             h.live[rid][1] += 1
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_a_little_short_of_a_timed_row_count_are_padded_onto_the_null_page(tmp_path, dtype):
+    """Once the library's kernels have been timed for a number of rows, a step of prompt portions with a few rows less runs
+    with that many: the extra rows belong to a sequence on the null page, and nobody's logits change."""
+    folder = make_folder(tmp_path, "B", dtype)
+    config, weights = read_model_folder(folder)
+    prompts = [random_tokens(config["vocab_size"], n, seed=90 + n) for n in (29, 30, 3)]  # 62 rows in the first step, 3 in the next ones
+    plain = engine_for(folder, "B", dtype, max_num_batched_tokens=64, max_prefill_chunk_size=32).generate(greedy(prompts, 5))
+    engine = engine_for(folder, "B", dtype, max_num_batched_tokens=64, max_prefill_chunk_size=32)
+    engine.runner.tuned_row_counts = [16, 64]  # (as tune_matrix_products leaves them)
+    padded = engine.generate(greedy(prompts, 5, prefix="padded"))
+    assert engine.runner.num_padded_steps == 1  # 62 -> 64; decode-sized steps and steps far from a timed count stay as they are
+    assert [r.output_token_ids for r in padded] == [r.output_token_ids for r in plain]
+    if dtype == "float32":
+        for request, prompt in zip(padded, prompts):
+            assert request.output_token_ids == plain_greedy(config, weights, prompt, 5)
+    assert engine.cache.num_used_pages() == 0
+    engine.cache.assert_consistent([])
+
+
 def test_library_tuning_recaptures_the_decode_graphs_and_keeps_the_logits(tmp_path):
     """bfloat16: after the matrix library has picked kernels for a decode batch size, the captured steps are captured
     again (they hold the library's kernels) and generation still agrees with the plain model to rounding."""
@@ -181,6 +201,7 @@ def test_library_tuning_recaptures_the_decode_graphs_and_keeps_the_logits(tmp_pa
     assert not engine.ops.library_serves(32, 256, 64)  # too small for the library's timing to mean anything
     before = dict(engine.runner._graphs)
     assert engine.tune_matrix_products([128]) > 0
+    assert engine.runner.tuned_row_counts == [128]
     assert all(engine.runner._graphs[b] is before[b] for b in before)  # no captured step has 128 rows
     engine.ops.library_serves = lambda m, n, k: m > 16  # (tiny weights: pretend they are worth timing)
     assert engine.tune_matrix_products([32]) > 0

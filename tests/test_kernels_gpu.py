@@ -646,6 +646,67 @@ def test_argmax_and_sampling(ops, ref):
     assert got[5] == int(logits[5].argmax())  # top_k = 1 is greedy
 
 
+@pytest.mark.parametrize("vocab,spread", [(152064, 1.2), (151936 + 3, 4.0), (320, 2.0), (4099, 0.3)])
+def test_sampling_keeps_exactly_the_tokens_the_filters_allow(ops, vocab, spread):
+    """The threshold of top-k / top-p at the real vocabulary size, flat and peaked rows, ties across the threshold: over many
+    draws per row, every drawn token is one the plain filter keeps, and the tokens at the filter's edge (the last kept ones)
+    are drawn as well, so the kept set is neither too small nor too large.  A row's draw does not depend on its place."""
+    settings = [(0.8, 0.9, 0), (1.0, 1.0, 7), (0.7, 0.5, 50), (1.3, 0.95, 1000), (1.0, 0.999, 0), (0.5, 0.3, 3), (1.0, 1.0, 0), (2.0, 0.6, 20000)]
+    base = rand((len(settings), vocab), torch.float32, 77, spread)
+    base[2, 5] = base[2, 11] = base[2, vocab - 1] = float(base[2].max()) + 0.5  # three equal tokens at the top
+    base[5, :40] = float(base[5].max())  # forty equal tokens: rank 0 for all of them, so top_k = 3 keeps all forty
+    draws = 300
+    logits = base.repeat_interleave(draws, 0).contiguous()
+    options = np.zeros((len(settings) * draws, 6), dtype=np.int32)
+    f = options.view(np.float32)
+    for r, (temp, top_p, top_k) in enumerate(settings):
+        rows = slice(r * draws, (r + 1) * draws)
+        f[rows, 0], f[rows, 1] = temp, top_p
+        options[rows, 2] = top_k if 0 < top_k < vocab else 0
+        options[rows, 3], options[rows, 4] = 4242 + r, 17
+        options[rows, 5] = np.arange(draws)
+    got = ops.sample(logits, torch.from_numpy(options).cuda()).cpu().numpy()
+    for r, (temp, top_p, top_k) in enumerate(settings):
+        _, scores = TorchOps.sample_row(base[r].cpu().numpy(), options[r * draws])
+        kept = np.isfinite(scores)
+        drawn = got[r * draws:(r + 1) * draws]
+        assert kept[drawn].all(), f"row {r}: tokens {sorted(set(drawn[~kept[drawn]]))} were drawn but are filtered out"
+        if kept.sum() <= 50:
+            # few tokens are kept: 300 draws at these temperatures reach every one of them, the edge of the filter included
+            x = base[r].cpu().numpy().astype(np.float64)
+            share = np.where(kept, np.exp((x - x.max()) / temp), 0.0)
+            probable = share / share.sum() > 0.04  # (missed by 300 draws with probability below 1e-5)
+            assert set(np.flatnonzero(probable)) <= set(drawn), f"row {r}: kept tokens {sorted(set(np.flatnonzero(probable)) - set(drawn))} never drawn"
+        # each draw is the best score among the kept tokens, with the generator's noise for its own counter
+        for j in (0, 1, draws - 1):
+            token, scores = TorchOps.sample_row(base[r].cpu().numpy(), options[r * draws + j])
+            assert scores[drawn[j]] >= scores.max() - 1e-3, (r, j, int(drawn[j]), token)
+    # the same rows in another order and beside other rows: the same tokens
+    order = torch.randperm(len(settings) * draws, generator=torch.Generator().manual_seed(5))[:97]
+    again = ops.sample(logits[order.cuda()].contiguous(), torch.from_numpy(options[order.numpy()]).cuda()).cpu().numpy()
+    assert (again == got[order.numpy()]).all()
+
+
+def test_penalties_over_long_histories_and_a_large_vocabulary(ops, ref):
+    vocab, rows, width = 152064, 4, 6000
+    logits = rand((rows, vocab), torch.float32, 34, 2.0)
+    g = torch.Generator().manual_seed(35)
+    tokens = torch.randint(0, vocab, (rows, width), generator=g).to(torch.int32)
+    tokens[1, :3000] = torch.randint(8000, 8200, (3000,), generator=g).to(torch.int32)  # many repeats inside one range of the table
+    tokens[2, :] = 151000  # one token, 6000 times
+    tokens = tokens.cuda()
+    lengths = torch.tensor([6000, 3500, 6000, 1], dtype=torch.int32).cuda()
+    coeffs = torch.tensor([[1.3, 0.5, 0.2], [2.0, 1.0, 0.01], [0.8, 0.0, 0.001], [1.1, 0.2, 0.3]], dtype=torch.float32).cuda()
+    got, want = logits.clone(), logits.clone()
+    ops.apply_penalties(got, tokens, lengths, coeffs)
+    ref.apply_penalties(want, tokens, lengths, coeffs)
+    torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-6)
+    assert int((got != logits).sum()) > 5000
+    again = logits.clone()
+    ops.apply_penalties(again, tokens, lengths, coeffs)
+    assert torch.equal(again, got)
+
+
 def test_sampling_follows_the_distribution(ops):
     vocab = 50
     logits = rand((1, vocab), torch.float32, 31, 1.5).repeat(4000, 1).contiguous()

@@ -139,7 +139,7 @@ constexpr int GENERAL_MIN_WAVES = D <= 128 ? 2 : 1;
 // KSPLIT = 2: the workgroup has two sets of 4 waves that own the same rows and take the key tiles alternately, each
 // set staging its own tiles; at the end the second set hands its running (maximum, sum, output) to the first
 // through LDS.  The longest workgroups of a causal step, which decide how long the step takes, finish in half the time.
-template <typename T, int BN, int CT, int KSPLIT, int WAVES = 4>
+template <typename T, int BN, int CT, int KSPLIT, int WAVES = 4, int DB = 0>
 __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_waves_per_eu(GENERAL_MIN_WAVES, WAVES > 4 ? 4 : 2))) paged_attention_kernel(
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
@@ -163,15 +163,16 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
   constexpr int ROWS_PER_BLOCK = 16 * WAVES * CT;
   constexpr int TILE_ELEMS = BN * KS + D * VS;                      // one set's K tile and V^T tile
   constexpr int MERGE_FLOATS = KSPLIT > 1 ? 256 * CT * (4 * NC + 2) : 0;  // what the second set hands over at the end
-  constexpr int TILE_BYTES = KSPLIT * TILE_ELEMS * (int)sizeof(T);
+  static_assert(DB == 0 || KSPLIT == 1, "two tile buffers are for one set of waves");
+  constexpr int TILE_BYTES = (KSPLIT + DB) * TILE_ELEMS * (int)sizeof(T);
   constexpr int SMEM_BYTES = TILE_BYTES > 4 * MERGE_FLOATS ? TILE_BYTES : 4 * MERGE_FLOATS;
   __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
   __shared__ int page_ids[PREFILL_PAGE_IDS];
 
   const int set = KSPLIT > 1 ? threadIdx.x / 256 : 0;  // which set of 4 waves
   const int tid = KSPLIT > 1 ? threadIdx.x % 256 : threadIdx.x;  // thread within the set
-  T* const k_tile = reinterpret_cast<T*>(smem) + set * TILE_ELEMS;
-  T* const v_tile = k_tile + BN * KS;
+  T* k_tile = reinterpret_cast<T*>(smem) + set * TILE_ELEMS;  // (with two buffers: the one being filled or read, see the loop)
+  T* v_tile = k_tile + BN * KS;
   const int lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 4, i = lane & 15;
   const int group = nh / nkv;
@@ -251,7 +252,10 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
   };
   load_page_ids();
   if constexpr (DP > D) {
-    for (int e = tid; e < BN * (DP - D); e += SETW) k_tile[(e / (DP - D)) * KS + D + e % (DP - D)] = from_f32<T>(0.f);
+    for (int e = tid; e < BN * (DP - D); e += SETW) {
+      k_tile[(e / (DP - D)) * KS + D + e % (DP - D)] = from_f32<T>(0.f);
+      if constexpr (DB) k_tile[TILE_ELEMS + (e / (DP - D)) * KS + D + e % (DP - D)] = from_f32<T>(0.f);
+    }
   }
   auto page_of = [&](int n) -> size_t { return (size_t)page_ids[(n >> page_shift) - first_page]; };
 
@@ -365,28 +369,8 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     }
   };
 
-  __syncthreads();  // page ids are in place
-  // iteration `it` covers tiles tile_lo + it * KSPLIT .. + KSPLIT - 1, one per set (the last iteration may leave a set without one)
-  const int iterations = tile_hi > tile_lo ? (tile_hi - tile_lo + KSPLIT - 1) / KSPLIT : 0;
-  if (tile_lo + set < tile_hi) fetch(n_begin + (tile_lo + set) * BN);
-  for (int it = 0; it < iterations; ++it) {
-    const int tile = tile_lo + it * KSPLIT + set;
-    const bool have_tile = KSPLIT == 1 || tile < tile_hi;
-    const int n0 = n_begin + tile * BN;
-    __syncthreads();  // the previous tile has been read by every wave
-    if (have_tile) commit(n0);
-    __syncthreads();
-    if (it + 1 < iterations) {
-      const int next_first = n_begin + (tile_lo + (it + 1) * KSPLIT) * BN;  // first key of the next iteration's tiles
-      if (((next_first + KSPLIT * BN - 1) >> page_shift) - first_page >= PREFILL_PAGE_IDS) {  // the same for every thread
-        first_page = next_first >> page_shift;
-        load_page_ids();
-        __syncthreads();
-      }
-      if (tile + KSPLIT < tile_hi) fetch(n0 + KSPLIT * BN);  // in flight while this tile is computed
-    }
-    if (!have_tile || n0 > wave_last_pos) continue;  // nothing this wave may read; it still took part in the staging
-
+  // one staged tile of keys starting at n0, read from k_tile / v_tile: S^T = K Q^T, softmax update, O^T += V^T P^T
+  auto process = [&](int n0) {
     // ---- S^T = K Q^T ----------------------------------------------------------------------
     float4_t s[CT][NT];
 #pragma unroll
@@ -459,6 +443,67 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) acc_o[ct][c] = B::mma(vf, pf[ct][kb], acc_o[ct][c]);
       }
+    }
+  };
+
+  __syncthreads();  // page ids are in place
+  if constexpr (!DB) {
+  // iteration `it` covers tiles tile_lo + it * KSPLIT .. + KSPLIT - 1, one per set (the last iteration may leave a set without one)
+  const int iterations = tile_hi > tile_lo ? (tile_hi - tile_lo + KSPLIT - 1) / KSPLIT : 0;
+  if (tile_lo + set < tile_hi) fetch(n_begin + (tile_lo + set) * BN);
+  for (int it = 0; it < iterations; ++it) {
+    const int tile = tile_lo + it * KSPLIT + set;
+    const bool have_tile = KSPLIT == 1 || tile < tile_hi;
+    const int n0 = n_begin + tile * BN;
+    __syncthreads();  // the previous tile has been read by every wave
+    if (have_tile) commit(n0);
+    __syncthreads();
+    if (it + 1 < iterations) {
+      const int next_first = n_begin + (tile_lo + (it + 1) * KSPLIT) * BN;  // first key of the next iteration's tiles
+      if (((next_first + KSPLIT * BN - 1) >> page_shift) - first_page >= PREFILL_PAGE_IDS) {  // the same for every thread
+        first_page = next_first >> page_shift;
+        load_page_ids();
+        __syncthreads();
+      }
+      if (tile + KSPLIT < tile_hi) fetch(n0 + KSPLIT * BN);  // in flight while this tile is computed
+    }
+    if (!have_tile || n0 > wave_last_pos) continue;  // nothing this wave may read; it still took part in the staging
+    process(n0);
+  }
+  }
+
+  if constexpr (DB) {
+    // Two tile buffers: while the waves compute on one, the next tile is written into the other, so the waves meet at one
+    // barrier per tile instead of two.  Tile `it` lives in buffer it % 2; its registers were asked for an iteration ago.
+    T* const base = reinterpret_cast<T*>(smem);
+    const int iterations = tile_hi > tile_lo ? tile_hi - tile_lo : 0;
+    if (iterations > 0) {
+      fetch(n_begin + tile_lo * BN);
+      commit(n_begin + tile_lo * BN);
+      if (iterations > 1) fetch(n_begin + (tile_lo + 1) * BN);
+    }
+    __syncthreads();
+    for (int it = 0; it < iterations; ++it) {
+      const int n0 = n_begin + (tile_lo + it) * BN;
+      if (it + 1 < iterations) {
+        k_tile = base + ((it + 1) & 1) * TILE_ELEMS;
+        v_tile = k_tile + BN * KS;
+        commit(n0 + BN);  // read last in iteration it - 1, which every wave has left
+        if (it + 2 < iterations) {
+          const int next_first = n0 + 2 * BN;
+          if (((next_first + BN - 1) >> page_shift) - first_page >= PREFILL_PAGE_IDS) {  // the same for every thread
+            __syncthreads();
+            first_page = next_first >> page_shift;
+            load_page_ids();
+            __syncthreads();
+          }
+          fetch(next_first);
+        }
+      }
+      k_tile = base + (it & 1) * TILE_ELEMS;
+      v_tile = k_tile + BN * KS;
+      if (n0 <= wave_last_pos) process(n0);
+      __syncthreads();
     }
   }
 
@@ -806,6 +851,9 @@ static int compute_units() {
   return cached;
 }
 
+static int g_experiment = 0;
+extern "C" void velox_attention_experiment(int variant) { g_experiment = variant; }
+
 template <typename T> constexpr int tile_keys() { return (sizeof(T) * D > 512) ? 32 : 64; }
 
 template <typename T>
@@ -839,6 +887,40 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
   // keys 315 us against 426 the other way round; the two meet where an average row reads about 1,300 keys.
   constexpr int WIDE = (sizeof(T) == 2 && D <= 128) ? 2 : 1;
   const int rows = max_q_len * group;
+  if (WIDE == 2 && g_experiment > 0) {
+    if (g_experiment == 1) {
+      dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
+      paged_attention_kernel<T, BN, WIDE, 1, 4><<<grid, 256, 0, stream>>>(
+          (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+    } else if (g_experiment == 4) {
+      dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
+      paged_attention_kernel<T, BN, 1, 1, 8, 1><<<grid, 512, 0, stream>>>(
+          (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+    } else if (g_experiment == 5) {
+      dim3 grid((rows + 255) / 256, nkv, num_seqs * splits);
+      paged_attention_kernel<T, BN, WIDE, 1, 8, 1><<<grid, 512, 0, stream>>>(
+          (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+    } else if (g_experiment == 6) {
+      dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
+      paged_attention_kernel<T, BN, WIDE, 1, 4, 1><<<grid, 256, 0, stream>>>(
+          (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+    } else if (g_experiment == 2) {
+      dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
+      paged_attention_kernel<T, BN, WIDE, WIDE, 4><<<grid, 512, 0, stream>>>(
+          (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+    } else {
+      dim3 grid((rows + 63) / 64, nkv, num_seqs * splits);
+      paged_attention_kernel<T, BN, 1, WIDE, 4><<<grid, 512, 0, stream>>>(
+          (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+    }
+    return (int)hipGetLastError();
+  }
   if (WIDE == 2 && rows > 64 && (long long)total_tokens * group / 128 * nkv * splits >= compute_units()) {
     if (max_kv_len - max_q_len / 2 <= 1280 || rows < 192) {  // (keys an average row reads)
       dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);

@@ -184,16 +184,121 @@ __device__ __forceinline__ uint32_t sort_key(float v) {
   return (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
 }
 
+// ---- the threshold of top-k / top-p: a radix search over the ordered keys ------------------------------------------
+// A token is kept iff fewer than top_k tokens have a larger x and the tokens with a larger x hold less than top_p of the
+// probability.  Both conditions only get harder to meet as x falls, so the kept tokens are those whose key is at least
+// some threshold.  The threshold is found digit by digit (11, 11 and 10 bits of the 32-bit key): one pass over the row
+// fills, for the tokens that match the digits found so far, a table per value of the next digit (how many tokens, how
+// much probability); a walk down the table from the largest digit finds the last digit whose largest member is still
+// kept.  Probabilities are summed as 40-bit fixed-point integers, so a sum does not depend on the order in which the
+// threads add and a row's threshold is the same in every run and every batch.
+#define SELECT_BINS 2048
+__device__ __forceinline__ unsigned long long fixed_point_mass(float p) { return (unsigned long long)(p * 1099511627776.f); }  // p in [0, 1], 2^40
+
+struct Above { unsigned int count; unsigned long long mass; };
+
+// Visits every element of a row: f(index, value).  Whole quads of four consecutive elements come as 16-byte loads when
+// the row starts at a 16-byte boundary, four loads in flight per thread (one workgroup reads the whole row: with one
+// load at a time a pass would take as many trips to the caches as a thread has quads).
+template <typename F> __device__ __forceinline__ void for_each_in_row(const float* __restrict__ row, int vocab, F f) {
+  if ((reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+    const int quads = vocab / 4;
+    const float4_t* body = reinterpret_cast<const float4_t*>(row);
+    const int stride = blockDim.x;
+    int q = threadIdx.x;
+    for (; q + 3 * stride < quads; q += 4 * stride) {
+      const float4_t v0 = body[q], v1 = body[q + stride], v2 = body[q + 2 * stride], v3 = body[q + 3 * stride];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) f(4 * q + e, v0[e]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) f(4 * (q + stride) + e, v1[e]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) f(4 * (q + 2 * stride) + e, v2[e]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) f(4 * (q + 3 * stride) + e, v3[e]);
+    }
+    for (; q < quads; q += stride) {
+      const float4_t v = body[q];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) f(4 * q + e, v[e]);
+    }
+    for (int i = 4 * quads + threadIdx.x; i < vocab; i += blockDim.x) f(i, row[i]);
+  } else {
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) f(i, row[i]);
+  }
+}
+
+// One digit of the search.  `counts` and `masses` hold the table of this digit (SELECT_BINS entries, filled by the whole
+// workgroup, barrier behind it); `above` is what lies above every token that matches the digits found so far.  Wave 0 walks
+// the table; every thread gets the digit found, and `above` grows by what lies above that digit's tokens.
+__device__ __forceinline__ int select_digit(const unsigned int* counts, const unsigned long long* masses, int bins, int top_k, bool use_mass,
+                                            unsigned long long mass_limit, Above& above, int* found_digit, Above* found_above) {
+  if (threadIdx.x < 64) {
+    const int lane = threadIdx.x;
+    const int per_lane = bins / 64;  // lane 0 holds the largest digits
+    const int hi = bins - 1 - lane * per_lane;  // this lane's digits: hi, hi - 1, ..., hi - per_lane + 1
+    unsigned int c = 0;
+    unsigned long long m = 0;
+    for (int j = 0; j < per_lane; ++j) { c += counts[hi - j]; m += masses[hi - j]; }
+    // what lies above this lane's first digit: the sums of the lanes before it
+    unsigned int c_before = c;
+    unsigned long long m_before = m;
+#pragma unroll
+    for (int offset = 1; offset < 64; offset <<= 1) {
+      const unsigned int oc = __shfl_up(c_before, offset, VELOX_WAVE);
+      const unsigned long long om = __shfl_up(m_before, offset, VELOX_WAVE);
+      if (lane >= offset) { c_before += oc; m_before += om; }
+    }
+    c_before = above.count + c_before - c;
+    m_before = above.mass + m_before - m;
+    // the smallest digit of this lane whose members' top is still kept
+    int lowest = 0x7fffffff;
+    unsigned int lowest_c = 0;
+    unsigned long long lowest_m = 0;
+    for (int j = 0; j < per_lane; ++j) {
+      const bool kept = (top_k <= 0 || c_before < (unsigned int)top_k) && (!use_mass || m_before < mass_limit);
+      if (kept) { lowest = hi - j; lowest_c = c_before; lowest_m = m_before; }
+      c_before += counts[hi - j];
+      m_before += masses[hi - j];
+    }
+    // over the wave: kept digits form a run from the top, so the smallest one overall is the answer
+    int best = lowest;
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) {
+      const int other = __shfl_xor(best, offset, VELOX_WAVE);
+      best = other < best ? other : best;
+    }
+    if (best == lowest && lowest != 0x7fffffff) {
+      *found_digit = lowest;
+      found_above->count = lowest_c;
+      found_above->mass = lowest_m;
+    }
+    if (best == 0x7fffffff && lane == 0) {  // (cannot happen: the largest digit's top is always kept)
+      *found_digit = bins - 1;
+      *found_above = above;
+    }
+  }
+  __syncthreads();
+  above = *found_above;
+  return *found_digit;
+}
+
 // options per row, int32[6]: temperature (float bits), top_p (float bits), top_k, seed low 31 bits, seed high 31 bits, counter
 //   temperature == 0: argmax.
 //   otherwise x = logit / max(T, 1e-5); p = softmax(x); token i is kept iff fewer than top_k tokens have a larger x
 //   (top_k > 0) and the tokens with a larger x hold less than top_p of the probability; among the kept tokens the
 //   draw is argmax(x - max - log(e)), e = max(-log(u), 1e-10), u uniform from Philox(key = seed, counter = (i / 4, counter)).
+// One workgroup per row.  Passes over the row (from the caches: a row is a few hundred kilobytes): the maximum; with a
+// filter, the sum and three digits of the threshold; the draw.
 __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(const float* __restrict__ logits, const int* __restrict__ options,
                                                                 int* __restrict__ out, int vocab) {
   __shared__ Best best_scratch[16];
   __shared__ float scratch[16];
-  __shared__ float scratch2[16];
+  __shared__ unsigned int counts[SELECT_BINS];
+  __shared__ unsigned long long masses[SELECT_BINS];
+  __shared__ unsigned long long total_mass;
+  __shared__ int found_digit;
+  __shared__ Above found_above;
   const float* row = logits + (size_t)blockIdx.x * vocab;
   const int* opt = options + (size_t)blockIdx.x * 6;
   const float temperature = __int_as_float(opt[0]);
@@ -204,58 +309,102 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(const float* __r
 
   if (temperature == 0.f) {
     Best best{-INFINITY, 0x7fffffff};
-    for (int i = tid; i < vocab; i += blockDim.x) {
-      const float v = row[i];
-      if (v > best.value || best.index == 0x7fffffff) best = Best{v, i};
-    }
+    for_each_in_row(row, vocab, [&](int i, float v) { best = better(best, Best{v, i}); });
     best = block_best(best, best_scratch);
     if (tid == 0) out[blockIdx.x] = best.index;
     return;
   }
   const float inv_t = 1.f / fmaxf(temperature, 1e-5f);
   float mx = -INFINITY;
-  for (int i = tid; i < vocab; i += blockDim.x) mx = fmaxf(mx, row[i] * inv_t);
+  for_each_in_row(row, vocab, [&](int, float v) { mx = fmaxf(mx, v * inv_t); });
   mx = block_max(mx, scratch);
-  float z = 0.f;
-  for (int i = tid; i < vocab; i += blockDim.x) z += expf(row[i] * inv_t - mx);
-  z = block_sum(z, scratch);
 
   // smallest key whose tokens are kept
   uint32_t threshold = 0u;
-  const bool filter = (top_k > 0 && top_k < vocab) || top_p < 1.f;
+  const bool use_mass = top_p < 1.f;
+  const bool filter = (top_k > 0 && top_k < vocab) || use_mass;
   if (filter) {
-    const float mass_limit = top_p * z;
-    uint32_t lo = 0u, hi = 0xffffffffu;  // predicate(hi) holds (nothing is larger); find the smallest key where it holds
-    while (lo < hi) {
-      const uint32_t mid = lo + ((hi - lo) >> 1);
-      float count = 0.f, mass = 0.f;
-      for (int i = tid; i < vocab; i += blockDim.x) {
-        const float x = row[i] * inv_t;
-        if (sort_key(x) > mid) { count += 1.f; mass += expf(x - mx); }
-      }
-      count = block_sum(count, scratch);
-      mass = block_sum(mass, scratch2);
-      const bool ok = (top_k <= 0 || count < (float)top_k) && (mass < mass_limit);
-      if (ok) hi = mid; else lo = mid + 1u;
+    Above above{0u, 0ull};
+    unsigned long long mass_limit = 0ull;
+    // digits: bits 31..21, 20..10, 9..0
+    uint32_t prefix = 0u;  // the digits found so far, in place
+#pragma unroll 1
+    for (int level = 0; level < 3; ++level) {
+      const int shift = level == 0 ? 21 : level == 1 ? 10 : 0;
+      const int width = level == 2 ? 10 : 11;
+      const int bins = 1 << width;
+      for (int b = tid; b < bins; b += blockDim.x) { counts[b] = 0u; masses[b] = 0ull; }
+      if (tid == 0 && level == 0) total_mass = 0ull;
+      __syncthreads();
+      const uint32_t known = level == 0 ? 0u : ~((1u << (shift + width)) - 1u);  // mask of the digits found so far
+      unsigned long long my_total = 0ull;
+      for_each_in_row(row, vocab, [&](int, float v) {
+        const float x = v * inv_t;
+        const uint32_t key = sort_key(x);
+        const bool match = (key & known) == prefix;
+        if (level == 0 || match) {
+          const unsigned long long mass = use_mass ? fixed_point_mass(expf(x - mx)) : 0ull;
+          if (level == 0) my_total += mass;
+          if (match) {
+            const int digit = (int)((key >> shift) & (uint32_t)(bins - 1));
+            atomicAdd(&counts[digit], 1u);
+            if (use_mass && mass != 0ull) atomicAdd(&masses[digit], mass);
+          }
+        }
+      });
+      if (level == 0 && use_mass) atomicAdd(&total_mass, my_total);
+      __syncthreads();
+      if (level == 0) mass_limit = (unsigned long long)((double)top_p * (double)total_mass);
+      const int digit = select_digit(counts, masses, bins, top_k, use_mass, mass_limit, above, &found_digit, &found_above);
+      prefix |= (uint32_t)digit << shift;
+      __syncthreads();  // the tables are free again
     }
-    threshold = lo;
+    threshold = prefix;
   }
 
   Best best{-INFINITY, 0x7fffffff};
   const int quads = (vocab + 3) / 4;
-  for (int q = tid; q < quads; q += blockDim.x) {
+  const bool aligned = (reinterpret_cast<uintptr_t>(row) & 15) == 0;
+  auto load_quad = [&](int q, float (&v)[4]) {
+    if (aligned && 4 * q + 3 < vocab) {
+      const float4_t loaded = *reinterpret_cast<const float4_t*>(row + 4 * q);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = loaded[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = 4 * q + e < vocab ? row[4 * q + e] : -INFINITY;
+    }
+  };
+  constexpr int AHEAD = 4;  // quads in flight per thread
+  for (int q0 = tid; q0 < quads; q0 += AHEAD * blockDim.x) {
+    float ahead[AHEAD][4];
+#pragma unroll
+    for (int a = 0; a < AHEAD; ++a) {
+      const int qa = q0 + a * blockDim.x;
+      load_quad(qa < quads ? qa : q0, ahead[a]);
+    }
+#pragma unroll
+    for (int a = 0; a < AHEAD; ++a) {
+    const int q = q0 + a * blockDim.x;
+    if (q >= quads) break;
+    float (&v)[4] = ahead[a];
+    bool any = false;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) any = any || (4 * q + e < vocab && !(filter && sort_key(v[e] * inv_t) < threshold));
+    if (!any) continue;  // (the noise of a quad is only worked out where a token of it is kept)
     uint32_t bits[4];
     philox4x32((uint32_t)q, counter, 0u, 0u, seed_lo, seed_hi, bits);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int i = 4 * q + e;
       if (i >= vocab) break;
-      const float x = row[i] * inv_t;
+      const float x = v[e] * inv_t;
       if (filter && sort_key(x) < threshold) continue;
       const float u = ((float)(bits[e] >> 8) + 0.5f) * (1.0f / 16777216.0f);
       const float noise = fmaxf(-logf(u), 1e-10f);
       const float score = (x - mx) - logf(noise);
       if (score > best.value || best.index == 0x7fffffff) best = Best{score, i};
+    }
     }
   }
   best = block_best(best, best_scratch);
@@ -270,27 +419,50 @@ extern "C" int velox_sample(const float* logits, const int* options, int* out, i
 
 // Penalties over the tokens a request has seen (prompt and output), each distinct token once:
 //   v = logit - frequency * count;  v = v > 0 ? v / repetition : v * repetition;  v -= presence
-__global__ void penalties_kernel(float* __restrict__ logits, const int* __restrict__ tokens, const int* __restrict__ lengths,
-                                 const float* __restrict__ coeffs, int vocab, int width) {
+// One workgroup per row.  The vocabulary is taken a range of PENALTY_RANGE token ids at a time: the history's tokens
+// inside the range are counted into a table in LDS, then the history is walked again and whoever takes a token's count
+// out of the table (leaving zero behind, so the table is clean for the next range) applies it.  Work grows with the
+// history's length times the number of ranges, never with its square.
+#define PENALTY_RANGE 8192
+__global__ void __launch_bounds__(256) penalties_kernel(float* __restrict__ logits, const int* __restrict__ tokens, const int* __restrict__ lengths,
+                                                        const float* __restrict__ coeffs, int vocab, int width) {
+  __shared__ int table[PENALTY_RANGE];
+  __shared__ unsigned int touched[(1 << 20) / PENALTY_RANGE / 32 + 1];  // one bit per range (vocabularies up to 2^20 ids and beyond: see below)
   const int r = blockIdx.x;
-  const int n = lengths[r];
+  const int n = lengths[r] < width ? lengths[r] : width;
   const int* seen = tokens + (size_t)r * width;
   const float repetition = coeffs[3 * r], presence = coeffs[3 * r + 1], frequency = coeffs[3 * r + 2];
   float* row = logits + (size_t)r * vocab;
-  for (int i = threadIdx.x; i < n; i += blockDim.x) {
-    const int token = seen[i];
-    if (token < 0 || token >= vocab) continue;
-    int count = 0;
-    bool first = true;
-    for (int j = 0; j < n; ++j) {
-      const bool same = seen[j] == token;
-      count += same ? 1 : 0;
-      if (same && j < i) first = false;
+  const int ranges = (vocab + PENALTY_RANGE - 1) / PENALTY_RANGE;
+  const bool track = ranges <= (1 << 20) / PENALTY_RANGE;  // (a larger vocabulary visits every range)
+  for (int i = threadIdx.x; i < PENALTY_RANGE; i += blockDim.x) table[i] = 0;
+  for (int i = threadIdx.x; i < (int)(sizeof(touched) / sizeof(touched[0])); i += blockDim.x) touched[i] = 0u;
+  __syncthreads();
+  if (track) {
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+      const int token = seen[i];
+      if (token >= 0 && token < vocab) atomicOr(&touched[(token / PENALTY_RANGE) >> 5], 1u << ((token / PENALTY_RANGE) & 31));
     }
-    if (!first) continue;
-    float v = row[token] - frequency * (float)count;
-    v = v > 0.f ? v / repetition : v * repetition;
-    row[token] = v - presence;
+    __syncthreads();
+  }
+  for (int range = 0; range < ranges; ++range) {
+    if (track && !((touched[range >> 5] >> (range & 31)) & 1u)) continue;  // (the same for every thread)
+    const int lo = range * PENALTY_RANGE;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+      const int token = seen[i];
+      if (token >= lo && token < lo + PENALTY_RANGE && token < vocab) atomicAdd(&table[token - lo], 1);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+      const int token = seen[i];
+      if (token < lo || token >= lo + PENALTY_RANGE || token >= vocab) continue;
+      const int count = atomicExch(&table[token - lo], 0);
+      if (count == 0) continue;  // another occurrence of the token took the count
+      float v = row[token] - frequency * (float)count;
+      v = v > 0.f ? v / repetition : v * repetition;
+      row[token] = v - presence;
+    }
+    __syncthreads();
   }
 }
 

@@ -156,7 +156,8 @@ class Engine:
     def tune_matrix_products(self, token_counts: Sequence[int]) -> int:
         """Optional, bfloat16 only: has the matrix library time its candidate kernels for this model's weight shapes at
         the given numbers of tokens per step (typically the prefill chunk size and the larger decode batch sizes) and
-        keep the fastest.  Takes seconds per shape; steps with other token counts are unaffected.  Only products that
+        keep the fastest.  Takes seconds per shape.  A step of prompt portions with a few rows less than one of these
+        counts is padded up to it from then on (``ModelRunner.tuned_row_counts``); other steps are unaffected.  Only products that
         the engine hands to the library are timed (``ops.library_serves``); captured decode steps are captured again
         if one of them holds such a product."""
         if self.dtype != torch.bfloat16 or self.device.type != "cuda" or not hasattr(self.ops, "tune_library_products"):
@@ -174,6 +175,8 @@ class Engine:
             if served:
                 done += self.ops.tune_library_products(served, [count])
                 recapture = recapture or count <= self.config.max_num_seqs
+                if count > self.config.max_num_seqs and count not in self.runner.tuned_row_counts:
+                    self.runner.tuned_row_counts = sorted(self.runner.tuned_row_counts + [count])  # steps a little shorter are padded up to it
         if recapture and self.runner.uses_graphs:
             self.runner.capture_decode_graphs()
             torch.cuda.synchronize()

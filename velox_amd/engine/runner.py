@@ -61,7 +61,14 @@ class ModelRunner:
         self.device = torch.device(device)
         self.max_num_tokens = max(int(max_num_tokens), int(max_num_seqs))
         self.max_num_seqs = int(max_num_seqs)
-        self.builder = BatchBuilder(cache, self.device, self.max_num_tokens, self.max_num_seqs)
+        self.builder = BatchBuilder(cache, self.device, self.max_num_tokens, self.max_num_seqs + 1)  # (+1: the rows that pad a step, see tuned_row_counts)
+        # Numbers of rows for which the matrix library's kernels have been timed (``Engine.tune_matrix_products``).  The
+        # library picks a kernel per exact shape, and an untimed number of rows gets its default choice, about a quarter
+        # slower at these sizes: a step of portions that is a little short of a timed number of rows is padded up to it with
+        # rows of a sequence on the null page.
+        self.tuned_row_counts: List[int] = []
+        self.max_padding = 0.12  # the most a step is made longer, as a share of its own rows
+        self.num_padded_steps = 0
         # every part's scratch at its largest, before anything runs: captured steps hold these addresses
         self.workspace = Workspace(self.device)
         limits = StepLimits(self.max_num_tokens, self.max_num_seqs, cache.max_model_len)
@@ -89,8 +96,25 @@ class ModelRunner:
                 bucket = self._bucket_for(len(entries))
                 if bucket is not None:
                     return self._replay(bucket, entries, ids_on_device)
+        if self.tuned_row_counts and ids_on_device is None:
+            entries = self._padded_to_tuned_rows(entries)
         ctx = self.builder.build(entries, self.ops, self.dtype, self.workspace, ids_on_device=ids_on_device)
         return self._forward(ctx)
+
+    def _padded_to_tuned_rows(self, entries: Sequence[StepEntry]) -> Sequence[StepEntry]:
+        total = sum(len(e.token_ids) for e in entries)
+        if total <= self.max_num_seqs:
+            return entries  # decode-sized: the skinny kernels do not care, captured steps pad themselves
+        target = next((n for n in self.tuned_row_counts if n >= total), None)
+        if target is None or target == total or target > self.max_num_tokens or target - total > self.max_padding * total:
+            return entries
+        from ..cache.manager import SequenceCache
+
+        extra = target - total
+        pages = (extra + self.cache.page_size - 1) // self.cache.page_size
+        null_seq = SequenceCache(slot=self.cache.state.pad_slot, tables=[[0] * pages for _ in self.cache.groups], released=[0 for _ in self.cache.groups])
+        self.num_padded_steps += 1
+        return list(entries) + [StepEntry(null_seq, [0] * extra, 0, [])]
 
     def _forward(self, ctx: StepContext) -> Optional[torch.Tensor]:
         residual, pending = self.model.forward(ctx.token_ids, ctx)

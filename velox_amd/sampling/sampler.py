@@ -23,12 +23,48 @@ import torch
 from .params import SamplingParams
 
 
+class _Upload:
+    """Small int32 arrays from the host to the device without a wait: a ring of pinned buffers, each guarded by an event
+    (a buffer is written again only when the copy that read it has run), copied with ``non_blocking``.  From pageable
+    memory the same copy would make the host wait for everything queued on the stream before it."""
+
+    def __init__(self, device: torch.device, ring: int = 4) -> None:
+        self.device = device
+        self.pinned = device.type == "cuda"
+        self._host: List[Optional[torch.Tensor]] = [None] * ring
+        self._device: List[Optional[torch.Tensor]] = [None] * ring
+        self._events = [torch.cuda.Event() if self.pinned else None for _ in range(ring)]
+        self._used = [False] * ring
+        self._next = 0
+
+    def send(self, values: np.ndarray) -> torch.Tensor:
+        """``values``: int32, any shape -> a device tensor of that shape (valid until the ring comes round again)."""
+        flat = np.ascontiguousarray(values, dtype=np.int32).reshape(-1)
+        if not self.pinned:
+            return torch.from_numpy(flat.copy()).to(self.device).view(values.shape)
+        index = self._next
+        self._next = (index + 1) % len(self._host)
+        if self._used[index]:
+            self._events[index].synchronize()
+        if self._host[index] is None or self._host[index].numel() < flat.size:
+            size = max(1024, 1 << int(flat.size - 1).bit_length())
+            self._host[index] = torch.empty(size, dtype=torch.int32, pin_memory=True)
+            self._device[index] = torch.empty(size, dtype=torch.int32, device=self.device)
+        self._host[index].numpy()[:flat.size] = flat
+        target = self._device[index][:flat.size]
+        target.copy_(self._host[index][:flat.size], non_blocking=True)
+        self._events[index].record()
+        self._used[index] = True
+        return target.view(values.shape)
+
+
 class Sampler:
     def __init__(self, ops, device, seed: Optional[int] = None) -> None:
         self.ops = ops
         self.device = torch.device(device)
         self._rng = random.Random(seed)
         self._seeds: Dict[str, int] = {}
+        self._upload = _Upload(self.device)
 
     def _seed_for(self, request_id: str, params: SamplingParams) -> int:
         seed = self._seeds.get(request_id)
@@ -79,24 +115,26 @@ class Sampler:
             packed[r, 3] = seed & 0x7FFFFFFF
             packed[r, 4] = (seed >> 31) & 0x7FFFFFFF
             packed[r, 5] = int(n)
-        options = torch.from_numpy(packed).to(self.device)
-        return self.ops.sample(logits, options)
+        return self.ops.sample(logits, self._upload.send(packed))
 
     def _apply_penalties(self, logits, sampling_params, histories) -> torch.Tensor:
+        """A penalised copy of ``logits``.  Histories, their lengths and the coefficients travel as one int32 array."""
         rows = logits.shape[0]
         width = max(1, max(len(h) for h in histories))
-        tokens = np.zeros((rows, width), dtype=np.int32)
-        lengths = np.zeros(rows, dtype=np.int32)
-        coeffs = np.zeros((rows, 3), dtype=np.float32)
+        packed = np.zeros(rows * (width + 4), dtype=np.int32)
+        tokens = packed[: rows * width].reshape(rows, width)
+        lengths = packed[rows * width: rows * (width + 1)]
+        coeffs = packed[rows * (width + 1):].view(np.float32).reshape(rows, 3)
         for r, (p, h) in enumerate(zip(sampling_params, histories)):
             tokens[r, : len(h)] = np.asarray(h, dtype=np.int32)
             lengths[r] = len(h)
             coeffs[r] = (p.repetition_penalty, p.presence_penalty, p.frequency_penalty)
+        sent = self._upload.send(packed)
         out = logits.clone()
         self.ops.apply_penalties(
             out,
-            torch.from_numpy(tokens).to(self.device),
-            torch.from_numpy(lengths).to(self.device),
-            torch.from_numpy(coeffs).to(self.device),
+            sent[: rows * width].view(rows, width),
+            sent[rows * width: rows * (width + 1)],
+            sent[rows * (width + 1):].view(torch.float32).view(rows, 3),
         )
         return out
