@@ -139,7 +139,7 @@ constexpr int GENERAL_MIN_WAVES = D <= 128 ? 2 : 1;
 // KSPLIT = 2: the workgroup has two sets of 4 waves that own the same rows and take the key tiles alternately, each
 // set staging its own tiles; at the end the second set hands its running (maximum, sum, output) to the first
 // through LDS.  The longest workgroups of a causal step, which decide how long the step takes, finish in half the time.
-template <typename T, int BN, int CT, int KSPLIT, int WAVES = 4, int DB = 0>
+template <typename T, int BN, int CT, int KSPLIT, int WAVES = 4>
 __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_waves_per_eu(GENERAL_MIN_WAVES, WAVES > 4 ? 4 : 2))) paged_attention_kernel(
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
@@ -163,16 +163,15 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
   constexpr int ROWS_PER_BLOCK = 16 * WAVES * CT;
   constexpr int TILE_ELEMS = BN * KS + D * VS;                      // one set's K tile and V^T tile
   constexpr int MERGE_FLOATS = KSPLIT > 1 ? 256 * CT * (4 * NC + 2) : 0;  // what the second set hands over at the end
-  static_assert(DB == 0 || KSPLIT == 1, "two tile buffers are for one set of waves");
-  constexpr int TILE_BYTES = (KSPLIT + DB) * TILE_ELEMS * (int)sizeof(T);
+  constexpr int TILE_BYTES = KSPLIT * TILE_ELEMS * (int)sizeof(T);
   constexpr int SMEM_BYTES = TILE_BYTES > 4 * MERGE_FLOATS ? TILE_BYTES : 4 * MERGE_FLOATS;
   __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
   __shared__ int page_ids[PREFILL_PAGE_IDS];
 
   const int set = KSPLIT > 1 ? threadIdx.x / 256 : 0;  // which set of 4 waves
   const int tid = KSPLIT > 1 ? threadIdx.x % 256 : threadIdx.x;  // thread within the set
-  T* k_tile = reinterpret_cast<T*>(smem) + set * TILE_ELEMS;  // (with two buffers: the one being filled or read, see the loop)
-  T* v_tile = k_tile + BN * KS;
+  T* const k_tile = reinterpret_cast<T*>(smem) + set * TILE_ELEMS;
+  T* const v_tile = k_tile + BN * KS;
   const int lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 4, i = lane & 15;
   const int group = nh / nkv;
@@ -252,10 +251,7 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
   };
   load_page_ids();
   if constexpr (DP > D) {
-    for (int e = tid; e < BN * (DP - D); e += SETW) {
-      k_tile[(e / (DP - D)) * KS + D + e % (DP - D)] = from_f32<T>(0.f);
-      if constexpr (DB) k_tile[TILE_ELEMS + (e / (DP - D)) * KS + D + e % (DP - D)] = from_f32<T>(0.f);
-    }
+    for (int e = tid; e < BN * (DP - D); e += SETW) k_tile[(e / (DP - D)) * KS + D + e % (DP - D)] = from_f32<T>(0.f);
   }
   auto page_of = [&](int n) -> size_t { return (size_t)page_ids[(n >> page_shift) - first_page]; };
 
@@ -369,19 +365,56 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     }
   };
 
-  // one staged tile of keys starting at n0, read from k_tile / v_tile: S^T = K Q^T, softmax update, O^T += V^T P^T
-  auto process = [&](int n0) {
+  __syncthreads();  // page ids are in place
+  // iteration `it` covers tiles tile_lo + it * KSPLIT .. + KSPLIT - 1, one per set (the last iteration may leave a set without one)
+  const int iterations = tile_hi > tile_lo ? (tile_hi - tile_lo + KSPLIT - 1) / KSPLIT : 0;
+  if (tile_lo + set < tile_hi) fetch(n_begin + (tile_lo + set) * BN);
+  for (int it = 0; it < iterations; ++it) {
+    const int tile = tile_lo + it * KSPLIT + set;
+    const bool have_tile = KSPLIT == 1 || tile < tile_hi;
+    const int n0 = n_begin + tile * BN;
+    __syncthreads();  // the previous tile has been read by every wave
+    if (have_tile) commit(n0);
+    __syncthreads();
+    if (it + 1 < iterations) {
+      const int next_first = n_begin + (tile_lo + (it + 1) * KSPLIT) * BN;  // first key of the next iteration's tiles
+      if (((next_first + KSPLIT * BN - 1) >> page_shift) - first_page >= PREFILL_PAGE_IDS) {  // the same for every thread
+        first_page = next_first >> page_shift;
+        load_page_ids();
+        __syncthreads();
+      }
+      if (tile + KSPLIT < tile_hi) fetch(n0 + KSPLIT * BN);  // in flight while this tile is computed
+    }
+    if (!have_tile || n0 > wave_last_pos) continue;  // nothing this wave may read; it still took part in the staging
+
     // ---- S^T = K Q^T ----------------------------------------------------------------------
+    // bfloat16: the operands of the next 16 keys are asked for before this 16 keys' matrix instructions are issued, and
+    // the compiler is kept from moving each read down to just before its use (a read from LDS takes longer than the
+    // matrix instructions it feeds: 2,048 to 8,192 tokens 2-4% faster).  float32 operands and heads beyond 128 channels
+    // are too many registers for it.
+    constexpr int KEYS_AHEAD = (sizeof(T) == 2 && D <= 128) ? 1 : 0;
     float4_t s[CT][NT];
+    Operand kf[KEYS_AHEAD + 1][NQB];
+    if constexpr (KEYS_AHEAD > 0) {
+#pragma unroll
+      for (int cb = 0; cb < NQB; ++cb) kf[0][cb] = load_operand<T>(k_tile + i * KS + KB * cb + VEC * g);
+    }
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
+      if constexpr (KEYS_AHEAD > 0) {
+        if (t + 1 < NT) {
+#pragma unroll
+          for (int cb = 0; cb < NQB; ++cb) kf[(t + 1) & 1][cb] = load_operand<T>(k_tile + (16 * (t + 1) + i) * KS + KB * cb + VEC * g);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) s[ct][t] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int cb = 0; cb < NQB; ++cb) {
-        const Operand kf = load_operand<T>(k_tile + (16 * t + i) * KS + KB * cb + VEC * g);
+        if constexpr (KEYS_AHEAD == 0) kf[0][cb] = load_operand<T>(k_tile + (16 * t + i) * KS + KB * cb + VEC * g);
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) s[ct][t] = B::mma(kf, qf[ct][cb], s[ct][t]);
+        for (int ct = 0; ct < CT; ++ct) s[ct][t] = B::mma(kf[t & KEYS_AHEAD][cb], qf[ct][cb], s[ct][t]);
       }
     }
     // ---- scale, mask (only where the tile crosses a row's limits), running maximum ----------
@@ -433,77 +466,29 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
       m_i[ct] = m_new;
     }
     // ---- O^T = O^T * alpha + V^T P^T ------------------------------------------------------
+    constexpr int TILES_AHEAD = (sizeof(T) == 2 && D <= 128 && NC > 2) ? 2 : 0;  // channel tiles whose operands are in flight ahead of the one being multiplied
+    Operand vf[TILES_AHEAD + 1][NKB];
+#pragma unroll
+    for (int a = 0; a < TILES_AHEAD; ++a)
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb) vf[a][kb] = load_operand<T>(v_tile + (16 * a + i) * VS + KB * kb + VEC * g);
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
+      if constexpr (TILES_AHEAD > 0) {
+        if (c + TILES_AHEAD < NC) {
+#pragma unroll
+          for (int kb = 0; kb < NKB; ++kb) vf[(c + TILES_AHEAD) % (TILES_AHEAD + 1)][kb] = load_operand<T>(v_tile + (16 * (c + TILES_AHEAD) + i) * VS + KB * kb + VEC * g);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) acc_o[ct][c] = acc_o[ct][c] * alpha[ct];
 #pragma unroll
       for (int kb = 0; kb < NKB; ++kb) {
-        const Operand vf = load_operand<T>(v_tile + (16 * c + i) * VS + KB * kb + VEC * g);
+        if constexpr (TILES_AHEAD == 0) vf[0][kb] = load_operand<T>(v_tile + (16 * c + i) * VS + KB * kb + VEC * g);
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) acc_o[ct][c] = B::mma(vf, pf[ct][kb], acc_o[ct][c]);
+        for (int ct = 0; ct < CT; ++ct) acc_o[ct][c] = B::mma(vf[c % (TILES_AHEAD + 1)][kb], pf[ct][kb], acc_o[ct][c]);
       }
-    }
-  };
-
-  __syncthreads();  // page ids are in place
-  if constexpr (!DB) {
-  // iteration `it` covers tiles tile_lo + it * KSPLIT .. + KSPLIT - 1, one per set (the last iteration may leave a set without one)
-  const int iterations = tile_hi > tile_lo ? (tile_hi - tile_lo + KSPLIT - 1) / KSPLIT : 0;
-  if (tile_lo + set < tile_hi) fetch(n_begin + (tile_lo + set) * BN);
-  for (int it = 0; it < iterations; ++it) {
-    const int tile = tile_lo + it * KSPLIT + set;
-    const bool have_tile = KSPLIT == 1 || tile < tile_hi;
-    const int n0 = n_begin + tile * BN;
-    __syncthreads();  // the previous tile has been read by every wave
-    if (have_tile) commit(n0);
-    __syncthreads();
-    if (it + 1 < iterations) {
-      const int next_first = n_begin + (tile_lo + (it + 1) * KSPLIT) * BN;  // first key of the next iteration's tiles
-      if (((next_first + KSPLIT * BN - 1) >> page_shift) - first_page >= PREFILL_PAGE_IDS) {  // the same for every thread
-        first_page = next_first >> page_shift;
-        load_page_ids();
-        __syncthreads();
-      }
-      if (tile + KSPLIT < tile_hi) fetch(n0 + KSPLIT * BN);  // in flight while this tile is computed
-    }
-    if (!have_tile || n0 > wave_last_pos) continue;  // nothing this wave may read; it still took part in the staging
-    process(n0);
-  }
-  }
-
-  if constexpr (DB) {
-    // Two tile buffers: while the waves compute on one, the next tile is written into the other, so the waves meet at one
-    // barrier per tile instead of two.  Tile `it` lives in buffer it % 2; its registers were asked for an iteration ago.
-    T* const base = reinterpret_cast<T*>(smem);
-    const int iterations = tile_hi > tile_lo ? tile_hi - tile_lo : 0;
-    if (iterations > 0) {
-      fetch(n_begin + tile_lo * BN);
-      commit(n_begin + tile_lo * BN);
-      if (iterations > 1) fetch(n_begin + (tile_lo + 1) * BN);
-    }
-    __syncthreads();
-    for (int it = 0; it < iterations; ++it) {
-      const int n0 = n_begin + (tile_lo + it) * BN;
-      if (it + 1 < iterations) {
-        k_tile = base + ((it + 1) & 1) * TILE_ELEMS;
-        v_tile = k_tile + BN * KS;
-        commit(n0 + BN);  // read last in iteration it - 1, which every wave has left
-        if (it + 2 < iterations) {
-          const int next_first = n0 + 2 * BN;
-          if (((next_first + BN - 1) >> page_shift) - first_page >= PREFILL_PAGE_IDS) {  // the same for every thread
-            __syncthreads();
-            first_page = next_first >> page_shift;
-            load_page_ids();
-            __syncthreads();
-          }
-          fetch(next_first);
-        }
-      }
-      k_tile = base + (it & 1) * TILE_ELEMS;
-      v_tile = k_tile + BN * KS;
-      if (n0 <= wave_last_pos) process(n0);
-      __syncthreads();
     }
   }
 
@@ -851,9 +836,6 @@ static int compute_units() {
   return cached;
 }
 
-static int g_experiment = 0;
-extern "C" void velox_attention_experiment(int variant) { g_experiment = variant; }
-
 template <typename T> constexpr int tile_keys() { return (sizeof(T) * D > 512) ? 32 : 64; }
 
 template <typename T>
@@ -887,40 +869,6 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
   // keys 315 us against 426 the other way round; the two meet where an average row reads about 1,300 keys.
   constexpr int WIDE = (sizeof(T) == 2 && D <= 128) ? 2 : 1;
   const int rows = max_q_len * group;
-  if (WIDE == 2 && g_experiment > 0) {
-    if (g_experiment == 1) {
-      dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
-      paged_attention_kernel<T, BN, WIDE, 1, 4><<<grid, 256, 0, stream>>>(
-          (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
-    } else if (g_experiment == 4) {
-      dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
-      paged_attention_kernel<T, BN, 1, 1, 8, 1><<<grid, 512, 0, stream>>>(
-          (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
-    } else if (g_experiment == 5) {
-      dim3 grid((rows + 255) / 256, nkv, num_seqs * splits);
-      paged_attention_kernel<T, BN, WIDE, 1, 8, 1><<<grid, 512, 0, stream>>>(
-          (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
-    } else if (g_experiment == 6) {
-      dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
-      paged_attention_kernel<T, BN, WIDE, 1, 4, 1><<<grid, 256, 0, stream>>>(
-          (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
-    } else if (g_experiment == 2) {
-      dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
-      paged_attention_kernel<T, BN, WIDE, WIDE, 4><<<grid, 512, 0, stream>>>(
-          (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
-    } else {
-      dim3 grid((rows + 63) / 64, nkv, num_seqs * splits);
-      paged_attention_kernel<T, BN, 1, WIDE, 4><<<grid, 512, 0, stream>>>(
-          (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
-    }
-    return (int)hipGetLastError();
-  }
   if (WIDE == 2 && rows > 64 && (long long)total_tokens * group / 128 * nkv * splits >= compute_units()) {
     if (max_kv_len - max_q_len / 2 <= 1280 || rows < 192) {  // (keys an average row reads)
       dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
