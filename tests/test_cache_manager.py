@@ -160,3 +160,18 @@ def test_random_orders_of_requests(seed):
         m.free_sequence(seq)
     m.assert_consistent([])
     assert m.num_used_pages() == 0 and m.state.num_free == 5
+
+
+def test_pool_size_from_free_memory():
+    """Reference ``src/paged_kv_cache.py:183-194``: (free bytes x utilisation - reserve) / bytes per page, rounded down."""
+    from velox_amd.cache.manager import pages_that_fit
+
+    per_page = 2 * 16 * 4 * 128 * 2 * 28  # keys and values, 16 tokens, 4 KV heads of 128, bfloat16, 28 layers
+    assert pages_that_fit(per_page, 100 << 30, 0.9, 512 << 20) == (int((100 << 30) * 0.9) - (512 << 20)) // per_page
+    assert pages_that_fit(per_page, 10 * per_page + 1000, 1.0, 1000) == 10
+    with pytest.raises(RuntimeError, match="not enough free GPU memory"):
+        pages_that_fit(per_page, 1 << 20, 0.5, 1 << 20)
+    with pytest.raises(RuntimeError, match="even one cache page"):
+        pages_that_fit(per_page, per_page + 10, 1.0, 0)
+    m = CacheManager([PagedNeed(4, 128)] * 28, 16, 2, 4, torch.bfloat16, "cpu", allocate_tensors=False)
+    assert m.bytes_per_page() == per_page

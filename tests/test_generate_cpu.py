@@ -120,7 +120,7 @@ def test_launching_the_next_step_early_changes_no_token(tmp_path, name):
         engine = engine_for(folder, name, decode_lookahead=lookahead)
         launches = []
         inner = engine.runner.step
-        engine.runner.step = lambda entries, ids_on_device=None: (launches.append(ids_on_device is not None), inner(entries, ids_on_device=ids_on_device))[1]
+        engine.runner.step = lambda entries, device_ids=None: (launches.append(device_ids is not None), inner(entries, device_ids=device_ids))[1]
         done = engine.generate(requests("on-" if lookahead else "off-"))
         results[lookahead] = [(r.output_token_ids, r.finish_reason) for r in done]
         assert any(launches) == lookahead
@@ -197,3 +197,57 @@ def test_requests_and_aborts_from_another_thread(tmp_path):
     assert twin.finish_reason is FinishReason.ABORT and not again.finished
     assert engine.abort_all() == "aborted" and not engine.has_work()
     assert engine.cache.num_used_pages() == 0
+
+
+@pytest.mark.parametrize("prefix_caching", [False, True])
+def test_every_kind_of_step_is_launched_early_also_with_preemption_and_late_arrivals(tmp_path, prefix_caching):
+    """A pool so small that requests are preempted and recomputed, prompts that take several portions, a request that
+    arrives while others decode, one that stops on a token in flight: with the next step always launched before this one's
+    tokens are read, every request ends with the plain model's tokens, as with one step at a time."""
+    folder = make_folder(tmp_path, "B")
+    config, weights = read_model_folder(folder)
+    page = PAGE_SIZE["B"]
+    stem = random_tokens(config["vocab_size"], 2 * page + 1, seed=70)
+    prompts = [stem + random_tokens(config["vocab_size"], n, seed=71 + n) for n in (3, 14, 1, 9, 22)]
+    steps = 12
+    expected = [plain_greedy(config, weights, p, steps) for p in prompts]
+    stop_at = expected[3][6]
+    needed = max((len(p) + steps + page - 1) // page for p in prompts)
+
+    def run(lookahead):
+        engine = engine_for(folder, "B", decode_lookahead=lookahead, num_gpu_blocks=2 * needed + 2, max_model_len=needed * page,
+                            enable_prefix_caching=prefix_caching, max_num_batched_tokens=16, max_prefill_chunk_size=6)
+        requests = greedy(prompts, steps, prefix=f"{lookahead}-")
+        requests[3] = Request(f"{lookahead}-stop", prompts[3], SamplingParams(temperature=0.0, max_tokens=steps, stop_token_ids=[stop_at]))
+        early = {"portions": 0, "pending": 0}
+        inner = engine._launch
+
+        def launch(plan, pending=None):
+            if pending is not None:
+                early["portions"] += len(plan.portions)
+                early["pending"] += 1
+            return inner(plan, pending=pending)
+
+        engine._launch = launch
+        for request in requests[:3]:
+            engine.add_request(request)
+        for _ in range(4):
+            engine.step()
+        for request in requests[3:]:
+            engine.add_request(request)  # arrive while the others run
+        while engine.has_work():
+            engine.step()
+            engine.cache.assert_consistent([r.cache for r in engine.scheduler.running if r.cache is not None])
+        assert engine.cache.num_used_pages() == (engine.cache.prefix.num_nodes if prefix_caching else 0)
+        assert (early["pending"] > 0) == lookahead and (early["portions"] > 0) == lookahead
+        return requests, (engine.scheduler.num_preemptions, engine.cache.prefix.num_hits if prefix_caching else 0)
+
+    ahead, (preemptions, hits) = run(True)
+    plain, _ = run(False)
+    assert hits > 0 if prefix_caching else preemptions > 0  # (with the stem shared the pool is large enough)
+    cut = expected[3].index(stop_at) + 1
+    for index, (a, b) in enumerate(zip(ahead, plain)):
+        want = expected[index][:cut] if index == 3 else expected[index]
+        assert a.output_token_ids == want and b.output_token_ids == want, (index, a.output_token_ids, b.output_token_ids, want)
+        assert a.finish_reason is (FinishReason.STOP if index == 3 else FinishReason.LENGTH) and a.finish_reason is b.finish_reason
+        assert -1 not in a.all_token_ids

@@ -119,7 +119,7 @@ def test_launching_the_next_step_early_changes_no_token(tmp_path, graphs):
         engine = engine_for(folder, "B", "float32", enable_cuda_graphs=graphs, decode_lookahead=lookahead)
         launches = []
         inner = engine.runner.step
-        engine.runner.step = lambda entries, ids_on_device=None: (launches.append(ids_on_device is not None), inner(entries, ids_on_device=ids_on_device))[1]
+        engine.runner.step = lambda entries, device_ids=None: (launches.append(device_ids is not None), inner(entries, device_ids=device_ids))[1]
         done = engine.generate(requests("on-" if lookahead else "off-"))
         results[lookahead] = [(r.output_token_ids, r.finish_reason) for r in done]
         assert any(launches) == lookahead
@@ -327,6 +327,29 @@ def test_sampling_through_the_engine(tmp_path):
     for request, history, c in zip(penalised, histories, coefficients):
         assert request.output_token_ids == plain_penalised(history, 10, **c), request.request_id
     assert penalised[0].output_token_ids != plain_penalised(histories[0], 10)  # the penalties changed what is chosen
+
+
+def test_pool_sized_from_free_memory_when_no_page_count_is_given(tmp_path):
+    """``num_gpu_blocks=None``: the pool takes what the free memory allows (reference ``src/paged_kv_cache.py:159-194``), capped at
+    what ``max_num_seqs`` requests of ``max_model_len`` tokens can ever hold; a utilisation that leaves nothing is an error."""
+    folder = make_folder(tmp_path, "A", "bfloat16")
+    engine = engine_for(folder, "A", "bfloat16", num_gpu_blocks=None, gpu_memory_utilization=0.5, max_model_len=160, max_num_seqs=4)
+    page = PAGE_SIZE["A"]
+    assert engine.cache.num_total_pages == 4 * 160 // page  # the cap: far less than half of the card
+    config, weights = read_model_folder(folder)
+    prompt = random_tokens(config["vocab_size"], 30, seed=3)
+    assert len(engine.generate(greedy([prompt], 6))[0].output_token_ids) == 6
+    free_bytes, _ = torch.cuda.mem_get_info()
+    from velox_amd.cache.manager import pages_that_fit
+
+    with pytest.raises(RuntimeError, match="not enough free GPU memory"):
+        pages_that_fit(engine.cache.bytes_per_page(), free_bytes, 0.5, free_bytes)
+    # uncapped: a long context and many requests want more pages than fit in a sliver of the free memory
+    small = engine_for(folder, "A", "bfloat16", num_gpu_blocks=None, gpu_memory_utilization=0.9, kv_cache_reserve_mb=0, max_model_len=512, max_num_seqs=32,
+                       max_num_batched_tokens=64)
+    wanted = 32 * 512 // page
+    assert small.cache.num_total_pages == wanted  # still the cap on this card; the arithmetic below is what a small card would get
+    assert pages_that_fit(small.cache.bytes_per_page(), 3 * small.cache.bytes_per_page() + 5, 1.0, 0) == 3
 
 
 def test_command_line(tmp_path):

@@ -222,64 +222,39 @@ def test_a_victim_leaves_the_step_it_was_already_given_a_token_in():
     assert len(a.output_token_ids) == 2 and len(b.output_token_ids) == 9
 
 
-def decoding(s, lengths, max_tokens=8):
-    """Requests read in whole and given their first token: all decoding."""
-    requests = [request(f"d{i}", n, max_tokens) for i, n in enumerate(lengths)]
-    for r in requests:
-        s.add_request(r)
-    while any(r.status is not RequestStatus.RUNNING_DECODE for r in requests):
-        run_step(s, s.schedule())
-    return requests
+def test_a_step_can_be_decided_while_the_tokens_of_the_one_before_are_pending():
+    """What the engine does with a step in flight: positions advance and each sampled request gets a pending token at once;
+    on that state the next step is decided.  A request that reaches its length with the pending token is closed: it is
+    dropped at the next decision, and its token still arrives."""
+    from velox_amd.engine.request import PENDING_TOKEN
 
-
-def test_the_next_decode_step_can_be_fixed_while_one_is_in_flight():
-    s = make(pages=33, page=4, budget=16)
-    requests = decoding(s, [3, 4, 7])
-    out = s.schedule()  # a decode-only step: "in flight" until run_step books it
-    assert out.decodes == requests and not out.portions
-    pages_before = [len(r.cache.tables[0]) for r in requests]
-    ahead = s.schedule_ahead(out.decodes)
-    assert ahead == requests
-    # every table now covers the position after the one in flight
-    for r, before in zip(requests, pages_before):
-        assert len(r.cache.tables[0]) * 4 >= r.num_computed_tokens + 2 and len(r.cache.tables[0]) - before in (0, 1)
-    run_step(s, out)
-    # the step fixed ahead runs next, without schedule(): its pages are there
-    for r in ahead:
-        assert len(r.cache.tables[0]) * 4 >= r.num_computed_tokens + 1
-        s.advance(r, 1)
-        r.record_token(7)
-    s.cache.assert_consistent([r.cache for r in requests])
-
-
-def test_nothing_is_fixed_ahead_when_the_next_step_could_look_different():
-    # somebody waits
-    s = make(pages=33, page=4, seqs=2, budget=16)
-    requests = decoding(s, [3, 4])
-    s.add_request(request("late", 5))
-    out = s.schedule()  # both slots are taken: the late request waits
-    assert not out.portions and len(s.waiting) == 1
-    assert s.schedule_ahead(out.decodes) is None
-    # a request reaches its length limit with the token in flight
-    s = make(pages=33, page=4, budget=16)
-    requests = decoding(s, [3, 4], max_tokens=2)  # one token each so far
-    out = s.schedule()
-    assert s.schedule_ahead(out.decodes) is None
-    # not every running request is in the step
-    s = make(pages=33, page=4, budget=16)
-    requests = decoding(s, [3, 4, 5])
-    out = s.schedule()
-    assert s.schedule_ahead(out.decodes[:2]) is None
-    # pages are short: both requests sit at the end of a page and one page is free; nothing may be taken
-    s = make(pages=4, page=4, budget=16, watermark=0.01)  # 3 usable pages
-    requests = decoding(s, [3, 3])  # 4 tokens each after the first sampled one: position 4 needs a second page
-    out = s.schedule()
-    assert len(out.decodes) == 2
-    if True:
-        free_before = s.cache.groups[0].allocator.num_free
-        tables = [list(r.cache.tables[0]) for r in requests]
-        assert s.schedule_ahead(out.decodes) is None
-        assert s.cache.groups[0].allocator.num_free == free_before and [list(r.cache.tables[0]) for r in requests] == tables
+    s = make(pages=33, page=4, budget=16, chunk=8)
+    a, b = request("a", 6, max_tokens=2), request("b", 11, max_tokens=5)
+    s.add_request(a)
+    s.add_request(b)
+    first = s.schedule()  # a whole (6), b's first 8
+    assert portions(first) == [("a", 6), ("b", 8)]
+    # booked before its tokens are known
+    for p in first.portions:
+        s.advance(p.request, p.count)
+    slot = a.expect_token()
+    assert a.output_token_ids == [PENDING_TOKEN] and a.status is RequestStatus.RUNNING_DECODE and not a.finished
+    second = s.schedule()  # decided with a's token pending: a decodes, b goes on
+    assert second.decodes == [a] and portions(second) == [("b", 3)] and a.all_token_ids[a.num_computed_tokens] == PENDING_TOKEN
+    a.deliver_token(slot, 41)
+    assert a.output_token_ids == [41] and a.all_token_ids[-1] == 41
+    # the second step in flight: a's second token is its last
+    s.advance(a, 1)
+    s.advance(b, 3)
+    slot_a, slot_b = a.expect_token(), b.expect_token()
+    assert a.closing and a.finished and a.finish_reason is None and a.status is RequestStatus.FINISHED and not b.closing
+    third = s.schedule()
+    assert third.decodes == [b] and a not in s.running and a.cache is None and s.num_finished == 1
+    a.deliver_token(slot_a, 42)
+    a.finish(a.stop_reason(42, frozenset()))
+    b.deliver_token(slot_b, 7)
+    assert a.finish_reason is FinishReason.LENGTH and a.output_token_ids == [41, 42] and b.output_token_ids == [7]
+    s.cache.assert_consistent([b.cache])
 
 
 def test_listeners_hear_tokens_and_the_end_and_may_fail():

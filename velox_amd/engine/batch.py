@@ -133,17 +133,18 @@ class BatchBuilder:
 
     def section_total(self, t: int, b: int, r: int, w: int) -> int:
         n_groups = len(self.cache.groups)
-        return _align(t) * 2 + _align(b + 1) + _align(b) * 2 + _align(r) + n_groups * (_align(b) + _align(t) + _align(b * w))
+        return _align(t) * 2 + _align(b + 1) + _align(b) * 2 + _align(2 * b) + _align(r) + n_groups * (_align(b) + _align(t) + _align(b * w))
 
     def build(self, entries: Sequence[StepEntry], ops, dtype, workspace: Workspace, device_buffer: Optional[torch.Tensor] = None, pad_to: Optional[int] = None, width: Optional[int] = None,
-              ids_on_device: Optional[tuple] = None) -> StepContext:
+              device_ids: Optional[tuple] = None) -> StepContext:
         """Lays the step out.  ``pad_to``/``width``/``device_buffer`` are for captured decode steps:
         the batch is padded to ``pad_to`` one-token rows that read and write the null page, the
         block table has the fixed ``width``, and the sections land in the caller's buffer.
 
-        ``ids_on_device = (tokens int32 [R] on the device, rows)``: every entry has one token and entry ``i``'s is
-        ``tokens[rows[i]]``, which the host may not know yet; it is copied into place on the device, after the
-        staging copy, in stream order."""
+        ``device_ids = (tokens int32 [R] on the device, dest_rows, source_rows)``: token ids that the host does not know
+        yet (the step that samples them is still in flight): row ``dest_rows[k]`` of this step's tokens is
+        ``tokens[source_rows[k]]``; the entries hold a placeholder there.  They are copied into place on the device, behind
+        the staging copy, in stream order."""
         cache = self.cache
         page = cache.page_size
         b_real = len(entries)
@@ -209,12 +210,24 @@ class BatchBuilder:
         put("cu", cu, b + 1)
         put("slots", slots, b)
         put("rows", np.asarray(rows, dtype=np.int32), r)
-        source = np.zeros(b, dtype=np.int32)  # always laid out: a captured step reads its sections at fixed places
-        if ids_on_device is not None:
-            if t != b or len(ids_on_device[1]) != b_real:
-                raise ValueError("token ids on the device need one token per entry and one source row per entry")
-            source[:b_real] = np.asarray(ids_on_device[1], dtype=np.int32)
+        # always laid out: a captured step reads its sections at fixed places.  At most one token per entry is still to
+        # come (its newest); dest is laid out as 64-bit integers, which is what the scatter on the device takes
+        source = np.zeros(b, dtype=np.int32)
+        dest = np.zeros(2 * b, dtype=np.int32)
+        num_device_ids = 0
+        if device_ids is not None:
+            tokens_on_device, dest_rows, source_rows = device_ids
+            num_device_ids = len(dest_rows)
+            if num_device_ids != len(source_rows) or num_device_ids > b_real:
+                raise ValueError("token ids on the device: one source row per destination row, at most one per entry")
+            if num_device_ids and (min(dest_rows) < 0 or max(dest_rows) >= t or min(source_rows) < 0 or max(source_rows) >= tokens_on_device.shape[0]):
+                raise ValueError("token ids on the device: a row outside the step or outside the sampled tokens")
+            if tokens_on_device.dtype != torch.int32 or tokens_on_device.dim() != 1:
+                raise ValueError("token ids on the device must be int32 [R]")
+            source[:num_device_ids] = np.asarray(source_rows, dtype=np.int32)
+            dest[0:2 * num_device_ids:2] = np.asarray(dest_rows, dtype=np.int32)
         put("source", source, b)
+        put("dest", dest, 2 * b)
         max_kv: List[int] = []
         max_kv_portions: List[int] = []
         decode_prefix = next((i for i, n in enumerate(q_lens) if n != 1), len(q_lens))
@@ -250,11 +263,9 @@ class BatchBuilder:
             lo, n = sections[name]
             return device[lo:lo + n]
 
-        if ids_on_device is not None:
-            tokens = ids_on_device[0]
-            if tokens.dtype != torch.int32 or tokens.dim() != 1 or int(max(ids_on_device[1])) >= tokens.shape[0] or min(ids_on_device[1]) < 0:
-                raise ValueError("token ids on the device must be int32 [R] and every source row inside it")
-            torch.index_select(tokens, 0, view("source")[:b_real], out=view("ids")[:b_real])
+        if num_device_ids:
+            gathered = torch.index_select(device_ids[0], 0, view("source")[:num_device_ids])
+            view("ids").index_copy_(0, view("dest")[:2 * num_device_ids].view(torch.int64), gathered)
 
         groups = [
             GroupBatch(

@@ -27,9 +27,9 @@ from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from ..weights import bind_from_checkpoint, bind_random
 from .batch import StepEntry
-from .request import FinishReason, Request
+from .request import PENDING_TOKEN, FinishReason, Request
 from .runner import ModelRunner
-from .scheduler import Portion, Scheduler, SchedulerConfig
+from .scheduler import Portion, Scheduler, SchedulerConfig, StepPlan
 
 @dataclass
 class _Flight:
@@ -40,6 +40,11 @@ class _Flight:
     sampled: List[Request]  # the requests whose rows were sampled, in row order
     tokens: Optional[torch.Tensor]  # int32 [len(sampled)] on the device
     landing: Optional[tuple] = None  # (pinned host tensor the tokens are copied to, event recorded behind the copy)
+    booked: bool = False  # positions advanced and room made for the sampled tokens (Engine._book)
+    expected: Optional[List[Optional[int]]] = None  # per sampled row: the token's index in the request's output, None = nobody waits for it
+
+    def requests(self) -> List[Request]:
+        return self.decode + [portion.request for portion in self.prefill]
 
 
 logger = logging.getLogger(__name__)
@@ -242,29 +247,35 @@ class Engine:
     # -- one step -----------------------------------------------------------------------
     @torch.no_grad()
     def step(self) -> None:
-        """One step of every scheduled request.  When it returns, each of them holds its new token.  With
-        ``decode_lookahead`` the NEXT step may already be running by then: while the device works on a decode-only
-        step, the host fixes that step's successor (``Scheduler.schedule_ahead``), lays it out and launches it with
-        the token ids taken on the device from this step's sampler output, and only then waits for this step's
-        tokens.  The device so never waits for the host between decode steps.  A request that stops on a token that
-        was still in flight has a row in the successor that nobody reads."""
+        """One step of every scheduled request.  When it returns, each of them holds its new token.
+
+        With ``decode_lookahead`` the NEXT step is already running by then.  As soon as a step is queued, everything about
+        it that does not depend on the values of the tokens it samples is booked: positions advance, and each sampled
+        request gets a pending token in its lists (``Request.expect_token``; a request that reaches its length with it is
+        closed).  On that state the scheduler decides the next step, of any kind (prompt portions, admissions,
+        preemptions, decodes), and it is queued with the pending tokens' values taken on the device from this step's
+        sampler output.  Only then does the host wait for this step's tokens.  The device so never waits for the host to
+        schedule, lay out and launch, between decode steps (the reference's 1.5 ms gap per step) or between the steps of
+        long prompts.  A request that stops on a token that was still in flight has a row in the successor that nobody
+        reads; what it held goes back at the next scheduling decision (anything a later owner of those pages does
+        comes, in stream order, behind that row's writes)."""
         step_start = time.perf_counter()
         self._drain_control_queue()
         flight, self._ahead = self._ahead, None
-        if flight is not None and not any(self._alive(r) for r in flight.sampled):
+        if flight is not None and not any(self._alive(r) for r in flight.requests()):
             flight = None  # launched for requests that have all stopped or been aborted since
         if flight is None:
             scheduled = self.scheduler.schedule()
             self.stats["scheduler_ms"].append((time.perf_counter() - step_start) * 1000)
             if scheduled.is_empty():
                 return
-            flight = self._launch(scheduled.decodes, scheduled.portions)
-        if self.config.decode_lookahead and flight.tokens is not None and not flight.prefill:
-            alive = [(row, r) for row, r in enumerate(flight.sampled) if self._alive(r)]
-            if alive and not any(r.sampling_params.has_penalties for _, r in alive):
-                ahead = self.scheduler.schedule_ahead([r for _, r in alive])
-                if ahead is not None:
-                    self._ahead = self._launch(ahead, [], ids_on_device=(flight.tokens, [row for row, _ in alive]))
+            flight = self._launch(scheduled)
+        if self.config.decode_lookahead and not any(r.sampling_params.has_penalties for r in self.scheduler.running):
+            # (penalties read a request's history on the host: they need the token's value)
+            self._book(flight)
+            ahead = self.scheduler.schedule()
+            if not ahead.is_empty():
+                self._ahead = self._launch(ahead, pending=flight)
         self._finish_step(flight)
         self.num_steps += 1
         self.stats["step_ms"].append((time.perf_counter() - step_start) * 1000)
@@ -273,27 +284,39 @@ class Engine:
     def _alive(request: Request) -> bool:
         return not request.finished and request.cache is not None
 
-    def _launch(self, decode: List[Request], prefill: List[Portion], ids_on_device=None) -> "_Flight":
-        """Queues one step on the device: the forward over the batch and the sampler.  With ``ids_on_device`` the step
-        before this one has not been finished on the host yet: every request is one position and one generated token
-        further than its fields say."""
-        ahead = 1 if ids_on_device is not None else 0
+    def _launch(self, plan: StepPlan, pending: Optional["_Flight"] = None) -> "_Flight":
+        """Queues one step on the device: the forward over the batch and the sampler.  ``pending``: the step before this
+        one, booked but not finished: its sampled tokens are pending in the requests' lists, and their values are taken on
+        the device from its sampler's output."""
         entries: List[StepEntry] = []
         sampled: List[Request] = []
+        dest_rows: List[int] = []
+        source_rows: List[int] = []
+        source_of = {id(r): row for row, r in enumerate(pending.sampled)} if pending is not None else {}
+        at = 0  # rows of the step so far
         # decode rows first, then prompt portions; only rows that complete their tokens are sampled
-        for request in decode:
-            start = request.num_computed_tokens + ahead
-            token = 0 if ahead else request.all_token_ids[start]
+        for request in plan.decodes:
+            start = request.num_computed_tokens
+            token = request.all_token_ids[start]
+            if token == PENDING_TOKEN:
+                dest_rows.append(at)
+                source_rows.append(source_of[id(request)])
             entries.append(StepEntry(request.cache, [token], start, [0]))
             sampled.append(request)
-        for portion in prefill:
+            at += 1
+        for portion in plan.portions:
             request, start, count = portion.request, portion.start, portion.count
-            entries.append(StepEntry(request.cache, request.all_token_ids[start:start + count], start, [count - 1] if portion.completes else []))
+            tokens = request.all_token_ids[start:start + count]
+            if tokens[-1] == PENDING_TOKEN:  # (only a request's newest token can be pending)
+                dest_rows.append(at + count - 1)
+                source_rows.append(source_of[id(request)])
+            entries.append(StepEntry(request.cache, tokens, start, [count - 1] if portion.completes else []))
             if portion.completes:
                 sampled.append(request)
+            at += count
 
         t0 = time.perf_counter()
-        logits = self.runner.step(entries, ids_on_device=ids_on_device)
+        logits = self.runner.step(entries, device_ids=(pending.tokens, dest_rows, source_rows) if dest_rows else None)
         self.stats["forward_ms"].append((time.perf_counter() - t0) * 1000)
 
         tokens_gpu = None
@@ -304,7 +327,7 @@ class Engine:
                 logits,
                 [r.sampling_params for r in sampled],
                 [r.request_id for r in sampled],
-                [len(r.output_token_ids) + ahead for r in sampled],
+                [len(r.output_token_ids) for r in sampled],
                 histories=[r.all_token_ids for r in sampled] if needs_history else None,
             )
             self.stats["sampling_ms"].append((time.perf_counter() - t0) * 1000)
@@ -316,30 +339,42 @@ class Engine:
             self._next_landing = (self._next_landing + 1) % len(self._landings)
             landing[0][: len(sampled)].copy_(tokens_gpu, non_blocking=True)
             landing[1].record()
-        return _Flight(list(decode), list(prefill), sampled, tokens_gpu, landing)
+        return _Flight(list(plan.decodes), list(plan.portions), sampled, tokens_gpu, landing)
 
-    def _finish_step(self, flight: "_Flight") -> None:
-        """Waits for the step's tokens and books them: positions computed, tokens appended, stops."""
-        tokens: List[int] = []
-        if flight.tokens is not None:
-            sync_start = time.perf_counter()
-            # the one place per step where the host waits for the device
-            if flight.landing is not None:
-                flight.landing[1].synchronize()
-                tokens = flight.landing[0][: len(flight.sampled)].tolist()
-            else:
-                tokens = flight.tokens.tolist()
-            self.stats["cpu_sync_wait_ms"].append((time.perf_counter() - sync_start) * 1000)
+    def _book(self, flight: "_Flight") -> None:
+        """What a queued step changes whatever tokens it draws: its positions are in the cache, and every sampled request
+        has one more token (pending until the step's tokens arrive)."""
+        if flight.booked:
+            return
+        flight.booked = True
         for request in flight.decode:
             if self._alive(request):
                 self.scheduler.advance(request, 1)
         for portion in flight.prefill:
             if self._alive(portion.request):
                 self.scheduler.advance(portion.request, portion.count)
-        for request, token in zip(flight.sampled, tokens):
-            if not self._alive(request):
-                continue  # stopped or aborted while this step was in flight
-            request.record_token(int(token))
+        flight.expected = [request.expect_token() if self._alive(request) else None for request in flight.sampled]
+
+    def _finish_step(self, flight: "_Flight") -> None:
+        """Waits for the step's tokens and hands them to their requests; stops."""
+        self._book(flight)
+        if flight.tokens is None:
+            return
+        sync_start = time.perf_counter()
+        # the one place per step where the host waits for the device
+        if flight.landing is not None:
+            flight.landing[1].synchronize()
+            tokens = flight.landing[0][: len(flight.sampled)].tolist()
+        else:
+            tokens = flight.tokens.tolist()
+        self.stats["cpu_sync_wait_ms"].append((time.perf_counter() - sync_start) * 1000)
+        for request, index, token in zip(flight.sampled, flight.expected, tokens):
+            if index is None:
+                continue  # it had stopped or been aborted before this step was booked
+            aborted = request.finish_reason is FinishReason.ABORT
+            request.deliver_token(index, int(token), announce=not aborted)
+            if aborted:
+                continue
             reason = request.stop_reason(int(token), self.eos_token_ids)
             if reason is not None:
                 request.finish(reason)

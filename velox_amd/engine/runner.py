@@ -87,18 +87,18 @@ class ModelRunner:
 
     # -- the step -----------------------------------------------------------------------
     @torch.no_grad()
-    def step(self, entries: Sequence[StepEntry], ids_on_device: Optional[tuple] = None) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], device_ids: Optional[tuple] = None) -> Optional[torch.Tensor]:
         """Runs the entries' tokens as one batch; returns float32 logits ``[wanted, vocab]``
         in the order of the entries and of their ``want`` (None when nothing is wanted).
-        ``ids_on_device``: see ``BatchBuilder.build`` (the entries' own ``token_ids`` are placeholders then)."""
+        ``device_ids``: see ``BatchBuilder.build`` (token ids that are still being sampled by the step in flight)."""
         if self.enable_graphs and all(len(e.token_ids) == 1 for e in entries):
             if all(list(e.want) == [0] for e in entries):
                 bucket = self._bucket_for(len(entries))
                 if bucket is not None:
-                    return self._replay(bucket, entries, ids_on_device)
-        if self.tuned_row_counts and ids_on_device is None:
+                    return self._replay(bucket, entries, device_ids)
+        if self.tuned_row_counts:
             entries = self._padded_to_tuned_rows(entries)
-        ctx = self.builder.build(entries, self.ops, self.dtype, self.workspace, ids_on_device=ids_on_device)
+        ctx = self.builder.build(entries, self.ops, self.dtype, self.workspace, device_ids=device_ids)
         return self._forward(ctx)
 
     def _padded_to_tuned_rows(self, entries: Sequence[StepEntry]) -> Sequence[StepEntry]:
@@ -129,12 +129,12 @@ class ModelRunner:
                 return bucket
         return None
 
-    def _padded_entries_context(self, bucket: int, entries: Sequence[StepEntry], ids_on_device: Optional[tuple] = None) -> StepContext:
+    def _padded_entries_context(self, bucket: int, entries: Sequence[StepEntry], device_ids: Optional[tuple] = None) -> StepContext:
         buffer = self._graph_buffers[bucket]
         padded = [StepEntry(e.seq, e.token_ids, e.start, [0]) for e in entries]
         ctx = self.builder.build(
             padded, self.ops, self.dtype, self.workspace,
-            device_buffer=buffer, pad_to=bucket, width=self.builder.width, ids_on_device=ids_on_device,
+            device_buffer=buffer, pad_to=bucket, width=self.builder.width, device_ids=device_ids,
         )
         return ctx
 
@@ -209,12 +209,12 @@ class ModelRunner:
         ctx = self.builder.build([StepEntry(null_seq, [0] * num_tokens, 0, [num_tokens - 1])], self.ops, self.dtype, self.workspace)
         self._forward(ctx)
 
-    def _replay(self, bucket: int, entries: Sequence[StepEntry], ids_on_device: Optional[tuple] = None) -> torch.Tensor:
+    def _replay(self, bucket: int, entries: Sequence[StepEntry], device_ids: Optional[tuple] = None) -> torch.Tensor:
         graph, logits, _ = self._graphs[bucket]
         if bucket in self._short_graphs and all(e.start < SHORT_CONTEXT_KEYS for e in entries):
             graph, logits, _ = self._short_graphs[bucket]
             self.num_short_graph_replays += 1
-        self._padded_entries_context(bucket, entries, ids_on_device)  # refreshes the bucket's buffer in place
+        self._padded_entries_context(bucket, entries, device_ids)  # refreshes the bucket's buffer in place
         graph.replay()
         self.num_graph_replays += 1
         return logits[: len(entries)]

@@ -178,41 +178,6 @@ class Scheduler:
         self._admit_waiting(plan, budget)
         return plan
 
-    def schedule_ahead(self, in_flight: List[Request]) -> Optional[List[Request]]:
-        """The decode step after the one in flight, decided before that one's tokens are known (not in the reference,
-        which waits for every step's tokens before it schedules the next).
-
-        ``in_flight`` are the requests of a decode-only step that has been launched but whose tokens have not been
-        appended yet: each will hold one token more than ``all_token_ids`` shows and one computed position more than
-        ``num_computed_tokens``.  The next step can be fixed now only if nothing else could claim a place in it: no
-        request waits, every running request is one of ``in_flight`` and keeps decoding whatever token it draws (its
-        length limit is not reached by the token in flight), and every one finds its next page without preemption.
-        Then the requests' tables are grown and the list comes back (order kept); otherwise None, and nothing has
-        changed.  A request that stops on the token in flight has then been given a place it does not use: the caller
-        drops its row, and its pages go back when it leaves ``running``."""
-        self._drop_finished()
-        if self.waiting or not in_flight or len(self.running) != len(in_flight) or len(in_flight) > self.config.max_num_batched_tokens:
-            return None
-        chosen = set(id(r) for r in in_flight)
-        needed = [0] * len(self.cache.groups)
-        for request in self.running:
-            if id(request) not in chosen or request.status is not RequestStatus.RUNNING_DECODE or request.finished or request.cache is None:
-                return None
-            if len(request.output_token_ids) + 1 >= request.sampling_params.max_tokens:
-                return None  # finishes by length on the token in flight: a step of another shape follows
-            after = request.num_computed_tokens + 1
-            if after + 1 > self.config.max_model_len:
-                return None
-            for index, pages in enumerate(self.cache.pages_to_append(request.cache, after, 1)):
-                needed[index] += pages
-        reclaimable = self.cache.num_reclaimable_pages()
-        if any(n > group.allocator.num_free + reclaimable for n, group in zip(needed, self.cache.groups)):
-            return None
-        for request in in_flight:
-            if not self.cache.append(request.cache, request.num_computed_tokens + 1, 1):
-                raise RuntimeError("pages counted as free could not be taken")  # single-threaded: cannot happen
-        return list(in_flight)
-
     def _place_decodes(self, plan: StepPlan, budget: int) -> int:
         """One token for every decoding request, oldest first.  When the token's page cannot be had, the newest running
         request is preempted, as often as it takes; if that comes to be the request itself, it waits."""
