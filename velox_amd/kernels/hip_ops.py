@@ -94,6 +94,7 @@ class HipOps:
         self.pack_decode_weights = True
         self.fuse_residual_norm = True
         self._mm_out_dtype_ok: Optional[bool] = None
+        self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
     # -- loading --------------------------------------------------------------------------------
     def _declare_core(self) -> None:
@@ -222,6 +223,10 @@ class HipOps:
 
     # -- helpers --------------------------------------------------------------------------------
     def _stream(self):
+        # (the raw handle of the current stream: the same value as torch.cuda.current_stream(device).cuda_stream, without
+        # building a Stream object for every kernel call, which costs more host time than the launch itself)
+        if self._raw_stream is not None:
+            return _P(self._raw_stream(self.device.index))
         return _P(torch.cuda.current_stream(self.device).cuda_stream)
 
     def _check(self, name: str, t: torch.Tensor, dtype=None, shape=None, align: int = 4) -> None:
