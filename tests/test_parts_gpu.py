@@ -87,6 +87,55 @@ def test_gated_mlp_part(ops):
     torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embedding_and_head_parts(ops, dtype):
+    """The parts at the two ends alone: the looked-up rows come out as the float32 residual stream, exactly; the head is a
+    product without bias on the rows it is given, in float32; tied, it declares the table's name as its source."""
+    vocab, hidden = 263, 80
+    embedding = make_part("embedding", "table", name="emb.weight", vocab_size=vocab, hidden_size=hidden)
+    table = fill(embedding, 3, dtype)["table"]
+    ids = torch.tensor([5, 262, 0, 5, 77], dtype=torch.int32).cuda()
+    out = embedding.forward(ids, Ctx(ops, dtype))
+    assert out.dtype == torch.float32 and torch.equal(out.cpu(), table.to(dtype).float()[ids.long().cpu()])
+    assert embedding.params()["table"].product is False
+    head = make_part("head", "linear", name="out.weight", vocab_size=vocab, hidden_size=hidden, tied_to=None)
+    w = fill(head, 4, dtype)["weight"]
+    rows = (torch.randn(6, hidden) * 0.5).to(dtype)
+    logits = head.forward(rows.cuda(), Ctx(ops, dtype))
+    assert logits.dtype == torch.float32 and logits.shape == (6, vocab)
+    want = rows.float() @ w.to(dtype).float().T
+    torch.testing.assert_close(logits.cpu(), want, rtol=2e-4, atol=2e-4)
+    tied = make_part("head", "linear", name="out.weight", vocab_size=vocab, hidden_size=hidden, tied_to="emb.weight")
+    assert tied.params()["weight"].alias_of == "emb.weight" and head.params()["weight"].alias_of is None
+
+
+def test_pre_norm_block_alone(ops):
+    """h + mixer(norm1(h)), then + ff(norm2(.)): the block's last output is handed on, not added; with the norm that reads
+    it next the caller gets the same sum.  The mixer here is a stand-in without a cache."""
+    from velox_amd.parts.base import Mixer
+
+    class Twice(Mixer):
+        def forward(self, x, ctx, cache, owns_cache=True):
+            return 2 * x
+
+    hidden, inter = 96, 160
+    norm1 = make_part("norm", "rmsnorm", prefix="n1.", hidden_size=hidden, eps=1e-5)
+    norm2 = make_part("norm", "rmsnorm", prefix="n2.", hidden_size=hidden, eps=1e-5)
+    ff = make_part("feed_forward", "gated_mlp", prefix="m.", hidden_size=hidden, intermediate_size=inter)
+    block = make_part("arrangement", "pre_norm", prefix="b.", mixer=Twice("x."), feed_forward=ff, mixer_norm=norm1, ff_norm=norm2)
+    assert block.input_norm() is norm1 and block.cache_need() is None and block.children() == (norm1, block.mixer, norm2, ff)
+    w1, w2, wf = fill(norm1, 5)["weight"], fill(norm2, 6)["weight"], fill(ff, 7)
+    h = torch.randn(7, hidden)
+    carried = torch.randn(7, hidden) * 0.1  # what the block before handed on
+    residual = h.clone().cuda()
+    pending = block.forward(residual, carried.cuda(), Ctx(ops, torch.float32), None, True)
+    start = h + carried
+    after_mixer = start + 2 * rms_norm(start, w1, 1e-5)
+    torch.testing.assert_close(residual.cpu(), after_mixer, rtol=1e-5, atol=1e-5)  # the mixer's output is in, the feed-forward's is pending
+    want = gated_mlp(rms_norm(after_mixer, w2, 1e-5), wf["gate_up_weight"][:inter], wf["gate_up_weight"][inter:], wf["down_weight"])
+    torch.testing.assert_close(pending.float().cpu(), want, rtol=1e-4, atol=1e-5)
+
+
 @pytest.mark.parametrize("nh,nkv,d,hidden,bias,window", [(4, 2, 16, 64, True, None), (6, 2, 48, 80, False, None), (3, 1, 32, 96, True, 5)])
 def test_attention_part_alone(ops, nh, nkv, d, hidden, bias, window):
     """One attention layer over two sequences cut in two steps each, against plain whole-sequence attention."""

@@ -186,6 +186,51 @@ def test_layers_of_the_real_size_in_four_ways_of_cutting(tmp_path, dtype):
                 torch.testing.assert_close(results[label][rid], results["whole"][rid], **tol)
 
 
+OTHER_REAL_WIDTHS = {
+    # two layers each; the vocabulary is cut down (and made odd), it does not touch the layers' kernels
+    "qwen2.5-1.5b": dict(num_hidden_layers=2, hidden_size=1536, num_attention_heads=12, num_key_value_heads=2, intermediate_size=8960,
+                         vocab_size=32003, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=True),
+    "qwen2.5-32b": dict(num_hidden_layers=2, hidden_size=5120, num_attention_heads=40, num_key_value_heads=8, intermediate_size=27648,
+                        vocab_size=32003, rope_theta=1000000.0, rms_norm_eps=1e-5, tie_word_embeddings=False),
+}
+
+
+@pytest.mark.parametrize("shape", sorted(OTHER_REAL_WIDTHS))
+def test_layers_of_the_other_real_sizes(tmp_path, shape):
+    """bfloat16, two layers with the widths of Qwen2.5-1.5B and of Qwen2.5-32B: the products' kernels are picked by width and
+    by the number of rows (up to 16, up to 32, up to 64, more), and these are the widths the picking was measured at.  Whole
+    prompts, portions of changing size, single tokens, and 20 requests decoding together through a captured step, against
+    the plain model, to the bound that the 7B widths are held to."""
+    from velox_amd.weights import write_random_model
+
+    config = dict(OTHER_REAL_WIDTHS[shape], architectures=["Qwen2ForCausalLM"], model_type="qwen2", use_sliding_window=False, max_position_embeddings=4096)
+    folder = write_random_model(config, str(tmp_path / shape), 9, dtype="bfloat16")
+    config, weights = read_model_folder(folder)
+    requests = rc.request_set(config["vocab_size"], [70, 33, 121] + [18 + (5 * i) % 13 for i in range(20)], seed=81)
+    expected = rc.expected_logits(config, weights, requests)
+    names = list(requests)
+    few = {rid: requests[rid] for rid in names[:3]}
+    crowd = names[3:]
+    together = []  # the crowd: prompts eight at a time without their last five tokens, then five steps of 20 single tokens
+    for lo in range(0, len(crowd), 8):
+        together.append({"step": len(together), "end": [], "entries": [{"id": rid, "tokens": requests[rid][:-5], "want": list(range(len(requests[rid]) - 5))} for rid in crowd[lo:lo + 8]]})
+    for i in range(5):
+        together.append({"step": len(together), "end": crowd if i == 4 else [],
+                         "entries": [{"id": rid, "tokens": [requests[rid][len(requests[rid]) - 5 + i]], "want": [0]} for rid in crowd]})
+    traces = {"tail": rc.tail_one_by_one(few), "portions": rc.changing_portions(few, sizes=(40, 2, 17, 33, 1, 64)), "mixed": rc.mixed(few, seed=3),
+              "together": together}
+    replayer = Replayer(folder, "bfloat16", max(rc.tokens_needed(t, 16) for t in traces.values()), block_size=16, max_live=32, enable_graphs=True)
+    for label, trace in traces.items():
+        subset = {rid: requests[rid] for rid in (crowd if label == "together" else few)}
+        got = rc.collect(trace, rc.run_trace(replayer, trace), subset)
+        for rid in subset:
+            spread = float(expected[rid].std())
+            error = got[rid] - expected[rid]
+            assert float(error.pow(2).mean().sqrt()) < 0.0175 * spread, (shape, label, rid, float(error.pow(2).mean().sqrt()), spread)
+            assert float(error.abs().max()) < 8 * 0.0175 * spread, (shape, label, rid, float(error.abs().max()), spread)
+    assert replayer.runner.num_graph_replays >= 5
+
+
 @pytest.mark.parametrize("live", [40, 12])
 def test_captured_decode_steps_of_many_requests_at_the_real_size(tmp_path, live):
     """40 and 12 requests decode together through the captured steps of 64 and 16 rows, at the widths of Qwen2.5-7B:
