@@ -273,7 +273,9 @@ class Engine:
         if self.config.decode_lookahead and not any(r.sampling_params.has_penalties for r in self.scheduler.running):
             # (penalties read a request's history on the host: they need the token's value)
             self._book(flight)
+            t0 = time.perf_counter()
             ahead = self.scheduler.schedule()
+            self.stats["scheduler_ms"].append((time.perf_counter() - t0) * 1000)
             if not ahead.is_empty():
                 self._ahead = self._launch(ahead, pending=flight)
         self._finish_step(flight)
@@ -317,7 +319,8 @@ class Engine:
 
         t0 = time.perf_counter()
         logits = self.runner.step(entries, device_ids=(pending.tokens, dest_rows, source_rows) if dest_rows else None)
-        self.stats["forward_ms"].append((time.perf_counter() - t0) * 1000)
+        self.stats["prepare_ms"].append(self.runner.last_prepare_ms)
+        self.stats["forward_ms"].append((time.perf_counter() - t0) * 1000 - self.runner.last_prepare_ms)
 
         tokens_gpu = None
         if sampled:

@@ -16,6 +16,7 @@ addresses that the host refreshes before each replay.
 """
 from __future__ import annotations
 
+import time
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
@@ -69,6 +70,7 @@ class ModelRunner:
         self.tuned_row_counts: List[int] = []
         self.max_padding = 0.12  # the most a step is made longer, as a share of its own rows
         self.num_padded_steps = 0
+        self.last_prepare_ms = 0.0  # host time of the last step's batch layout (block tables, positions, ids)
         # every part's scratch at its largest, before anything runs: captured steps hold these addresses
         self.workspace = Workspace(self.device)
         limits = StepLimits(self.max_num_tokens, self.max_num_seqs, cache.max_model_len)
@@ -98,7 +100,9 @@ class ModelRunner:
                     return self._replay(bucket, entries, device_ids)
         if self.tuned_row_counts:
             entries = self._padded_to_tuned_rows(entries)
+        t0 = time.perf_counter()
         ctx = self.builder.build(entries, self.ops, self.dtype, self.workspace, device_ids=device_ids)
+        self.last_prepare_ms = (time.perf_counter() - t0) * 1000
         return self._forward(ctx)
 
     def _padded_to_tuned_rows(self, entries: Sequence[StepEntry]) -> Sequence[StepEntry]:
@@ -130,12 +134,14 @@ class ModelRunner:
         return None
 
     def _padded_entries_context(self, bucket: int, entries: Sequence[StepEntry], device_ids: Optional[tuple] = None) -> StepContext:
+        t0 = time.perf_counter()
         buffer = self._graph_buffers[bucket]
         padded = [StepEntry(e.seq, e.token_ids, e.start, [0]) for e in entries]
         ctx = self.builder.build(
             padded, self.ops, self.dtype, self.workspace,
             device_buffer=buffer, pad_to=bucket, width=self.builder.width, device_ids=device_ids,
         )
+        self.last_prepare_ms = (time.perf_counter() - t0) * 1000
         return ctx
 
     @torch.no_grad()
