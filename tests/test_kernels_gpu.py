@@ -687,6 +687,40 @@ def test_sampling_keeps_exactly_the_tokens_the_filters_allow(ops, vocab, spread)
     assert (again == got[order.numpy()]).all()
 
 
+@pytest.mark.parametrize("vocab,spread", [(152064, 1.2), (151936 + 3, 4.0), (321, 2.0), (4099, 0.3)])
+def test_sampling_with_rows_cut_into_chunks_gives_the_same_tokens(ops, vocab, spread):
+    """Few rows are sampled with several workgroups per row, one kernel per pass, the tables of the threshold's digits
+    added up in global memory: the tokens are those of the one-workgroup kernel, bit for bit, for every number of chunks
+    (chunks that end inside the last quad, chunks beyond the row's end, rows that start off a 16-byte boundary), for
+    greedy rows, rows without a filter and rows with one, side by side."""
+    settings = [(0.8, 0.9, 0), (1.0, 1.0, 7), (0.0, 1.0, 0), (0.7, 0.5, 50), (1.3, 0.95, 1000), (1.0, 0.999, 0), (0.5, 0.3, 3), (1.0, 1.0, 0), (2.0, 0.6, 20000)]
+    base = rand((len(settings), vocab), torch.float32, 78, spread)
+    base[3, 5] = base[3, 11] = base[3, vocab - 1] = float(base[3].max()) + 0.5
+    base[6, :40] = float(base[6].max())
+    base[2, 17] = base[2, vocab - 2] = float(base[2].max()) + 1.0  # a tie in the greedy row, in different chunks: the first wins
+    draws = 5
+    logits = base.repeat_interleave(draws, 0).contiguous()
+    options = np.zeros((len(settings) * draws, 6), dtype=np.int32)
+    f = options.view(np.float32)
+    for r, (temp, top_p, top_k) in enumerate(settings):
+        rows = slice(r * draws, (r + 1) * draws)
+        f[rows, 0], f[rows, 1] = temp, top_p
+        options[rows, 2] = top_k if 0 < top_k < vocab else 0
+        options[rows, 3], options[rows, 4] = 999 + r, 3
+        options[rows, 5] = np.arange(draws)
+    device_options = torch.from_numpy(options).cuda()
+    whole = ops.sample(logits, device_options, chunks=1).cpu().numpy()
+    assert whole[2 * draws] == 17
+    for chunks in (None, 2, 3, 7, 16, 64):
+        got = ops.sample(logits, device_options, chunks=chunks).cpu().numpy()
+        assert (got == whole).all(), (chunks, np.flatnonzero(got != whole)[:10], got[got != whole][:10], whole[got != whole][:10])
+    # no row with a filter: the kernels of the digits are left out
+    plain = [r for r, (temp, top_p, top_k) in enumerate(settings) if temp == 0.0 or (top_p >= 1.0 and top_k == 0)]
+    pick = torch.tensor([r * draws + j for r in plain for j in range(draws)])
+    got = ops.sample(logits[pick.cuda()].contiguous(), device_options[pick.cuda()].contiguous(), with_filter=False, chunks=5).cpu().numpy()
+    assert (got == whole[pick.numpy()]).all()
+
+
 def test_penalties_over_long_histories_and_a_large_vocabulary(ops, ref):
     vocab, rows, width = 152064, 4, 6000
     logits = rand((rows, vocab), torch.float32, 34, 2.0)

@@ -169,7 +169,7 @@ class TorchOps:
     def argmax(self, logits):
         return logits.argmax(dim=-1).to(torch.int32)
 
-    def sample(self, logits, options):
+    def sample(self, logits, options, with_filter=True, chunks=None):
         return torch.tensor(
             [self.sample_row(logits[r].cpu().numpy(), options[r].cpu().numpy())[0] for r in range(logits.shape[0])],
             dtype=torch.int32, device=logits.device,

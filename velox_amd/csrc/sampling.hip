@@ -197,35 +197,35 @@ __device__ __forceinline__ unsigned long long fixed_point_mass(float p) { return
 
 struct Above { unsigned int count; unsigned long long mass; };
 
-// Visits every element of a row: f(index, value).  Whole quads of four consecutive elements come as 16-byte loads when
-// the row starts at a 16-byte boundary, four loads in flight per thread (one workgroup reads the whole row: with one
+// Visits the elements of quads [q_lo, q_hi) of a row (quad q = elements 4q .. 4q + 3, those below vocab): f(index, value).
+// Whole quads come as 16-byte loads when the row starts at a 16-byte boundary, four loads in flight per thread (with one
 // load at a time a pass would take as many trips to the caches as a thread has quads).
-template <typename F> __device__ __forceinline__ void for_each_in_row(const float* __restrict__ row, int vocab, F f) {
-  if ((reinterpret_cast<uintptr_t>(row) & 15) == 0) {
-    const int quads = vocab / 4;
-    const float4_t* body = reinterpret_cast<const float4_t*>(row);
-    const int stride = blockDim.x;
-    int q = threadIdx.x;
-    for (; q + 3 * stride < quads; q += 4 * stride) {
-      const float4_t v0 = body[q], v1 = body[q + stride], v2 = body[q + 2 * stride], v3 = body[q + 3 * stride];
+template <typename F> __device__ __forceinline__ void for_each_in_quads(const float* __restrict__ row, int vocab, int q_lo, int q_hi, F f) {
+  const bool aligned = (reinterpret_cast<uintptr_t>(row) & 15) == 0;
+  int whole = aligned ? vocab / 4 : q_lo;  // quads below `whole` are complete and can be loaded as one
+  whole = whole < q_hi ? whole : q_hi;
+  whole = whole > q_lo ? whole : q_lo;
+  const float4_t* body = reinterpret_cast<const float4_t*>(row);
+  const int stride = blockDim.x;
+  int q = q_lo + threadIdx.x;
+  for (; q + 3 * stride < whole; q += 4 * stride) {
+    const float4_t v0 = body[q], v1 = body[q + stride], v2 = body[q + 2 * stride], v3 = body[q + 3 * stride];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) f(4 * q + e, v0[e]);
+    for (int e = 0; e < 4; ++e) f(4 * q + e, v0[e]);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) f(4 * (q + stride) + e, v1[e]);
+    for (int e = 0; e < 4; ++e) f(4 * (q + stride) + e, v1[e]);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) f(4 * (q + 2 * stride) + e, v2[e]);
+    for (int e = 0; e < 4; ++e) f(4 * (q + 2 * stride) + e, v2[e]);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) f(4 * (q + 3 * stride) + e, v3[e]);
-    }
-    for (; q < quads; q += stride) {
-      const float4_t v = body[q];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) f(4 * q + e, v[e]);
-    }
-    for (int i = 4 * quads + threadIdx.x; i < vocab; i += blockDim.x) f(i, row[i]);
-  } else {
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) f(i, row[i]);
+    for (int e = 0; e < 4; ++e) f(4 * (q + 3 * stride) + e, v3[e]);
   }
+  for (; q < whole; q += stride) {
+    const float4_t v = body[q];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) f(4 * q + e, v[e]);
+  }
+  const int end = 4 * q_hi < vocab ? 4 * q_hi : vocab;
+  for (int i = 4 * whole + threadIdx.x; i < end; i += stride) f(i, row[i]);
 }
 
 // One digit of the search.  `counts` and `masses` hold the table of this digit (SELECT_BINS entries, filled by the whole
@@ -288,83 +288,70 @@ __device__ __forceinline__ int select_digit(const unsigned int* counts, const un
 //   otherwise x = logit / max(T, 1e-5); p = softmax(x); token i is kept iff fewer than top_k tokens have a larger x
 //   (top_k > 0) and the tokens with a larger x hold less than top_p of the probability; among the kept tokens the
 //   draw is argmax(x - max - log(e)), e = max(-log(u), 1e-10), u uniform from Philox(key = seed, counter = (i / 4, counter)).
-// One workgroup per row.  Passes over the row (from the caches: a row is a few hundred kilobytes): the maximum; with a
-// filter, the sum and three digits of the threshold; the draw.
-__global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(const float* __restrict__ logits, const int* __restrict__ options,
-                                                                int* __restrict__ out, int vocab) {
-  __shared__ Best best_scratch[16];
-  __shared__ float scratch[16];
-  __shared__ unsigned int counts[SELECT_BINS];
-  __shared__ unsigned long long masses[SELECT_BINS];
-  __shared__ unsigned long long total_mass;
-  __shared__ int found_digit;
-  __shared__ Above found_above;
-  const float* row = logits + (size_t)blockIdx.x * vocab;
-  const int* opt = options + (size_t)blockIdx.x * 6;
-  const float temperature = __int_as_float(opt[0]);
-  const float top_p = __int_as_float(opt[1]);
-  const int top_k = opt[2];
-  const uint32_t seed_lo = (uint32_t)opt[3], seed_hi = (uint32_t)opt[4], counter = (uint32_t)opt[5];
-  const int tid = threadIdx.x;
+// Passes over the row (from the caches: a row is a few hundred kilobytes): the maximum; with a filter, the sum and three
+// digits of the threshold; the draw.  Either one workgroup walks the whole row (sample_kernel), or, when the rows are
+// too few to fill the GPU that way, the row is cut into chunks of quads with a workgroup each and every pass is a
+// kernel (the sample_chunk_* kernels): the same functions over a range of quads, the tables added up in global memory
+// as integers, so both ways give the same token.
+struct RowOptions {
+  float temperature, top_p, inv_t;
+  int top_k;
+  uint32_t seed_lo, seed_hi, counter;
+  bool use_mass, filter;
+};
 
-  if (temperature == 0.f) {
-    Best best{-INFINITY, 0x7fffffff};
-    for_each_in_row(row, vocab, [&](int i, float v) { best = better(best, Best{v, i}); });
-    best = block_best(best, best_scratch);
-    if (tid == 0) out[blockIdx.x] = best.index;
-    return;
-  }
-  const float inv_t = 1.f / fmaxf(temperature, 1e-5f);
-  float mx = -INFINITY;
-  for_each_in_row(row, vocab, [&](int, float v) { mx = fmaxf(mx, v * inv_t); });
-  mx = block_max(mx, scratch);
+__device__ __forceinline__ RowOptions read_options(const int* __restrict__ opt, int vocab) {
+  RowOptions o;
+  o.temperature = __int_as_float(opt[0]);
+  o.top_p = __int_as_float(opt[1]);
+  o.top_k = opt[2];
+  o.seed_lo = (uint32_t)opt[3];
+  o.seed_hi = (uint32_t)opt[4];
+  o.counter = (uint32_t)opt[5];
+  o.inv_t = 1.f / fmaxf(o.temperature, 1e-5f);
+  o.use_mass = o.top_p < 1.f;
+  o.filter = (o.top_k > 0 && o.top_k < vocab) || o.use_mass;
+  return o;
+}
 
-  // smallest key whose tokens are kept
-  uint32_t threshold = 0u;
-  const bool use_mass = top_p < 1.f;
-  const bool filter = (top_k > 0 && top_k < vocab) || use_mass;
-  if (filter) {
-    Above above{0u, 0ull};
-    unsigned long long mass_limit = 0ull;
-    // digits: bits 31..21, 20..10, 9..0
-    uint32_t prefix = 0u;  // the digits found so far, in place
-#pragma unroll 1
-    for (int level = 0; level < 3; ++level) {
-      const int shift = level == 0 ? 21 : level == 1 ? 10 : 0;
-      const int width = level == 2 ? 10 : 11;
-      const int bins = 1 << width;
-      for (int b = tid; b < bins; b += blockDim.x) { counts[b] = 0u; masses[b] = 0ull; }
-      if (tid == 0 && level == 0) total_mass = 0ull;
-      __syncthreads();
-      const uint32_t known = level == 0 ? 0u : ~((1u << (shift + width)) - 1u);  // mask of the digits found so far
-      unsigned long long my_total = 0ull;
-      for_each_in_row(row, vocab, [&](int, float v) {
-        const float x = v * inv_t;
-        const uint32_t key = sort_key(x);
-        const bool match = (key & known) == prefix;
-        if (level == 0 || match) {
-          const unsigned long long mass = use_mass ? fixed_point_mass(expf(x - mx)) : 0ull;
-          if (level == 0) my_total += mass;
-          if (match) {
-            const int digit = (int)((key >> shift) & (uint32_t)(bins - 1));
-            atomicAdd(&counts[digit], 1u);
-            if (use_mass && mass != 0ull) atomicAdd(&masses[digit], mass);
-          }
-        }
-      });
-      if (level == 0 && use_mass) atomicAdd(&total_mass, my_total);
-      __syncthreads();
-      if (level == 0) mass_limit = (unsigned long long)((double)top_p * (double)total_mass);
-      const int digit = select_digit(counts, masses, bins, top_k, use_mass, mass_limit, above, &found_digit, &found_above);
-      prefix |= (uint32_t)digit << shift;
-      __syncthreads();  // the tables are free again
+// digits of the threshold: bits 31..21, 20..10, 9..0
+__device__ __forceinline__ int level_shift(int level) { return level == 0 ? 21 : level == 1 ? 10 : 0; }
+__device__ __forceinline__ int level_bins(int level) { return level == 2 ? 1024 : 2048; }
+
+// Adds the tokens of quads [q_lo, q_hi) that match the digits found so far (`prefix`) to the tables of digit `level`
+// (`counts`, `masses`: LDS, cleared by the caller, barrier behind the clearing).  At level 0 every token's mass also goes
+// into the returned sum.
+__device__ __forceinline__ unsigned long long add_to_tables(const float* __restrict__ row, int vocab, int q_lo, int q_hi, const RowOptions& o, float mx,
+                                                            int level, uint32_t prefix, unsigned int* counts, unsigned long long* masses) {
+  const int shift = level_shift(level);
+  const int bins = level_bins(level);
+  const uint32_t known = level == 0 ? 0u : ~((1u << (shift + (level == 2 ? 10 : 11))) - 1u);  // mask of the digits found so far
+  unsigned long long my_total = 0ull;
+  const bool use_mass = o.use_mass;
+  const float inv_t = o.inv_t;
+  for_each_in_quads(row, vocab, q_lo, q_hi, [&](int, float v) {
+    const float x = v * inv_t;
+    const uint32_t key = sort_key(x);
+    const bool match = (key & known) == prefix;
+    if (level == 0 || match) {
+      const unsigned long long mass = use_mass ? fixed_point_mass(expf(x - mx)) : 0ull;
+      if (level == 0) my_total += mass;
+      if (match) {
+        const int digit = (int)((key >> shift) & (uint32_t)(bins - 1));
+        atomicAdd(&counts[digit], 1u);
+        if (use_mass && mass != 0ull) atomicAdd(&masses[digit], mass);
+      }
     }
-    threshold = prefix;
-  }
+  });
+  return my_total;
+}
 
+// The draw among the kept tokens of quads [q_lo, q_hi): this thread's best (score, index).
+__device__ __forceinline__ Best draw_in_quads(const float* __restrict__ row, int vocab, int q_lo, int q_hi, const RowOptions& o, float mx, uint32_t threshold) {
   Best best{-INFINITY, 0x7fffffff};
-  const int quads = (vocab + 3) / 4;
   const bool aligned = (reinterpret_cast<uintptr_t>(row) & 15) == 0;
+  const bool filter = o.filter;
+  const float inv_t = o.inv_t;
   auto load_quad = [&](int q, float (&v)[4]) {
     if (aligned && 4 * q + 3 < vocab) {
       const float4_t loaded = *reinterpret_cast<const float4_t*>(row + 4 * q);
@@ -376,37 +363,90 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(const float* __r
     }
   };
   constexpr int AHEAD = 4;  // quads in flight per thread
-  for (int q0 = tid; q0 < quads; q0 += AHEAD * blockDim.x) {
+  for (int q0 = q_lo + threadIdx.x; q0 < q_hi; q0 += AHEAD * blockDim.x) {
     float ahead[AHEAD][4];
 #pragma unroll
     for (int a = 0; a < AHEAD; ++a) {
       const int qa = q0 + a * blockDim.x;
-      load_quad(qa < quads ? qa : q0, ahead[a]);
+      load_quad(qa < q_hi ? qa : q0, ahead[a]);
     }
 #pragma unroll
     for (int a = 0; a < AHEAD; ++a) {
-    const int q = q0 + a * blockDim.x;
-    if (q >= quads) break;
-    float (&v)[4] = ahead[a];
-    bool any = false;
+      const int q = q0 + a * blockDim.x;
+      if (q >= q_hi) break;
+      float (&v)[4] = ahead[a];
+      bool any = false;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) any = any || (4 * q + e < vocab && !(filter && sort_key(v[e] * inv_t) < threshold));
-    if (!any) continue;  // (the noise of a quad is only worked out where a token of it is kept)
-    uint32_t bits[4];
-    philox4x32((uint32_t)q, counter, 0u, 0u, seed_lo, seed_hi, bits);
+      for (int e = 0; e < 4; ++e) any = any || (4 * q + e < vocab && !(filter && sort_key(v[e] * inv_t) < threshold));
+      if (!any) continue;  // (the noise of a quad is only worked out where a token of it is kept)
+      uint32_t bits[4];
+      philox4x32((uint32_t)q, o.counter, 0u, 0u, o.seed_lo, o.seed_hi, bits);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int i = 4 * q + e;
-      if (i >= vocab) break;
-      const float x = v[e] * inv_t;
-      if (filter && sort_key(x) < threshold) continue;
-      const float u = ((float)(bits[e] >> 8) + 0.5f) * (1.0f / 16777216.0f);
-      const float noise = fmaxf(-logf(u), 1e-10f);
-      const float score = (x - mx) - logf(noise);
-      if (score > best.value || best.index == 0x7fffffff) best = Best{score, i};
-    }
+      for (int e = 0; e < 4; ++e) {
+        const int i = 4 * q + e;
+        if (i >= vocab) break;
+        const float x = v[e] * inv_t;
+        if (filter && sort_key(x) < threshold) continue;
+        const float u = ((float)(bits[e] >> 8) + 0.5f) * (1.0f / 16777216.0f);
+        const float noise = fmaxf(-logf(u), 1e-10f);
+        const float score = (x - mx) - logf(noise);
+        if (score > best.value || best.index == 0x7fffffff) best = Best{score, i};
+      }
     }
   }
+  return best;
+}
+
+// One workgroup per row.
+__global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(const float* __restrict__ logits, const int* __restrict__ options,
+                                                                int* __restrict__ out, int vocab) {
+  __shared__ Best best_scratch[16];
+  __shared__ float scratch[16];
+  __shared__ unsigned int counts[SELECT_BINS];
+  __shared__ unsigned long long masses[SELECT_BINS];
+  __shared__ unsigned long long total_mass;
+  __shared__ int found_digit;
+  __shared__ Above found_above;
+  const float* row = logits + (size_t)blockIdx.x * vocab;
+  const RowOptions o = read_options(options + (size_t)blockIdx.x * 6, vocab);
+  const int tid = threadIdx.x;
+  const int quads = (vocab + 3) / 4;
+
+  if (o.temperature == 0.f) {
+    Best best{-INFINITY, 0x7fffffff};
+    for_each_in_quads(row, vocab, 0, quads, [&](int i, float v) { best = better(best, Best{v, i}); });
+    best = block_best(best, best_scratch);
+    if (tid == 0) out[blockIdx.x] = best.index;
+    return;
+  }
+  float mx = -INFINITY;
+  for_each_in_quads(row, vocab, 0, quads, [&](int, float v) { mx = fmaxf(mx, v * o.inv_t); });
+  mx = block_max(mx, scratch);
+
+  // smallest key whose tokens are kept
+  uint32_t threshold = 0u;
+  if (o.filter) {
+    Above above{0u, 0ull};
+    unsigned long long mass_limit = 0ull;
+    uint32_t prefix = 0u;  // the digits found so far, in place
+#pragma unroll 1
+    for (int level = 0; level < 3; ++level) {
+      const int bins = level_bins(level);
+      for (int b = tid; b < bins; b += blockDim.x) { counts[b] = 0u; masses[b] = 0ull; }
+      if (tid == 0 && level == 0) total_mass = 0ull;
+      __syncthreads();
+      const unsigned long long my_total = add_to_tables(row, vocab, 0, quads, o, mx, level, prefix, counts, masses);
+      if (level == 0 && o.use_mass) atomicAdd(&total_mass, my_total);
+      __syncthreads();
+      if (level == 0) mass_limit = (unsigned long long)((double)o.top_p * (double)total_mass);
+      const int digit = select_digit(counts, masses, bins, o.top_k, o.use_mass, mass_limit, above, &found_digit, &found_above);
+      prefix |= (uint32_t)digit << level_shift(level);
+      __syncthreads();  // the tables are free again
+    }
+    threshold = prefix;
+  }
+
+  Best best = draw_in_quads(row, vocab, 0, quads, o, mx, threshold);
   best = block_best(best, best_scratch);
   if (tid == 0) out[blockIdx.x] = best.index;
 }
@@ -414,6 +454,193 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(const float* __r
 extern "C" int velox_sample(const float* logits, const int* options, int* out, int rows, int vocab, hipStream_t stream) {
   if (rows <= 0) return 0;
   sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, options, out, vocab);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---- a row cut into chunks: one kernel per pass ---------------------------------------------------------------------
+// What the chunks of a row share, in global memory: each chunk's maximum and best pair, the tables of the three digits
+// (cleared by the first kernel, added to with integer atomics by the kernels of the digits) and what the search has
+// found so far.  Every workgroup of a kernel reads what the kernel before left and works out the digit before its own
+// once more for itself (a walk down 2,048 entries); the workgroup of chunk 0 writes it down for the kernels after.
+struct RowSearch {
+  unsigned long long total_mass;
+  unsigned long long above_mass[2];
+  unsigned int above_count[2];
+  unsigned int prefix[2];  // the digits found after level 0 and after level 1, in place
+};
+
+struct ChunkedScratch {
+  float* chunk_max;            // [rows, chunks]
+  Best* chunk_best;            // [rows, chunks]
+  RowSearch* search;           // [rows]
+  unsigned int* counts;        // [rows, 3, SELECT_BINS]
+  unsigned long long* masses;  // [rows, 3, SELECT_BINS]
+};
+
+static size_t chunked_scratch_layout(int rows, int chunks, void* base, ChunkedScratch* scratch) {
+  auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  size_t at = 0;
+  char* p = (char*)base;
+  auto take = [&](size_t bytes) { char* here = p + at; at += up(bytes); return here; };
+  ChunkedScratch s;
+  s.masses = (unsigned long long*)take((size_t)rows * 3 * SELECT_BINS * sizeof(unsigned long long));
+  s.counts = (unsigned int*)take((size_t)rows * 3 * SELECT_BINS * sizeof(unsigned int));
+  s.search = (RowSearch*)take((size_t)rows * sizeof(RowSearch));
+  s.chunk_best = (Best*)take((size_t)rows * chunks * sizeof(Best));
+  s.chunk_max = (float*)take((size_t)rows * chunks * sizeof(float));
+  if (scratch != nullptr) *scratch = s;
+  return at;
+}
+
+__device__ __forceinline__ void chunk_quads(int vocab, int& q_lo, int& q_hi) {
+  const int quads = (vocab + 3) / 4;
+  const int per_chunk = (quads + gridDim.y - 1) / gridDim.y;
+  q_lo = blockIdx.y * per_chunk;
+  q_hi = q_lo + per_chunk < quads ? q_lo + per_chunk : quads;
+  if (q_lo > quads) q_lo = quads;
+}
+
+// pass 1: clears the row's tables, leaves the chunk's maximum (or, for a greedy row, its best pair)
+__global__ void __launch_bounds__(SAMPLE_THREADS) sample_chunk_max_kernel(const float* __restrict__ logits, const int* __restrict__ options,
+                                                                          ChunkedScratch s, int vocab) {
+  __shared__ Best best_scratch[16];
+  __shared__ float scratch[16];
+  const int r = blockIdx.x, c = blockIdx.y, chunks = gridDim.y;
+  const float* row = logits + (size_t)r * vocab;
+  const RowOptions o = read_options(options + (size_t)r * 6, vocab);
+  int q_lo, q_hi;
+  chunk_quads(vocab, q_lo, q_hi);
+  if (o.temperature == 0.f) {
+    Best best{-INFINITY, 0x7fffffff};
+    for_each_in_quads(row, vocab, q_lo, q_hi, [&](int i, float v) { best = better(best, Best{v, i}); });
+    best = block_best(best, best_scratch);
+    if (threadIdx.x == 0) s.chunk_best[r * chunks + c] = best;
+    return;
+  }
+  if (o.filter) {
+    const int entries = 3 * SELECT_BINS;
+    for (int e = c * blockDim.x + threadIdx.x; e < entries; e += chunks * blockDim.x) {
+      s.counts[(size_t)r * entries + e] = 0u;
+      s.masses[(size_t)r * entries + e] = 0ull;
+    }
+    if (c == 0 && threadIdx.x == 0) s.search[r].total_mass = 0ull;
+  }
+  float mx = -INFINITY;
+  for_each_in_quads(row, vocab, q_lo, q_hi, [&](int, float v) { mx = fmaxf(mx, v * o.inv_t); });
+  mx = block_max(mx, scratch);
+  if (threadIdx.x == 0) s.chunk_max[r * chunks + c] = mx;
+}
+
+__device__ __forceinline__ float row_max_of_chunks(const float* __restrict__ chunk_max, int chunks) {
+  float mx = -INFINITY;
+  for (int c = 0; c < chunks; ++c) mx = fmaxf(mx, chunk_max[c]);
+  return mx;
+}
+
+// The digit of `level` from the row's finished tables (global), given what was found before; `counts`, `masses`: LDS.
+__device__ __forceinline__ uint32_t finished_digit(const ChunkedScratch& s, int r, int level, const RowOptions& o, uint32_t prefix_before, Above& above,
+                                                   unsigned int* counts, unsigned long long* masses, int* found_digit, Above* found_above) {
+  const int bins = level_bins(level);
+  const size_t base = ((size_t)r * 3 + level) * SELECT_BINS;
+  for (int b = threadIdx.x; b < bins; b += blockDim.x) { counts[b] = s.counts[base + b]; masses[b] = s.masses[base + b]; }
+  __syncthreads();
+  const unsigned long long mass_limit = (unsigned long long)((double)o.top_p * (double)s.search[r].total_mass);
+  const int digit = select_digit(counts, masses, bins, o.top_k, o.use_mass, mass_limit, above, found_digit, found_above);
+  __syncthreads();  // the tables are free again
+  return prefix_before | ((uint32_t)digit << level_shift(level));
+}
+
+// passes 2..4: the tables of digit LEVEL
+template <int LEVEL>
+__global__ void __launch_bounds__(SAMPLE_THREADS) sample_chunk_tables_kernel(const float* __restrict__ logits, const int* __restrict__ options,
+                                                                             ChunkedScratch s, int vocab) {
+  __shared__ unsigned int counts[SELECT_BINS];
+  __shared__ unsigned long long masses[SELECT_BINS];
+  __shared__ unsigned long long total_mass;
+  __shared__ int found_digit;
+  __shared__ Above found_above;
+  const int r = blockIdx.x, c = blockIdx.y, chunks = gridDim.y;
+  const float* row = logits + (size_t)r * vocab;
+  const RowOptions o = read_options(options + (size_t)r * 6, vocab);
+  if (o.temperature == 0.f || !o.filter) return;
+  const int tid = threadIdx.x;
+  int q_lo, q_hi;
+  chunk_quads(vocab, q_lo, q_hi);
+  const float mx = row_max_of_chunks(s.chunk_max + r * chunks, chunks);
+  uint32_t prefix = 0u;
+  if (LEVEL >= 1) {
+    Above above{0u, 0ull};
+    if (LEVEL == 2) { prefix = s.search[r].prefix[0]; above.count = s.search[r].above_count[0]; above.mass = s.search[r].above_mass[0]; }
+    prefix = finished_digit(s, r, LEVEL - 1, o, prefix, above, counts, masses, &found_digit, &found_above);
+    if (c == 0 && tid == 0) {
+      s.search[r].prefix[LEVEL - 1] = prefix;
+      s.search[r].above_count[LEVEL - 1] = above.count;
+      s.search[r].above_mass[LEVEL - 1] = above.mass;
+    }
+  }
+  const int bins = level_bins(LEVEL);
+  for (int b = tid; b < bins; b += blockDim.x) { counts[b] = 0u; masses[b] = 0ull; }
+  if (tid == 0) total_mass = 0ull;
+  __syncthreads();
+  const unsigned long long my_total = add_to_tables(row, vocab, q_lo, q_hi, o, mx, LEVEL, prefix, counts, masses);
+  if (LEVEL == 0 && o.use_mass && my_total != 0ull) atomicAdd(&total_mass, my_total);
+  __syncthreads();
+  const size_t base = ((size_t)r * 3 + LEVEL) * SELECT_BINS;
+  for (int b = tid; b < bins; b += blockDim.x) {
+    if (counts[b] != 0u) atomicAdd(&s.counts[base + b], counts[b]);
+    if (masses[b] != 0ull) atomicAdd(&s.masses[base + b], masses[b]);
+  }
+  if (LEVEL == 0 && tid == 0 && total_mass != 0ull) atomicAdd(&s.search[r].total_mass, total_mass);
+}
+
+// pass 5: the last digit, then the draw among the chunk's kept tokens
+__global__ void __launch_bounds__(SAMPLE_THREADS) sample_chunk_draw_kernel(const float* __restrict__ logits, const int* __restrict__ options,
+                                                                           ChunkedScratch s, int vocab) {
+  __shared__ Best best_scratch[16];
+  __shared__ unsigned int counts[SELECT_BINS];
+  __shared__ unsigned long long masses[SELECT_BINS];
+  __shared__ int found_digit;
+  __shared__ Above found_above;
+  const int r = blockIdx.x, c = blockIdx.y, chunks = gridDim.y;
+  const float* row = logits + (size_t)r * vocab;
+  const RowOptions o = read_options(options + (size_t)r * 6, vocab);
+  if (o.temperature == 0.f) return;  // (its chunks' best pairs are there since the first pass)
+  int q_lo, q_hi;
+  chunk_quads(vocab, q_lo, q_hi);
+  const float mx = row_max_of_chunks(s.chunk_max + r * chunks, chunks);
+  uint32_t threshold = 0u;
+  if (o.filter) {
+    Above above{s.search[r].above_count[1], s.search[r].above_mass[1]};
+    threshold = finished_digit(s, r, 2, o, s.search[r].prefix[1], above, counts, masses, &found_digit, &found_above);
+  }
+  Best best = draw_in_quads(row, vocab, q_lo, q_hi, o, mx, threshold);
+  best = block_best(best, best_scratch);
+  if (threadIdx.x == 0) s.chunk_best[r * chunks + c] = best;
+}
+
+extern "C" long long velox_sample_chunked_scratch_bytes(int rows, int chunks) {
+  if (rows < 1 || chunks < 1) return 0;
+  return (long long)chunked_scratch_layout(rows, chunks, nullptr, nullptr);
+}
+
+// The same tokens as velox_sample, every row cut into `chunks` chunks.  scratch: velox_sample_chunked_scratch_bytes(rows,
+// chunks) bytes at a 256-byte boundary, contents arbitrary.  with_filter = 0 promises that no row has top-k or top-p (the
+// three kernels of the digits are then left out).
+extern "C" int velox_sample_chunked(const float* logits, const int* options, int* out, int rows, int vocab, int chunks, void* scratch,
+                                    long long scratch_bytes, int with_filter, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (chunks < 2 || chunks > 1024 || rows > 65535 || scratch == nullptr || ((uintptr_t)scratch & 255) != 0) return -1;
+  ChunkedScratch s;
+  if ((long long)chunked_scratch_layout(rows, chunks, scratch, &s) > scratch_bytes) return -1;
+  const dim3 grid(rows, chunks);
+  sample_chunk_max_kernel<<<grid, SAMPLE_THREADS, 0, stream>>>(logits, options, s, vocab);
+  if (with_filter) {
+    sample_chunk_tables_kernel<0><<<grid, SAMPLE_THREADS, 0, stream>>>(logits, options, s, vocab);
+    sample_chunk_tables_kernel<1><<<grid, SAMPLE_THREADS, 0, stream>>>(logits, options, s, vocab);
+    sample_chunk_tables_kernel<2><<<grid, SAMPLE_THREADS, 0, stream>>>(logits, options, s, vocab);
+  }
+  sample_chunk_draw_kernel<<<grid, SAMPLE_THREADS, 0, stream>>>(logits, options, s, vocab);
+  argmax_merge_kernel<<<rows, 64, 0, stream>>>(s.chunk_best, out, chunks);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 

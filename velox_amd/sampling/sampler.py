@@ -115,7 +115,8 @@ class Sampler:
             packed[r, 3] = seed & 0x7FFFFFFF
             packed[r, 4] = (seed >> 31) & 0x7FFFFFFF
             packed[r, 5] = int(n)
-        return self.ops.sample(logits, self._upload.send(packed))
+        with_filter = any((not p.is_greedy) and (0 < p.top_k < vocab or p.top_p < 1.0) for p in sampling_params)
+        return self.ops.sample(logits, self._upload.send(packed), with_filter=with_filter)
 
     def _apply_penalties(self, logits, sampling_params, histories) -> torch.Tensor:
         """A penalised copy of ``logits``.  Histories, their lengths and the coefficients travel as one int32 array."""
