@@ -33,6 +33,41 @@ def test_whole_then_decode_matches_plain(tmp_path, ops, name, dtype):
     torch.testing.assert_close(got, expected, **TOL[dtype])
 
 
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_the_cache_holds_the_first_layers_rotated_keys_and_values(tmp_path, ops, name):
+    """What the pages hold, read back in sequence order (``CacheManager.gather_sequence``): layer 0's keys with bias and
+    rotation and its values with bias, as the plain formulas give them from the embeddings, for a prompt fed in portions
+    that end inside pages, then single tokens, beside another request whose pages lie between this one's."""
+    from plain_qwen2 import apply_rope, rms_norm, rope_tables
+
+    folder = make_folder(tmp_path, name, "float32")
+    config, weights = read_model_folder(folder)
+    tokens = random_tokens(config["vocab_size"], 61, seed=17)
+    other = random_tokens(config["vocab_size"], 30, seed=18)
+    h = Harness(folder, ops, torch.float32, "cuda", PAGE_SIZE[name], num_pages=64)
+    h.feed([("a", tokens[:7], [])])
+    h.feed([("b", other[:11], []), ("a", tokens[7:30], [])])
+    h.feed([("a", tokens[30:55], []), ("b", other[11:], [])])
+    for i in range(55, 61):
+        h.feed([("a", [tokens[i]], [0])])
+
+    nh = int(config["num_attention_heads"])
+    nkv = int(config.get("num_key_value_heads", nh))
+    d = int(config.get("head_dim") or config["hidden_size"] // nh)
+    scaling = config.get("rope_scaling") or {}
+    factor = float(scaling.get("factor", 1.0)) if (scaling.get("type") or scaling.get("rope_type")) == "linear" else 1.0
+    cos, sin = rope_tables(d, float(config.get("rope_theta", 10000.0)), len(tokens), factor)
+    x = rms_norm(weights["model.embed_tokens.weight"][torch.tensor(tokens)], weights["model.layers.0.input_layernorm.weight"],
+                 float(config.get("rms_norm_eps", 1e-6)))
+    p = "model.layers.0.self_attn."
+    keys = apply_rope((x @ weights[p + "k_proj.weight"].T + weights[p + "k_proj.bias"]).view(-1, nkv, d), cos, sin, torch.arange(len(tokens)))
+    values = (x @ weights[p + "v_proj.weight"].T + weights[p + "v_proj.bias"]).view(-1, nkv, d)
+    got_keys, got_values = h.cache.gather_sequence(0, h.live["a"][0], len(tokens))
+    torch.testing.assert_close(got_keys.float().cpu(), keys, rtol=2e-5, atol=2e-6)
+    torch.testing.assert_close(got_values.float().cpu(), values, rtol=2e-5, atol=2e-6)
+    assert len(set(h.live["a"][0].tables[0]) & set(h.live["b"][0].tables[0])) == 0
+
+
 def test_workspace_addresses_never_change_once_the_runner_exists(tmp_path, ops):
     """Captured steps hold the addresses of the attention's partial buffers: they are sized once, for the largest step the
     limits allow, and capture, a warm-up portion, a mixed step and a portion whose keys are split all find them in place."""
