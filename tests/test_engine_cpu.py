@@ -71,3 +71,25 @@ def test_a_fixed_workspace_refuses_to_replace_a_buffer():
         workspace.get("a", 101)
     with pytest.raises(WorkspaceError, match="nothing"):
         workspace.get("c", 1)
+
+
+def test_without_a_gpu_the_engine_refuses_loudly(tmp_path, monkeypatch):
+    """No CPU path stands behind the kernels: asking for the product's operations without a GPU, or on the CPU, is one
+    clear error, also through the Python entry point; so is a box without the compiler and without built libraries."""
+    from velox_amd import Engine, EngineConfig
+    from velox_amd.kernels import KernelError, build, load_ops
+
+    with pytest.raises(KernelError, match="no CPU path"):
+        load_ops("cpu")
+    if not torch.cuda.is_available():
+        with pytest.raises(KernelError, match="no GPU is visible"):
+            load_ops("cuda")
+        folder = make_folder(tmp_path, "A")
+        with pytest.raises(KernelError, match="no GPU is visible"):
+            Engine.from_pretrained(EngineConfig(model=folder, dtype="bfloat16"))
+    monkeypatch.setenv("HIPCC", str(tmp_path / "no_such_compiler"))
+    monkeypatch.setenv("PATH", str(tmp_path))
+    real_isfile = build.os.path.isfile
+    monkeypatch.setattr(build.os.path, "isfile", lambda path: False if str(path).endswith("hipcc") else real_isfile(path))
+    with pytest.raises(build.BuildError, match="hipcc not found"):
+        build.find_hipcc()
