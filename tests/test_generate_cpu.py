@@ -251,3 +251,41 @@ def test_every_kind_of_step_is_launched_early_also_with_preemption_and_late_arri
         assert a.output_token_ids == want and b.output_token_ids == want, (index, a.output_token_ids, b.output_token_ids, want)
         assert a.finish_reason is (FinishReason.STOP if index == 3 else FinishReason.LENGTH) and a.finish_reason is b.finish_reason
         assert -1 not in a.all_token_ids
+
+
+def test_penalties_keep_their_counts_through_early_launches_and_preemption(tmp_path):
+    """Penalties over prompt and output with every step launched before the tokens of the one before are read: the
+    sampler counts a request's tokens on the device from its own output, so the penalised tokens are those of the plain
+    model under the reference's formula, also for requests that are preempted and recomputed in a small pool, beside a
+    request without penalties; at the end the sampler holds nothing of any request."""
+    folder = make_folder(tmp_path, "B")
+    config, weights = read_model_folder(folder)
+    page = PAGE_SIZE["B"]
+    vocab = config["vocab_size"]
+    prompts = [[5, 9, 5, 9, 5, 9, 5, 9, 12, 5, 9], random_tokens(vocab, 19, seed=91), [7] * 13 + random_tokens(vocab, 4, seed=92), random_tokens(vocab, 9, seed=93)]
+    coefficients = [dict(repetition_penalty=1.6, frequency_penalty=0.05, presence_penalty=0.02), dict(repetition_penalty=1.3, presence_penalty=0.03),
+                    dict(frequency_penalty=0.4), {}]
+    steps = 14
+
+    def plain_penalised(prompt, repetition_penalty=1.0, presence_penalty=0.0, frequency_penalty=0.0):
+        tokens = list(prompt)
+        for _ in range(steps):
+            logits = qwen2_logits(config, weights, tokens)[-1:].clone()
+            TorchOps().apply_penalties(logits, torch.tensor([tokens]), torch.tensor([len(tokens)]),
+                                       torch.tensor([[repetition_penalty, presence_penalty, frequency_penalty]]))
+            tokens.append(int(logits[0].argmax()))
+        return tokens[len(prompt):]
+
+    expected = [plain_penalised(p, **c) for p, c in zip(prompts, coefficients)]
+    assert expected[0] != plain_greedy(config, weights, prompts[0], steps)  # the penalties decide
+    needed = max((len(p) + steps + page - 1) // page for p in prompts)
+    for lookahead in (True, False):
+        engine = engine_for(folder, "B", decode_lookahead=lookahead, num_gpu_blocks=2 * needed + 2, max_model_len=needed * page,
+                            max_num_batched_tokens=16, max_prefill_chunk_size=6)
+        requests = [Request(f"{lookahead}-{i}", p, SamplingParams(temperature=0.0, max_tokens=steps, ignore_eos=True, **c))
+                    for i, (p, c) in enumerate(zip(prompts, coefficients))]
+        done = engine.generate(requests)
+        assert engine.scheduler.num_preemptions > 0
+        for index, request in enumerate(done):
+            assert request.output_token_ids == expected[index], (lookahead, index, request.output_token_ids, expected[index])
+        assert engine.sampler._seen.row_of_request == {} and engine.sampler._seeds == {}

@@ -741,6 +741,45 @@ def test_penalties_over_long_histories_and_a_large_vocabulary(ops, ref):
     assert torch.equal(again, got)
 
 
+def test_penalties_from_a_table_of_counts_kept_on_the_device(ops, ref):
+    """The table of counts is built from a request's tokens, grows by the sampler's tokens, and penalises the rows that
+    point into it exactly as the history-walking kernel does with the same tokens; rows that point nowhere keep their logits."""
+    vocab, rows = 152064, 5
+    logits = rand((rows, vocab), torch.float32, 36, 2.0)
+    g = torch.Generator().manual_seed(37)
+    histories = [torch.randint(0, vocab, (n,), generator=g).to(torch.int32) for n in (6000, 1, 3500, 0, 777)]
+    histories[2][:3000] = torch.randint(8000, 8200, (3000,), generator=g).to(torch.int32)
+    histories[0][:500] = 151000
+    counts = torch.zeros((8, vocab), dtype=torch.int32, device="cuda")
+    place = [6, 0, 3, -1, 2]  # row 3 has no penalties; the table's rows are in no particular order
+    for h, at in zip(histories, place):
+        if at >= 0 and h.numel():
+            ops.count_tokens(counts[at], h.cuda())
+    new_tokens = torch.tensor([151000, 17, 8100, 5, vocab - 1], dtype=torch.int32)
+    row_of = torch.tensor(place, dtype=torch.int32).cuda()
+    ops.count_sampled(counts, row_of, new_tokens.cuda())
+    coeffs = torch.tensor([[1.3, 0.5, 0.2], [2.0, 1.0, 0.01], [0.8, 0.0, 0.001], [1.7, 0.3, 0.3], [1.1, 0.2, 0.3]], dtype=torch.float32).cuda()
+    got = logits.clone()
+    ops.apply_penalties_from_counts(got, counts, row_of, coeffs)
+    # the same through the history-walking kernel and through the plain formula
+    width = 6001
+    tokens = torch.zeros((rows, width), dtype=torch.int32)
+    lengths = torch.zeros(rows, dtype=torch.int32)
+    for r, (h, at) in enumerate(zip(histories, place)):
+        if at < 0:
+            continue
+        whole = torch.cat([h, new_tokens[r:r + 1]])
+        tokens[r, : whole.numel()] = whole
+        lengths[r] = whole.numel()
+    walked, want = logits.clone(), logits.clone()
+    ops.apply_penalties(walked, tokens.cuda(), lengths.cuda(), coeffs)
+    ref.apply_penalties(want, tokens.cuda(), lengths.cuda(), coeffs)
+    assert torch.equal(got, walked)
+    torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-6)
+    assert torch.equal(got[3], logits[3]) and int((got != logits).sum()) > 6000
+    assert int(counts[6, 151000]) == 501 + int((histories[0][500:] == 151000).sum()) and int(counts.sum()) == sum(h.numel() for h, at in zip(histories, place) if at >= 0) + 4
+
+
 def test_sampling_follows_the_distribution(ops):
     vocab = 50
     logits = rand((1, vocab), torch.float32, 31, 1.5).repeat(4000, 1).contiguous()

@@ -208,6 +208,26 @@ class TorchOps:
         scores = np.where(keep, x - np.log(noise), -np.inf).astype(np.float32)
         return int(scores.argmax()), scores
 
+    def count_tokens(self, counts_row, tokens):
+        ok = (tokens >= 0) & (tokens < counts_row.numel())
+        counts_row += torch.bincount(tokens[ok].long(), minlength=counts_row.numel()).to(counts_row.dtype)
+
+    def count_sampled(self, counts, row_of, tokens):
+        for r in range(tokens.numel()):
+            if int(row_of[r]) >= 0 and 0 <= int(tokens[r]) < counts.shape[1]:
+                counts[int(row_of[r]), int(tokens[r])] += 1
+
+    def apply_penalties_from_counts(self, logits, counts, row_of, coeffs):
+        for r in range(logits.shape[0]):
+            if int(row_of[r]) < 0:
+                continue
+            repetition, presence, frequency = (float(c) for c in coeffs[r])
+            seen = counts[int(row_of[r])]
+            ids = torch.nonzero(seen).flatten()
+            vals = logits[r, ids] - frequency * seen[ids].float()
+            vals = torch.where(vals > 0, vals / repetition, vals * repetition) - presence
+            logits[r, ids] = vals
+
     def apply_penalties(self, logits, tokens, lengths, coeffs):
         """engine/sampler.py:169-189 of the reference: frequency first (times the count), then repetition
         (positive / r, negative * r) and presence, each once per distinct seen token."""

@@ -699,3 +699,62 @@ extern "C" int velox_apply_penalties(float* logits, const int* tokens, const int
   penalties_kernel<<<rows, 256, 0, stream>>>(logits, tokens, lengths, coeffs, vocab, width);
   VELOX_RETURN_LAUNCH_STATUS();
 }
+
+// ---- penalties from a table of counts that lives on the device -------------------------------------------------------
+// counts: int32 [table rows, vocab], one row per request with penalties: how often the request has seen each token
+// (prompt and output).  The row is built once from the request's tokens and then kept up to date from the sampler's
+// output, on the device: a step's penalties need neither the history nor the value of the token before it on the host.
+__global__ void __launch_bounds__(256) count_tokens_kernel(int* __restrict__ counts_row, const int* __restrict__ tokens, int n, int vocab) {
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+    const int token = tokens[i];
+    if (token >= 0 && token < vocab) atomicAdd(&counts_row[token], 1);
+  }
+}
+
+// row_of[r]: the table row of batch row r, or -1 (no penalties)
+__global__ void __launch_bounds__(64) count_sampled_kernel(int* __restrict__ counts, const int* __restrict__ row_of, const int* __restrict__ tokens, int rows,
+                                                           int vocab) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= rows || row_of[r] < 0) return;
+  const int token = tokens[r];
+  if (token >= 0 && token < vocab) atomicAdd(&counts[(size_t)row_of[r] * vocab + token], 1);  // (one request may not sit in two rows; atomic all the same)
+}
+
+// v = logit - frequency * count;  v = v > 0 ? v / repetition : v * repetition;  v -= presence, where count > 0
+__global__ void __launch_bounds__(256) penalties_from_counts_kernel(float* __restrict__ logits, const int* __restrict__ counts, const int* __restrict__ row_of,
+                                                                    const float* __restrict__ coeffs, int vocab) {
+  const int r = blockIdx.x;
+  const int table_row = row_of[r];
+  if (table_row < 0) return;
+  const float repetition = coeffs[3 * r], presence = coeffs[3 * r + 1], frequency = coeffs[3 * r + 2];
+  float* row = logits + (size_t)r * vocab;
+  const int* seen = counts + (size_t)table_row * vocab;
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < vocab; i += gridDim.y * blockDim.x) {
+    const int count = seen[i];
+    if (count == 0) continue;
+    float v = row[i] - frequency * (float)count;
+    v = v > 0.f ? v / repetition : v * repetition;
+    row[i] = v - presence;
+  }
+}
+
+extern "C" int velox_count_tokens(int* counts_row, const int* tokens, int n, int vocab, hipStream_t stream) {
+  if (n <= 0) return 0;
+  const int blocks = (n + 255) / 256 < 256 ? (n + 255) / 256 : 256;
+  count_tokens_kernel<<<blocks, 256, 0, stream>>>(counts_row, tokens, n, vocab);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int velox_count_sampled(int* counts, const int* row_of, const int* tokens, int rows, int vocab, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  count_sampled_kernel<<<(rows + 63) / 64, 64, 0, stream>>>(counts, row_of, tokens, rows, vocab);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int velox_penalties_from_counts(float* logits, const int* counts, const int* row_of, const float* coeffs, int rows, int vocab, int chunks,
+                                           hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (chunks < 1 || chunks > 65535 || rows > 65535) return -1;
+  penalties_from_counts_kernel<<<dim3(rows, chunks), 256, 0, stream>>>(logits, counts, row_of, coeffs, vocab);
+  VELOX_RETURN_LAUNCH_STATUS();
+}

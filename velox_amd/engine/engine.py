@@ -270,8 +270,7 @@ class Engine:
             if scheduled.is_empty():
                 return
             flight = self._launch(scheduled)
-        if self.config.decode_lookahead and not any(r.sampling_params.has_penalties for r in self.scheduler.running):
-            # (penalties read a request's history on the host: they need the token's value)
+        if self.config.decode_lookahead:
             self._book(flight)
             t0 = time.perf_counter()
             ahead = self.scheduler.schedule()
@@ -325,13 +324,15 @@ class Engine:
         tokens_gpu = None
         if sampled:
             t0 = time.perf_counter()
+            # (penalties: the sampler counts a request's tokens itself once it has seen its history, which it asks for
+            # the first time only; a request is new to it at the end of its prompt, when no token of it is pending)
             needs_history = any(r.sampling_params.has_penalties for r in sampled)
             tokens_gpu = self.sampler.sample(
                 logits,
                 [r.sampling_params for r in sampled],
                 [r.request_id for r in sampled],
                 [len(r.output_token_ids) for r in sampled],
-                histories=[r.all_token_ids for r in sampled] if needs_history else None,
+                histories=[(lambda r=r: r.all_token_ids) for r in sampled] if needs_history else None,
             )
             self.stats["sampling_ms"].append((time.perf_counter() - t0) * 1000)
         # the copy of the tokens to the host is queued right behind the sampler, before a later step can be queued

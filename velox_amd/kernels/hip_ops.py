@@ -120,6 +120,9 @@ class HipOps:
         c.velox_skinny_gemm_splitk_bf16.restype = _I
         c.velox_argmax.argtypes = [_P, _P, _P, _I, _I, _I, _P]
         c.velox_sample.argtypes = [_P, _P, _P, _I, _I, _P]
+        c.velox_count_tokens.argtypes = [_P, _P, _I, _I, _P]
+        c.velox_count_sampled.argtypes = [_P, _P, _P, _I, _I, _P]
+        c.velox_penalties_from_counts.argtypes = [_P, _P, _P, _P, _I, _I, _I, _P]
         c.velox_sample_chunked.argtypes = [_P, _P, _P, _I, _I, _I, _P, ctypes.c_longlong, _I, _P]
         c.velox_sample_chunked_scratch_bytes.argtypes = [_I, _I]
         c.velox_sample_chunked_scratch_bytes.restype = ctypes.c_longlong
@@ -129,7 +132,8 @@ class HipOps:
         c.velox_probe_mfma.argtypes = [_I, _I, _P, _P]
         c.velox_probe_mfma.restype = _I
         for fn in (c.velox_embed, c.velox_add_rmsnorm, c.velox_silu_mul, c.velox_rope_kv_write, c.velox_gemm_fma,
-                   c.velox_argmax, c.velox_sample, c.velox_sample_chunked, c.velox_apply_penalties):
+                   c.velox_argmax, c.velox_sample, c.velox_sample_chunked, c.velox_apply_penalties, c.velox_count_tokens, c.velox_count_sampled,
+                   c.velox_penalties_from_counts):
             fn.restype = _I
 
     def attention_library(self, head_dim: int) -> ctypes.CDLL:
@@ -828,6 +832,38 @@ class HipOps:
         self._check("coeffs", coeffs, torch.float32, (rows, 3))
         status = self._core.velox_apply_penalties(_ptr(logits), _ptr(tokens), _ptr(lengths), _ptr(coeffs), rows, vocab, tokens.shape[1], self._stream())
         self._launched(status, "apply_penalties")
+
+    def count_tokens(self, counts_row: torch.Tensor, tokens: torch.Tensor) -> None:
+        """``counts_row[token] += 1`` for every token of int32 ``tokens`` (ids outside the row are skipped)."""
+        self._check("counts_row", counts_row, torch.int32)
+        self._check("tokens", tokens, torch.int32)
+        if counts_row.dim() != 1 or tokens.dim() != 1:
+            raise KernelError("count_tokens: a row of counts and a list of tokens are expected")
+        self._launched(self._core.velox_count_tokens(_ptr(counts_row), _ptr(tokens), tokens.numel(), counts_row.numel(), self._stream()), "count_tokens")
+
+    def count_sampled(self, counts: torch.Tensor, row_of: torch.Tensor, tokens: torch.Tensor) -> None:
+        """``counts[row_of[r], tokens[r]] += 1`` for every batch row ``r`` with ``row_of[r] >= 0``."""
+        self._check("counts", counts, torch.int32)
+        rows = tokens.numel()
+        self._check("row_of", row_of, torch.int32, (rows,))
+        self._check("tokens", tokens, torch.int32, (rows,))
+        if counts.dim() != 2:
+            raise KernelError("count_sampled: counts must be [table rows, vocab]")
+        self._launched(self._core.velox_count_sampled(_ptr(counts), _ptr(row_of), _ptr(tokens), rows, counts.shape[1], self._stream()), "count_sampled")
+
+    def apply_penalties_from_counts(self, logits: torch.Tensor, counts: torch.Tensor, row_of: torch.Tensor, coeffs: torch.Tensor) -> None:
+        """Penalises float32 ``logits`` [rows, vocab] in place: row ``r`` by the counts of table row ``row_of[r]`` (rows with
+        -1 are left alone) and ``coeffs[r] = (repetition, presence, frequency)``.  The host must keep ``row_of`` inside the table."""
+        self._check("logits", logits, torch.float32)
+        rows, vocab = logits.shape
+        self._check("counts", counts, torch.int32)
+        if counts.dim() != 2 or counts.shape[1] != vocab:
+            raise KernelError(f"apply_penalties_from_counts: counts must be [table rows, {vocab}], got {tuple(counts.shape)}")
+        self._check("row_of", row_of, torch.int32, (rows,))
+        self._check("coeffs", coeffs, torch.float32, (rows, 3))
+        chunks = max(1, min(2 * self.num_cus // rows, (vocab + 2047) // 2048))
+        status = self._core.velox_penalties_from_counts(_ptr(logits), _ptr(counts), _ptr(row_of), _ptr(coeffs), rows, vocab, chunks, self._stream())
+        self._launched(status, "penalties_from_counts")
 
     # -- probes ---------------------------------------------------------------------------------
     def _timed(self, launch, repeats: int) -> float:
