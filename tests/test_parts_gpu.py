@@ -460,7 +460,7 @@ def test_toy_architecture_with_routed_experts_and_learned_positions(ops, dtype):
 # read the same normalised input side by side; all defined and registered here.
 # ----------------------------------------------------------------------------------------------------
 from velox_amd.parts import Block, Embedding, OutputHead, register_arrangement  # noqa: E402
-from velox_amd.parts.base import Param  # noqa: E402
+from velox_amd.parts.base import Norm, Param  # noqa: E402
 
 
 class ScaledEmbedding(Embedding):
@@ -496,6 +496,31 @@ class SoftcapHead(OutputHead):
         return self.cap * torch.tanh(logits / self.cap)
 
 
+class CenteredNorm(Norm):
+    """y = (x - mean) / sqrt(var + eps) * weight + bias: no form that a product's epilogue could take over
+    (``deferred_form`` stays None), so the products before it hand back tensors and this part adds them itself."""
+
+    def __init__(self, prefix, hidden_size, eps):
+        super().__init__(prefix)
+        self.hidden_size, self.eps = hidden_size, eps
+        self.weight = self.bias = None
+
+    def params(self):
+        return {"weight": single("weight", (self.hidden_size,), role="vector", init="one_plus_normal"), "bias": single("bias", (self.hidden_size,), role="vector")}
+
+    def forward(self, residual, delta, ctx, rows=None):
+        if delta is not None:
+            delta = ctx.ops.materialize(delta)
+            delta = (delta.sum(0) if delta.dim() == 3 else delta).float()
+        if rows is None:
+            if delta is not None:
+                residual.add_(delta)
+            x = residual
+        else:
+            x = residual[rows.long()] + (delta[rows.long()] if delta is not None else 0.0)
+        return torch.nn.functional.layer_norm(x, (self.hidden_size,), self.weight, self.bias, self.eps).to(ctx.dtype)
+
+
 class ParallelBlock(Block):
     """h = h + mixer(norm(h)) + ff(norm(h)): one norm, both sub-layers read it."""
 
@@ -522,10 +547,11 @@ def ends_spec(config, max_position=None) -> ModelSpec:
     norm = PartSpec.of("rmsnorm", hidden_size=h, eps=raw["eps"])
     attention = PartSpec.of("attention", hidden_size=h, num_heads=3, num_kv_heads=3, head_dim=32, qkv_bias=False)
     ff = PartSpec.of("gated_mlp", hidden_size=h, intermediate_size=raw["inter"])
+    centered = PartSpec.of("toy_centered", hidden_size=h, eps=raw["eps"])
     layers = [LayerSpec("blocks.0.", attention, ff, norm, norm, position="rope", arrangement="toy_parallel"),
-              LayerSpec("blocks.1.", attention, ff, norm, norm, position="rope")]  # (the framework's own names for the tensors)
+              LayerSpec("blocks.1.", attention, ff, centered, norm, position="rope")]  # (the framework's own names for the tensors)
     return ModelSpec(vocab_size=raw["vocab_size"], hidden_size=h, max_position=128, layers=layers, schedule=[ScheduleEntry(0), ScheduleEntry(1)],
-                     final_norm=norm, positions={"rope": PartSpec.of("rotary", rotary_dim=32, theta=10000.0, max_position=128)},
+                     final_norm=centered, positions={"rope": PartSpec.of("rotary", rotary_dim=32, theta=10000.0, max_position=128)},
                      tie_head=raw["tied"], embedding=PartSpec.of("toy_scaled", scale=raw["embedding_scale"]), head=PartSpec.of("toy_softcap", cap=raw["cap"]))
 
 
@@ -546,10 +572,13 @@ def plain_ends(tensors, raw, tokens):
 
     a = rms_norm(x, tensors["blocks.0.mixer_norm.weight"], eps)
     x = x + attend("blocks.0.", a) + ff("blocks.0.", a)
-    x = x + attend("blocks.1.", rms_norm(x, tensors["blocks.1.mixer_norm.weight"], eps))
+    def centered(x, p):
+        return torch.nn.functional.layer_norm(x, (x.shape[-1],), tensors[p + "weight"], tensors[p + "bias"], eps)
+
+    x = x + attend("blocks.1.", centered(x, "blocks.1.mixer_norm."))
     x = x + ff("blocks.1.", rms_norm(x, tensors["blocks.1.feed_forward_norm.weight"], eps))
     head = table if raw["tied"] else tensors["head.weight"]
-    logits = rms_norm(x, tensors["final_norm.weight"], eps) @ head.T + tensors["head.bias"]
+    logits = centered(x, "final_norm.") @ head.T + tensors["head.bias"]
     return raw["cap"] * torch.tanh(logits / raw["cap"])
 
 
@@ -576,10 +605,12 @@ def test_toy_architecture_with_its_own_embedding_head_and_arrangement(ops, tied)
     register_part("embedding", "toy_scaled", ScaledEmbedding)
     register_part("head", "toy_softcap", SoftcapHead)
     register_arrangement("toy_parallel", ParallelBlock)
+    register_part("norm", "toy_centered", CenteredNorm)
     register_architecture("EndsToyForCausalLM", lambda raw: ModelConfig(architecture_name(raw), dict(raw)), ends_spec)
     raw = {"architectures": ["EndsToyForCausalLM"], "hidden_size": 96, "inter": 160, "vocab_size": 77, "eps": 1e-5, "embedding_scale": 9.5, "cap": 0.3, "tied": tied}
     model = build_model(config_from_dict(raw), torch.float32, "cuda")
     assert type(model.embedding) is ScaledEmbedding and type(model.head) is SoftcapHead and type(model.blocks[0]) is ParallelBlock
+    assert type(model.final_norm) is CenteredNorm and type(model.blocks[1].mixer_norm) is CenteredNorm and "final_norm.bias" in dict(random_tensors(model, 11))
     bind_random(model, 11, torch.float32, "cuda", storage_dtype=torch.float32)
     tensors = dict(random_tensors(model, 11))
     assert ("head.weight" in tensors) == (not tied) and "blocks.0.feed_forward_norm.weight" not in tensors
