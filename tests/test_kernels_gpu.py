@@ -719,6 +719,10 @@ def test_sampling_with_rows_cut_into_chunks_gives_the_same_tokens(ops, vocab, sp
     pick = torch.tensor([r * draws + j for r in plain for j in range(draws)])
     got = ops.sample(logits[pick.cuda()].contiguous(), device_options[pick.cuda()].contiguous(), with_filter=False, chunks=5).cpu().numpy()
     assert (got == whole[pick.numpy()]).all()
+    # a broken promise gives no token rather than one from the wrong set
+    broken = ops.sample(logits, device_options, with_filter=False, chunks=5).cpu().numpy()
+    has_filter = np.array([temp != 0.0 and (top_p < 1.0 or 0 < top_k < vocab) for temp, top_p, top_k in settings]).repeat(draws)
+    assert (broken[has_filter] == -1).all() and (broken[~has_filter] == whole[~has_filter]).all()
 
 
 def test_penalties_over_long_histories_and_a_large_vocabulary(ops, ref):

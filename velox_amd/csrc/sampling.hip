@@ -595,7 +595,7 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_chunk_tables_kernel(con
 
 // pass 5: the last digit, then the draw among the chunk's kept tokens
 __global__ void __launch_bounds__(SAMPLE_THREADS) sample_chunk_draw_kernel(const float* __restrict__ logits, const int* __restrict__ options,
-                                                                           ChunkedScratch s, int vocab) {
+                                                                           ChunkedScratch s, int vocab, int with_filter) {
   __shared__ Best best_scratch[16];
   __shared__ unsigned int counts[SELECT_BINS];
   __shared__ unsigned long long masses[SELECT_BINS];
@@ -609,6 +609,12 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_chunk_draw_kernel(const
   chunk_quads(vocab, q_lo, q_hi);
   const float mx = row_max_of_chunks(s.chunk_max + r * chunks, chunks);
   uint32_t threshold = 0u;
+  if (o.filter && !with_filter) {
+    // the caller promised that no row has a filter, and this one has: the kernels of the digits did not run.  No token
+    // rather than one drawn from the wrong set: the row's result is -1.
+    if (threadIdx.x == 0) s.chunk_best[r * chunks + c] = Best{INFINITY, -1};
+    return;
+  }
   if (o.filter) {
     Above above{s.search[r].above_count[1], s.search[r].above_mass[1]};
     threshold = finished_digit(s, r, 2, o, s.search[r].prefix[1], above, counts, masses, &found_digit, &found_above);
@@ -625,7 +631,7 @@ extern "C" long long velox_sample_chunked_scratch_bytes(int rows, int chunks) {
 
 // The same tokens as velox_sample, every row cut into `chunks` chunks.  scratch: velox_sample_chunked_scratch_bytes(rows,
 // chunks) bytes at a 256-byte boundary, contents arbitrary.  with_filter = 0 promises that no row has top-k or top-p (the
-// three kernels of the digits are then left out).
+// three kernels of the digits are then left out; a row that has one all the same gets the token -1).
 extern "C" int velox_sample_chunked(const float* logits, const int* options, int* out, int rows, int vocab, int chunks, void* scratch,
                                     long long scratch_bytes, int with_filter, hipStream_t stream) {
   if (rows <= 0) return 0;
@@ -639,7 +645,7 @@ extern "C" int velox_sample_chunked(const float* logits, const int* options, int
     sample_chunk_tables_kernel<1><<<grid, SAMPLE_THREADS, 0, stream>>>(logits, options, s, vocab);
     sample_chunk_tables_kernel<2><<<grid, SAMPLE_THREADS, 0, stream>>>(logits, options, s, vocab);
   }
-  sample_chunk_draw_kernel<<<grid, SAMPLE_THREADS, 0, stream>>>(logits, options, s, vocab);
+  sample_chunk_draw_kernel<<<grid, SAMPLE_THREADS, 0, stream>>>(logits, options, s, vocab, with_filter);
   argmax_merge_kernel<<<rows, 64, 0, stream>>>(s.chunk_best, out, chunks);
   VELOX_RETURN_LAUNCH_STATUS();
 }

@@ -798,7 +798,7 @@ class HipOps:
 
     def sample(self, logits: torch.Tensor, options: torch.Tensor, with_filter: bool = True, chunks: Optional[int] = None) -> torch.Tensor:
         """One token per row of float32 ``logits`` by the rows' ``options`` (int32 ``[rows, 6]``: see ``sample_kernel``).
-        ``with_filter=False`` promises that no row has top-k or top-p.  ``chunks``: into how many pieces a row is cut
+        ``with_filter=False`` promises that no row has top-k or top-p (a row that has one all the same comes back as -1 when rows are cut into chunks).  ``chunks``: into how many pieces a row is cut
         (default: one workgroup per row when the rows fill the GPU, else enough pieces to fill it); the tokens do not
         depend on it."""
         self._check("logits", logits, torch.float32)
