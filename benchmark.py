@@ -11,6 +11,7 @@ from __future__ import annotations
 
 import argparse
 import json
+import os
 import random
 import statistics
 import sys
@@ -248,6 +249,7 @@ def main(argv=None) -> int:
     if args.output_json:
         for result in results:
             result.pop("outputs", None)
+        os.makedirs(os.path.dirname(os.path.abspath(args.output_json)), exist_ok=True)
         with open(args.output_json, "w", encoding="utf-8") as handle:
             json.dump(results, handle, indent=2)
         print(f"\nWrote {args.output_json}")
