@@ -329,6 +329,42 @@ def test_sampling_through_the_engine(tmp_path):
     assert penalised[0].output_token_ids != plain_penalised(histories[0], 10)  # the penalties changed what is chosen
 
 
+def test_many_penalised_requests_admitted_in_one_step_with_captured_steps(tmp_path):
+    """Forty short prompts with penalties finish their prompts in a handful of steps: each brings its history to the
+    sampler's table of counts through the ring of pinned buffers (more uploads in one step than the ring has places),
+    the table grows twice, decode steps are captured and launched ahead; every request gets the plain model's penalised
+    tokens, and when all are done the sampler holds nothing."""
+    from torch_ops import TorchOps
+
+    folder = make_folder(tmp_path, "A")
+    config, weights = read_model_folder(folder)
+    vocab = config["vocab_size"]
+    prompts = [[3 + i % 5, 9, 3 + i % 5, 9, 17] + random_tokens(vocab, 1 + i % 4, seed=300 + i) for i in range(40)]
+    steps = 6
+
+    def plain_penalised(prompt, repetition, presence, frequency):
+        tokens = list(prompt)
+        for _ in range(steps):
+            logits = qwen2_logits(config, weights, tokens)[-1:].clone()
+            TorchOps().apply_penalties(logits, torch.tensor([tokens]), torch.tensor([len(tokens)]), torch.tensor([[repetition, presence, frequency]]))
+            tokens.append(int(logits[0].argmax()))
+        return tokens[len(prompt):]
+
+    engine = engine_for(folder, "A", max_num_seqs=40, max_num_batched_tokens=512, max_prefill_chunk_size=64, num_gpu_blocks=400, enable_cuda_graphs=True)
+    coefficients = [(1.0 + 0.1 * (i % 7), 0.02 * (i % 3), 0.05 * (i % 4)) for i in range(40)]
+    requests = [Request(f"many{i}", p, SamplingParams(temperature=0.0, max_tokens=steps, ignore_eos=True, repetition_penalty=c[0], presence_penalty=c[1],
+                                                      frequency_penalty=c[2])) for i, (p, c) in enumerate(zip(prompts, coefficients))]
+    done = engine.generate(requests)
+    assert engine.runner.num_graph_replays > 0
+    differs = 0
+    for request, prompt, c in zip(done, prompts, coefficients):
+        want = plain_penalised(prompt, *c)
+        assert request.output_token_ids == want, (request.request_id, request.output_token_ids, want)
+        differs += want != plain_greedy(config, weights, prompt, steps)
+    assert differs > 10  # the penalties decide for many of them
+    assert engine.sampler._seen.row_of_request == {} and engine.sampler._seen.table.shape[0] >= 40
+
+
 def test_pool_sized_from_free_memory_when_no_page_count_is_given(tmp_path):
     """``num_gpu_blocks=None``: the pool takes what the free memory allows (reference ``src/paged_kv_cache.py:159-194``), capped at
     what ``max_num_seqs`` requests of ``max_model_len`` tokens can ever hold; a utilisation that leaves nothing is an error."""
