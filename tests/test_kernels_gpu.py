@@ -960,3 +960,22 @@ def test_probes_report_rates_in_the_band_of_this_card(ops):
     mfma = ops.probe_mfma_rate(iterations=20000, repeats=3)
     assert 4000.0 < read < 8000.0, read
     assert 1250.0 < mfma <= 2600.0, mfma
+
+
+def test_place_tokens_puts_sampled_ids_into_a_steps_rows(ops, ref):
+    from velox_amd.kernels.hip_ops import KernelError
+
+    ids = torch.arange(100, 140, dtype=torch.int32).cuda()
+    tokens = torch.tensor([7, 8, 9, 10, 11], dtype=torch.int32).cuda()
+    dest = torch.tensor([3, 39, 0, 17, 99, 5], dtype=torch.int32).cuda()   # (the fifth pair points outside ids: skipped)
+    source = torch.tensor([4, 0, 2, 2, 1, 77], dtype=torch.int32).cuda()   # (the sixth outside tokens: skipped)
+    want = ids.clone()
+    ref.place_tokens(want, dest, source, tokens, 4)
+    got = ids.clone()
+    ops.place_tokens(got, dest, source, tokens, 6)
+    assert torch.equal(got, want) and got[3] == 11 and got[39] == 7 and got[0] == 9 and got[17] == 9 and got[5] == 105
+    untouched = ids.clone()
+    ops.place_tokens(untouched, dest, source, tokens, 0)
+    assert torch.equal(untouched, ids)
+    with pytest.raises(KernelError):
+        ops.place_tokens(got, dest, source, tokens, 7)

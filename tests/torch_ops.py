@@ -70,6 +70,9 @@ class TorchOps:
         return qkv
 
     # -- embedding and norms ------------------------------------------------------------
+    def place_tokens(self, ids, dest, source, tokens, count):
+        ids[dest[:count].long()] = tokens[source[:count].long()]
+
     def embed(self, token_ids, table):
         return table[token_ids.long()].float()
 

@@ -28,6 +28,23 @@ extern "C" int velox_embed(const int* ids, const void* table, float* out, int to
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
+// ids[dest[k]] = tokens[source[k]] for k < n: token ids that were sampled by the step before this one and have not been
+// to the host, put where this step's rows expect them.  (Pairs outside either array are skipped: the host has checked.)
+__global__ void __launch_bounds__(64) place_tokens_kernel(int* __restrict__ ids, const int* __restrict__ dest, const int* __restrict__ source,
+                                                          const int* __restrict__ tokens, int n, int num_ids, int num_tokens) {
+  const int k = blockIdx.x * blockDim.x + threadIdx.x;
+  if (k >= n) return;
+  const int to = dest[k], from = source[k];
+  if (to >= 0 && to < num_ids && from >= 0 && from < num_tokens) ids[to] = tokens[from];
+}
+
+extern "C" int velox_place_tokens(int* ids, const int* dest, const int* source, const int* tokens, int n, int num_ids, int num_tokens,
+                                  hipStream_t stream) {
+  if (n <= 0) return 0;
+  place_tokens_kernel<<<(n + 63) / 64, 64, 0, stream>>>(ids, dest, source, tokens, n, num_ids, num_tokens);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
 // ---------------------------------------------------------------------------------------------
 // residual add + RMSNorm.  One block per output row.
 //   rows == nullptr: r = residual[row] (+ delta[row]); residual[row] = r; out[row] = norm(r)

@@ -133,7 +133,7 @@ class BatchBuilder:
 
     def section_total(self, t: int, b: int, r: int, w: int) -> int:
         n_groups = len(self.cache.groups)
-        return _align(t) * 2 + _align(b + 1) + _align(b) * 2 + _align(2 * b) + _align(r) + n_groups * (_align(b) + _align(t) + _align(b * w))
+        return _align(t) * 2 + _align(b + 1) + _align(b) * 3 + _align(r) + n_groups * (_align(b) + _align(t) + _align(b * w))
 
     def build(self, entries: Sequence[StepEntry], ops, dtype, workspace: Workspace, device_buffer: Optional[torch.Tensor] = None, pad_to: Optional[int] = None, width: Optional[int] = None,
               device_ids: Optional[tuple] = None) -> StepContext:
@@ -211,9 +211,9 @@ class BatchBuilder:
         put("slots", slots, b)
         put("rows", np.asarray(rows, dtype=np.int32), r)
         # always laid out: a captured step reads its sections at fixed places.  At most one token per entry is still to
-        # come (its newest); dest is laid out as 64-bit integers, which is what the scatter on the device takes
+        # come (its newest)
         source = np.zeros(b, dtype=np.int32)
-        dest = np.zeros(2 * b, dtype=np.int32)
+        dest = np.zeros(b, dtype=np.int32)
         num_device_ids = 0
         if device_ids is not None:
             tokens_on_device, dest_rows, source_rows = device_ids
@@ -225,9 +225,9 @@ class BatchBuilder:
             if tokens_on_device.dtype != torch.int32 or tokens_on_device.dim() != 1:
                 raise ValueError("token ids on the device must be int32 [R]")
             source[:num_device_ids] = np.asarray(source_rows, dtype=np.int32)
-            dest[0:2 * num_device_ids:2] = np.asarray(dest_rows, dtype=np.int32)
+            dest[:num_device_ids] = np.asarray(dest_rows, dtype=np.int32)
         put("source", source, b)
-        put("dest", dest, 2 * b)
+        put("dest", dest, b)
         max_kv: List[int] = []
         max_kv_portions: List[int] = []
         decode_prefix = next((i for i, n in enumerate(q_lens) if n != 1), len(q_lens))
@@ -264,8 +264,7 @@ class BatchBuilder:
             return device[lo:lo + n]
 
         if num_device_ids:
-            gathered = torch.index_select(device_ids[0], 0, view("source")[:num_device_ids])
-            view("ids").index_copy_(0, view("dest")[:2 * num_device_ids].view(torch.int64), gathered)
+            ops.place_tokens(view("ids"), view("dest"), view("source"), device_ids[0], num_device_ids)
 
         groups = [
             GroupBatch(

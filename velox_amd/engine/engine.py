@@ -156,8 +156,6 @@ class Engine:
         # first use of a data type and of these shapes (about 50 ms for the first portion otherwise)
         for count in sorted({self.config.max_prefill_chunk_size, self.config.max_num_batched_tokens}):
             self.runner.warm_prefill(count)  # (a step's portions together may reach the token budget)
-        if self.config.decode_lookahead:
-            self.runner.warm_device_ids()
         torch.cuda.synchronize()
 
     def tune_matrix_products(self, token_counts: Sequence[int]) -> int:

@@ -215,19 +215,6 @@ class ModelRunner:
         ctx = self.builder.build([StepEntry(null_seq, [0] * num_tokens, 0, [num_tokens - 1])], self.ops, self.dtype, self.workspace)
         self._forward(ctx)
 
-    @torch.no_grad()
-    def warm_device_ids(self) -> None:
-        """Runs decode steps on the null page whose token ids are taken from a device tensor, for one row and for as many
-        rows as a step may hold, and drops the results: the gather and scatter kernels behind ``device_ids`` are loaded
-        at their first use (55 + 10 ms on MI355X, once for few indices and once for many), which the first request
-        would otherwise pay between its first and its second step."""
-        from ..cache.manager import SequenceCache
-
-        null_seq = SequenceCache(slot=self.cache.state.pad_slot, tables=[[0] for _ in self.cache.groups], released=[0 for _ in self.cache.groups])
-        for rows in sorted({1, self.max_num_seqs}):
-            tokens = torch.zeros(rows, dtype=torch.int32, device=self.device)
-            self.step([StepEntry(null_seq, [0], 0, [0]) for _ in range(rows)], device_ids=(tokens, list(range(rows)), list(range(rows))))
-
     def _replay(self, bucket: int, entries: Sequence[StepEntry], device_ids: Optional[tuple] = None) -> torch.Tensor:
         graph, logits, _ = self._graphs[bucket]
         if bucket in self._short_graphs and all(e.start < SHORT_CONTEXT_KEYS for e in entries):

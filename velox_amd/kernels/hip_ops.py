@@ -100,6 +100,7 @@ class HipOps:
     def _declare_core(self) -> None:
         c = self._core
         c.velox_embed.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
+        c.velox_place_tokens.argtypes = [_P, _P, _P, _P, _I, _I, _I, _P]
         c.velox_add_rmsnorm.argtypes = [_P, _P, _P, _P, _P, _I, _I, _F, _I, _I, _I, ctypes.c_longlong, _P]
         c.velox_skinny_qkv_rotary_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _I, _P]
         c.velox_silu_mul.argtypes = [_P, _P, _I, _I, _I, _P]
@@ -131,7 +132,7 @@ class HipOps:
         c.velox_probe_read.restype = _I
         c.velox_probe_mfma.argtypes = [_I, _I, _P, _P]
         c.velox_probe_mfma.restype = _I
-        for fn in (c.velox_embed, c.velox_add_rmsnorm, c.velox_silu_mul, c.velox_rope_kv_write, c.velox_gemm_fma,
+        for fn in (c.velox_embed, c.velox_place_tokens, c.velox_add_rmsnorm, c.velox_silu_mul, c.velox_rope_kv_write, c.velox_gemm_fma,
                    c.velox_argmax, c.velox_sample, c.velox_sample_chunked, c.velox_apply_penalties, c.velox_count_tokens, c.velox_count_sampled,
                    c.velox_penalties_from_counts):
             fn.restype = _I
@@ -264,6 +265,18 @@ class HipOps:
         status = self._core.velox_embed(_ptr(token_ids), _ptr(table), _ptr(out), token_ids.shape[0], hidden, vocab, _code(table.dtype), self._stream())
         self._launched(status, "embed")
         return out
+
+    def place_tokens(self, ids: torch.Tensor, dest: torch.Tensor, source: torch.Tensor, tokens: torch.Tensor, count: int) -> None:
+        """``ids[dest[k]] = tokens[source[k]]`` for ``k < count``, all int32 on the device: token ids that the step in flight
+        is still sampling, put into this step's rows without a trip to the host."""
+        for name, t in (("ids", ids), ("dest", dest), ("source", source), ("tokens", tokens)):
+            self._check(name, t, torch.int32)
+            if t.dim() != 1:
+                raise KernelError(f"place_tokens: {name} must have one dimension")
+        if count < 0 or count > dest.numel() or count > source.numel():
+            raise KernelError(f"place_tokens: {count} pairs do not fit dest [{dest.numel()}] and source [{source.numel()}]")
+        status = self._core.velox_place_tokens(_ptr(ids), _ptr(dest), _ptr(source), _ptr(tokens), int(count), ids.numel(), tokens.numel(), self._stream())
+        self._launched(status, "place_tokens")
 
     def _norm(self, residual, delta, rows, weight, eps, out_dtype):
         self._check("residual", residual, torch.float32)
