@@ -64,6 +64,28 @@ def test_four_ways_of_cutting(tmp_path, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", [21, 22, 23, 24, 25, 26])
+def test_mixed_traces_in_more_random_orders(tmp_path, seed, dtype):
+    """Other orders of arrival, other cuts and other requests that are ended half way and fed again, one configuration
+    per seed: up to four live requests, portions beside single tokens, a pool smaller than the requests' sum."""
+    name = "ABC"[seed % 3]
+    folder = make_folder(tmp_path, name, storage_for(dtype))
+    config, weights = read_model_folder(folder)
+    lengths = [33 + (seed * 7 + 29 * i) % 110 for i in range(8)]
+    requests = rc.request_set(config["vocab_size"], lengths, seed=seed)
+    expected = rc.expected_logits(config, weights, requests)
+    page = PAGE_SIZE[name]
+    again = tuple(f"r{i}" for i in range(8) if (seed + i) % 3 == 0)
+    trace = rc.mixed(requests, seed=seed, preempt=again)
+    replayer = Replayer(folder, dtype, rc.tokens_needed(trace, page), block_size=page)
+    got = rc.collect(trace, rc.run_trace(replayer, trace), requests)
+    for rid in requests:
+        torch.testing.assert_close(got[rid], expected[rid], msg=lambda m: f"{name} {dtype} seed {seed} {rid}: {m}", **TOL[dtype])
+    assert sum((len(t) + page - 1) // page for t in requests.values()) > replayer.cache.num_total_pages
+    replayer.cache.assert_consistent([])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_and_first_tokens(tmp_path, dtype):
     folder = make_folder(tmp_path, "B", storage_for(dtype))
     config, weights = read_model_folder(folder)
