@@ -134,7 +134,10 @@ def report(result: Dict, engine, show_outputs: bool) -> None:
     for stage, values in engine.stats.items():
         s = summarise(values)
         print(f"  {stage:<20}{s['n']:>7}{s['mean']:>10.3f}{s['p50']:>10.3f}{s['p90']:>10.3f}{s['p99']:>10.3f}{sum(values) / 1000:>11.3f}")
-    print(f"\n  HIP graphs    : {'on' if engine.runner.uses_graphs else 'off'}")
+    gpu_ms = sum(engine.stats.get("gpu_ms", []))
+    busy = gpu_ms / 1000 / result["wall_seconds"] if result["wall_seconds"] else 0.0
+    print(f"\n  GPU busy      : {gpu_ms / 1000:.3f} s  ({busy:.1%} of wall time)")
+    print(f"  HIP graphs    : {'on' if engine.runner.uses_graphs else 'off'}")
     print(f"  Peak GPU alloc: {torch.cuda.max_memory_allocated() / 1e9:.3f} GB")
     if show_outputs:
         rule("SAMPLE OUTPUTS (token ids)")

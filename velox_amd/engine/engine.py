@@ -42,6 +42,7 @@ class _Flight:
     landing: Optional[tuple] = None  # (pinned host tensor the tokens are copied to, event recorded behind the copy)
     booked: bool = False  # positions advanced and room made for the sampled tokens (Engine._book)
     expected: Optional[List[Optional[int]]] = None  # per sampled row: the token's index in the request's output, None = nobody waits for it
+    timer: Optional[tuple] = None  # (event before the step's first kernel, event behind its last): the device's time for it
 
     def requests(self) -> List[Request]:
         return self.decode + [portion.request for portion in self.prefill]
@@ -49,7 +50,7 @@ class _Flight:
 
 logger = logging.getLogger(__name__)
 
-_STAGES = ("scheduler_ms", "prepare_ms", "forward_ms", "sampling_ms", "cpu_sync_wait_ms", "step_ms")
+_STAGES = ("scheduler_ms", "prepare_ms", "forward_ms", "sampling_ms", "cpu_sync_wait_ms", "step_ms", "gpu_ms")
 
 
 def build_model(model_config, dtype: torch.dtype, device, max_position: Optional[int] = None) -> DecoderModel:
@@ -93,6 +94,7 @@ class Engine:
         self._pending_aborts: "queue.Queue[str]" = queue.Queue()
         self._landings = []
         self._next_landing = 0
+        self._timers: List[tuple] = []  # event pairs of queued steps whose device time has not been read yet
         if self.device.type == "cuda":
             rows = max(config.max_num_seqs, 1)
             self._landings = [(torch.zeros(rows, dtype=torch.int32, pin_memory=True), torch.cuda.Event()) for _ in range(3)]
@@ -316,6 +318,10 @@ class Engine:
                 sampled.append(request)
             at += count
 
+        timer = None
+        if self.device.type == "cuda":
+            timer = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+            timer[0].record()
         t0 = time.perf_counter()
         logits = self.runner.step(entries, device_ids=(pending.tokens, dest_rows, source_rows) if dest_rows else None)
         self.stats["prepare_ms"].append(self.runner.last_prepare_ms)
@@ -338,12 +344,14 @@ class Engine:
         # the copy of the tokens to the host is queued right behind the sampler, before a later step can be queued
         # behind it: waiting for it then waits for this step only
         landing = None
+        if timer is not None:
+            timer[1].record()
         if tokens_gpu is not None and self.device.type == "cuda":
             landing = self._landings[self._next_landing]
             self._next_landing = (self._next_landing + 1) % len(self._landings)
             landing[0][: len(sampled)].copy_(tokens_gpu, non_blocking=True)
             landing[1].record()
-        return _Flight(list(plan.decodes), list(plan.portions), sampled, tokens_gpu, landing)
+        return _Flight(list(plan.decodes), list(plan.portions), sampled, tokens_gpu, landing, timer=timer)
 
     def _book(self, flight: "_Flight") -> None:
         """What a queued step changes whatever tokens it draws: its positions are in the cache, and every sampled request
@@ -362,6 +370,8 @@ class Engine:
     def _finish_step(self, flight: "_Flight") -> None:
         """Waits for the step's tokens and hands them to their requests; stops."""
         self._book(flight)
+        if flight.timer is not None:
+            self._timers.append(flight.timer)
         if flight.tokens is None:
             return
         sync_start = time.perf_counter()
@@ -372,6 +382,10 @@ class Engine:
         else:
             tokens = flight.tokens.tolist()
         self.stats["cpu_sync_wait_ms"].append((time.perf_counter() - sync_start) * 1000)
+        # the device's time for the steps that have ended by now (this one has: its tokens are here)
+        while self._timers and self._timers[0][1].query():
+            begin, end = self._timers.pop(0)
+            self.stats["gpu_ms"].append(begin.elapsed_time(end))
         for request, index, token in zip(flight.sampled, flight.expected, tokens):
             if index is None:
                 continue  # it had stopped or been aborted before this step was booked
