@@ -272,6 +272,8 @@ def main() -> int:
             "hbm_read_gbs": round(read_gbs, 1), "mfma_bf16_tflops": round(mfma_tflops, 1),
             "decode_frac_of_read": round(achieved / read_gbs, 4),
         }
+        if args.dtype == "bf16":
+            result["probes"]["prefill_frac_of_mfma"] = round(flops / prefill_s / 1e12 / mfma_tflops, 4)
     print(json.dumps(result))
     return 0
 
