@@ -10,11 +10,12 @@ step function.  The one host wait per step is the read of the sampled tokens
 """
 from __future__ import annotations
 
+import collections
 import logging
 import queue
 import time
 from dataclasses import dataclass
-from typing import Dict, FrozenSet, Iterable, List, Optional, Sequence
+from typing import Deque, Dict, FrozenSet, Iterable, List, Optional, Sequence
 
 import torch
 
@@ -86,7 +87,8 @@ class Engine:
             enable_graphs=config.enable_cuda_graphs,
         )
         self.sampler = Sampler(ops, self.device, seed=config.seed)
-        self.stats: Dict[str, List[float]] = {name: [] for name in _STAGES}
+        # per-step times by stage, the most recent 65,536 steps (an engine that serves for days does not grow)
+        self.stats: Dict[str, Deque[float]] = {name: collections.deque(maxlen=65536) for name in _STAGES}
         self.num_steps = 0
         self._ahead: Optional[_Flight] = None
         # requests and aborts handed over by other threads, taken in at the start of the next step
