@@ -365,6 +365,70 @@ def test_many_penalised_requests_admitted_in_one_step_with_captured_steps(tmp_pa
     assert engine.sampler._seen.row_of_request == {} and engine.sampler._seen.table.shape[0] >= 40
 
 
+def test_two_hundred_requests_of_every_kind_in_a_small_pool_and_in_a_roomy_one(tmp_path):
+    """Greedy, penalised, sampled and sampled-with-penalties requests, some with stop tokens, some behind a shared stem,
+    arriving in bursts: once with a pool so small that requests are preempted hundreds of times, captured decode steps,
+    every step launched ahead and shared prefixes; once with room for all, one step at a time, nothing captured or
+    shared.  float32, so both give every request the same tokens.  Then the same with requests aborted at random: the
+    cache, the slots and the sampler's tables are left clean."""
+    import random
+
+    folder = make_folder(tmp_path, "B")
+    config, _ = read_model_folder(folder)
+    vocab = config["vocab_size"]
+
+    def make_requests(tag, count, seed):
+        rng = random.Random(seed)
+        stem = [rng.randrange(vocab) for _ in range(40)]
+        made = []
+        for i in range(count):
+            kind = rng.random()
+            prompt = (stem[:rng.choice([0, 16, 32, 40])] if rng.random() < 0.5 else []) + [rng.randrange(vocab) for _ in range(rng.randint(1, 70))]
+            options = dict(max_tokens=rng.randint(1, 40), ignore_eos=rng.random() < 0.7)
+            if kind < 0.4:
+                options.update(temperature=0.0)
+            elif kind < 0.6:
+                options.update(temperature=0.0, repetition_penalty=1.3, frequency_penalty=0.1)
+            elif kind < 0.8:
+                options.update(temperature=0.8, top_p=0.9, seed=i)
+            else:
+                options.update(temperature=0.7, top_k=20, top_p=0.8, repetition_penalty=1.05, seed=1000 + i)
+            if rng.random() < 0.2:
+                options["stop_token_ids"] = [rng.randrange(vocab) for _ in range(20)]
+            made.append(Request(f"{tag}{i}", prompt, SamplingParams(**options)))
+        return made
+
+    def run(tag, count, seed, aborts, **options):
+        engine = engine_for(folder, "B", max_num_seqs=8, max_num_batched_tokens=64, max_prefill_chunk_size=24, **options)
+        requests = make_requests(tag, count, seed)
+        rng = random.Random(seed + 1)
+        waiting, steps = list(requests), 0
+        while waiting or engine.has_work():
+            if steps % 25 == 0:
+                for _ in range(rng.randint(4, 14)):
+                    if waiting:
+                        engine.add_request(waiting.pop(0))
+            if aborts and rng.random() < 0.05 and engine.scheduler.running:
+                engine.abort_request(rng.choice(engine.scheduler.running).request_id)
+            engine.step()
+            steps += 1
+            if steps % 100 == 0:
+                engine.cache.assert_consistent([r.cache for r in engine.scheduler.running if r.cache is not None])
+        engine.cache.assert_consistent([])
+        assert engine.cache.num_used_pages() == (engine.cache.prefix.num_nodes if engine.cache.prefix is not None else 0)
+        assert engine.sampler._seen.row_of_request == {} and engine.sampler._seeds == {}
+        assert all(r.finished and -1 not in r.all_token_ids for r in requests)
+        return requests, engine
+
+    tight, engine = run("t", 200, 5, False, num_gpu_blocks=40, enable_cuda_graphs=True, decode_lookahead=True, enable_prefix_caching=True)
+    assert engine.scheduler.num_preemptions > 50 and engine.runner.num_graph_replays > 100 and engine.cache.prefix.num_hits > 0
+    roomy, _ = run("t", 200, 5, False, num_gpu_blocks=400, enable_cuda_graphs=False, decode_lookahead=False, enable_prefix_caching=False)
+    for a, b in zip(tight, roomy):
+        assert a.output_token_ids == b.output_token_ids and a.finish_reason is b.finish_reason, (a.request_id, a.sampling_params, a.output_token_ids, b.output_token_ids)
+    aborted, _ = run("x", 200, 9, True, num_gpu_blocks=40, enable_cuda_graphs=True, decode_lookahead=True, enable_prefix_caching=True)
+    assert sum(r.finish_reason.name == "ABORT" for r in aborted) > 10
+
+
 def test_pool_sized_from_free_memory_when_no_page_count_is_given(tmp_path):
     """``num_gpu_blocks=None``: the pool takes what the free memory allows (reference ``src/paged_kv_cache.py:159-194``), capped at
     what ``max_num_seqs`` requests of ``max_model_len`` tokens can ever hold; a utilisation that leaves nothing is an error."""
