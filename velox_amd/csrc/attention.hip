@@ -872,9 +872,22 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
   if (WIDE == 2 && rows > 64 && (long long)total_tokens * group / 128 * nkv * splits >= compute_units()) {
     if (max_kv_len - max_q_len / 2 <= 1280 || rows < 192) {  // (keys an average row reads)
       dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
-      paged_attention_kernel<T, BN, 1, 1, 8><<<grid, 512, 0, stream>>>(
-          (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+      // With enough workgroups to keep two on every compute unit, the 128 rows go to four waves of two row tiles: half
+      // the reads of K and V^T from LDS per row, which bound this kernel.  Measured on MI355X (us, eight waves of one
+      // tile against four of two): 4 x 512 tokens behind 1,024 keys 62.7 / 54.7, 2,048 tokens from an empty cache
+      // 75.0 / 71.5, two such sequences 130.9 / 108.5 (28 heads over 4); 93.8 / 77.9 and 171.9 / 147.3 with 40 heads
+      // over 8.  With fewer workgroups the eight waves hide more of a short stream's latency (12 heads over 2, two
+      // sequences of 2,048: 61.5 / 75.8).
+      const long long workgroups = (long long)grid.x * grid.y * grid.z;
+      if (rows >= 256 && workgroups * 4 >= 7LL * compute_units()) {
+        paged_attention_kernel<T, BN, 2, 1, 4><<<grid, 256, 0, stream>>>(
+            (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+            part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+      } else {
+        paged_attention_kernel<T, BN, 1, 1, 8><<<grid, 512, 0, stream>>>(
+            (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
+            part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+      }
     } else {
       dim3 grid((rows + 255) / 256, nkv, num_seqs * splits);
       paged_attention_kernel<T, BN, WIDE, 1, 8><<<grid, 512, 0, stream>>>(
