@@ -221,7 +221,7 @@ def main(argv=None) -> int:
             # a ladder of step sizes up to the token budget: a step is padded up to the next one when that is close
             budget = max(args.max_num_batched_tokens, max_num_seqs)
             ladder = sorted({args.max_prefill_chunk_size, budget} | {n for n in range(128, budget + 1, 128) if n * 8 >= budget})
-            engine.tune_matrix_products(ladder + [b for b in decode_buckets(max_num_seqs) if b > 16])
+            engine.tune_matrix_products(ladder + [b for b in decode_buckets(max_num_seqs) if b > 16], progress=lambda text: print(f"  [tune] {text}", flush=True))
         vocab = engine.model.spec.vocab_size
         limit = engine.max_model_len - args.max_tokens - 1
         if limit < 1:

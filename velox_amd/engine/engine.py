@@ -162,13 +162,14 @@ class Engine:
             self.runner.warm_prefill(count)  # (a step's portions together may reach the token budget)
         torch.cuda.synchronize()
 
-    def tune_matrix_products(self, token_counts: Sequence[int]) -> int:
+    def tune_matrix_products(self, token_counts: Sequence[int], progress=None) -> int:
         """Optional, bfloat16 only: has the matrix library time its candidate kernels for this model's weight shapes at
         the given numbers of tokens per step (typically the prefill chunk size and the larger decode batch sizes) and
         keep the fastest.  Takes seconds per shape.  A step of prompt portions with a few rows less than one of these
         counts is padded up to it from then on (``ModelRunner.tuned_row_counts``); other steps are unaffected.  Only products that
         the engine hands to the library are timed (``ops.library_serves``); captured decode steps are captured again
-        if one of them holds such a product."""
+        if one of them holds such a product.  ``progress(text)``, if given, is told after every count (a ladder of
+        counts takes minutes)."""
         if self.dtype != torch.bfloat16 or self.device.type != "cuda" or not hasattr(self.ops, "tune_library_products"):
             return 0
         shapes = set()
@@ -179,10 +180,13 @@ class Engine:
                     shapes.add(tuple(tensor.shape))
         done = 0
         recapture = False
-        for count in sorted(set(int(m) for m in token_counts)):
+        counts = sorted(set(int(m) for m in token_counts))
+        for index, count in enumerate(counts):
             served = [shape for shape in shapes if self.ops.library_serves(count, *shape)]
             if served:
                 done += self.ops.tune_library_products(served, [count])
+                if progress is not None:
+                    progress(f"timed the library's kernels for steps of {count} rows ({index + 1} of {len(counts)} counts, {len(served)} products)")
                 recapture = recapture or count <= self.config.max_num_seqs
                 if count > self.config.max_num_seqs and count not in self.runner.tuned_row_counts:
                     self.runner.tuned_row_counts = sorted(self.runner.tuned_row_counts + [count])  # steps a little shorter are padded up to it
