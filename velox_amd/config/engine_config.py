@@ -69,6 +69,9 @@ class EngineConfig:
     scatter_pages: bool = True
     # launch a decode step's successor before reading the step's tokens (not a reference option)
     decode_lookahead: bool = True
+    # where ``Engine.tune_matrix_products`` keeps what the matrix library's timings found, so that a later start does not
+    # time the same shapes again: "auto" = beside the built kernel libraries, None = nowhere (not a reference option)
+    library_tuning_file: Optional[str] = "auto"
     watermark: float = 0.01
 
     seed: Optional[int] = None

@@ -180,11 +180,12 @@ class Engine:
                     shapes.add(tuple(tensor.shape))
         done = 0
         recapture = False
+        results_file = self.ops.tuning_file() if self.config.library_tuning_file == "auto" else self.config.library_tuning_file
         counts = sorted(set(int(m) for m in token_counts))
         for index, count in enumerate(counts):
             served = [shape for shape in shapes if self.ops.library_serves(count, *shape)]
             if served:
-                done += self.ops.tune_library_products(served, [count])
+                done += self.ops.tune_library_products(served, [count], results_file=results_file)
                 if progress is not None:
                     progress(f"timed the library's kernels for steps of {count} rows ({index + 1} of {len(counts)} counts, {len(served)} products)")
                 recapture = recapture or count <= self.config.max_num_seqs

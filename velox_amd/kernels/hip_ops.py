@@ -204,14 +204,28 @@ class HipOps:
             return True
         return m > 16 and n > 8192 and n * k >= (32 << 20)
 
-    def tune_library_products(self, shapes, token_counts, seconds_per_shape: float = 0.2) -> int:
+    def tuning_file(self) -> Optional[str]:
+        """Where timings of the matrix library's kernels are kept between runs by default: beside the built kernel
+        libraries, one file per kind of GPU (the file's own header names the library versions it holds for, and
+        TunableOp refuses a file made by others)."""
+        directory = next((d for d in build.build_dirs() if build._writable(d)), None)
+        arch = torch.cuda.get_device_properties(self.device).gcnArchName.split(":")[0]
+        return os.path.join(directory, f"tunableop_{arch}.csv") if directory else None
+
+    def tune_library_products(self, shapes, token_counts, seconds_per_shape: float = 0.2, results_file: Optional[str] = None) -> int:
         """Lets PyTorch's TunableOp time the library's candidate kernels for ``x[M, K] @ w[N, K]^T`` at the given
         ``(N, K)`` shapes and ``M`` values, and keeps its choices for later calls.  Tuning stays off afterwards, so
-        other shapes keep the library's default choice and never pay for a search.  Returns the number of products tuned."""
+        other shapes keep the library's default choice and never pay for a search.  ``results_file``: what was found is
+        kept there, and shapes that an earlier run has timed are not timed again.  Returns the number of products run."""
         tunable = torch.cuda.tunable
         tunable.enable(True)
-        # the library writes what it found to a file when the process ends: keep that out of the working folder
-        tunable.set_filename(os.path.join(tempfile.gettempdir(), f"velox_amd_tunableop_{os.getuid()}_{os.getpid()}.csv"))
+        if results_file is None:
+            # TunableOp writes what it finds to a file: keep that out of the working folder
+            results_file = os.path.join(tempfile.gettempdir(), f"velox_amd_tunableop_{os.getuid()}_{os.getpid()}.csv")
+        if tunable.get_filename() != results_file:
+            tunable.set_filename(results_file)
+            if os.path.isfile(results_file) and not tunable.read_file(results_file):
+                os.remove(results_file)  # made with other versions of the libraries: start again
         tunable.set_max_tuning_duration(int(seconds_per_shape * 1000))
         tunable.tuning_enable(True)
         done = 0
