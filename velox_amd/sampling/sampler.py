@@ -77,6 +77,9 @@ class _SeenCounts:
         row = self.row_of_request.get(request_id)
         if row is not None:
             return row
+        tokens = np.asarray(history(), dtype=np.int32)
+        if tokens.size and int(tokens.min()) < 0:
+            raise ValueError(f"request {request_id}: its history holds a token that is still being sampled")
         if self.table is None or self.table.shape[1] != vocab:
             self.table = torch.zeros((8, vocab), dtype=torch.int32, device=self.device)
             self.row_of_request.clear()
@@ -87,9 +90,6 @@ class _SeenCounts:
             self.free_rows = list(range(2 * rows - 1, rows - 1, -1))
         row = self.free_rows.pop()
         self.row_of_request[request_id] = row
-        tokens = np.asarray(history(), dtype=np.int32)
-        if tokens.size and int(tokens.min()) < 0:
-            raise ValueError(f"request {request_id}: its history holds a token that is still being sampled")
         self.table[row].zero_()
         if tokens.size:
             self.ops.count_tokens(self.table[row], self.upload.send(tokens))
