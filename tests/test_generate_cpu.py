@@ -289,3 +289,59 @@ def test_penalties_keep_their_counts_through_early_launches_and_preemption(tmp_p
         for index, request in enumerate(done):
             assert request.output_token_ids == expected[index], (lookahead, index, request.output_token_ids, expected[index])
         assert engine.sampler._seen.row_of_request == {} and engine.sampler._seeds == {}
+
+
+def test_a_request_that_stops_on_the_token_pending_at_its_preemption_is_not_admitted_again(tmp_path):
+    """With the next step decided before this one's tokens are read, a request can lose its pages while its newest token
+    is still in flight, and wait.  If that token ends it (a stop token), it ends while it waits: it must leave the queue,
+    never take pages or a slot again, and the sampler must hold nothing of it."""
+    from velox_amd.engine.request import PENDING_TOKEN
+
+    folder = make_folder(tmp_path, "B")
+    config, weights = read_model_folder(folder)
+    steps = 20
+    found = 0
+    for lengths, pages in (((20, 31, 12, 25), 9), ((8, 50, 40, 12), 13), ((8, 50, 40, 12), 18)):
+        prompts = [random_tokens(config["vocab_size"], n, seed=42 + n) for n in lengths]
+
+        def build(stops):
+            engine = engine_for(folder, "B", num_gpu_blocks=pages, watermark=0.01)
+            requests = [Request(f"q{i}", p, SamplingParams(temperature=0.8, top_k=20, seed=7 + i, max_tokens=steps, stop_token_ids=stops.get(i, [])))
+                        for i, p in enumerate(prompts)]
+            return engine, requests
+
+        # first run: who waits, after a scheduling decision, with its newest token still pending, and what that token is
+        engine, requests = build({})
+        events = []
+        inner = engine.scheduler.schedule
+
+        def schedule():
+            plan = inner()
+            events.extend((requests.index(r), len(r.output_token_ids) - 1) for r in engine.scheduler.waiting if r.all_token_ids[-1] == PENDING_TOKEN)
+            return plan
+
+        engine.scheduler.schedule = schedule
+        engine.generate(requests)
+        usable = [(who, at) for who, at in events if requests[who].output_token_ids[at] not in requests[who].output_token_ids[:at]]
+        if not usable:
+            continue
+        who, at = usable[0]
+        stop_token = requests[who].output_token_ids[at]
+        reference = [list(r.output_token_ids) for r in requests]
+
+        # second run: that token is a stop token of that request
+        engine, again = build({who: [stop_token]})
+        admissions_after_end = []
+        for request in again:
+            inner_admitted = request.admitted
+            request.admitted = lambda cache, cached, request=request, inner_admitted=inner_admitted: (
+                admissions_after_end.append(request.request_id) if request.finished else None, inner_admitted(cache, cached))[1]
+        engine.generate(again)
+        assert again[who].finish_reason is FinishReason.STOP and again[who].output_token_ids == reference[who][:at + 1]
+        assert admissions_after_end == []
+        assert engine.sampler._seen.row_of_request == {} and engine.sampler._seeds == {}
+        assert engine.cache.num_used_pages() == 0 and not engine.scheduler.requests
+        engine.cache.assert_consistent([])
+        assert engine.snapshot()["num_finished"] == 4.0
+        found += 1
+    assert found > 0  # the case did occur

@@ -50,6 +50,39 @@ def test_greedy_generation_matches_plain(tmp_path, name):
     engine.cache.assert_consistent([])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_an_engine_over_weights_drawn_on_the_device_computes_the_plain_models_logits(name, dtype):
+    """``Engine.from_random(generator_device="cuda")`` is what every measurement runs on: its tensors, read back under
+    their checkpoint names, give the plain model the engine's logits and tokens (fused rows, the tied head, held dtypes
+    and the kernels' copies of the weights are all behind them)."""
+    from helpers import CONFIGS
+    from velox_amd.weights import named_tensors
+
+    config = CONFIGS[name]
+    engine = Engine.from_random(config, seed=21, config=EngineConfig(
+        dtype=dtype, device="cuda", max_model_len=160, max_num_seqs=4, max_num_batched_tokens=32, max_prefill_chunk_size=7,
+        block_size=PAGE_SIZE[name], num_gpu_blocks=96, enable_cuda_graphs=False, seed=0, enable_prefix_caching=False), generator_device="cuda")
+    weights = {key: value.float().cpu() for key, value in named_tensors(engine.model)}
+    assert ("lm_head.weight" in weights) != bool(config["tie_word_embeddings"])
+    assert abs(float(weights["model.norm.weight"].mean()) - 1.0) < 0.05 and abs(float(weights["model.embed_tokens.weight"].std()) - 0.02) < 0.003
+    prompts = [random_tokens(config["vocab_size"], n, seed=n) for n in (5, 9, 13, 40)]
+    done = engine.generate(greedy(prompts, 6))
+    from velox_amd.engine.batch import StepEntry
+    for request, prompt in zip(done, prompts):
+        if dtype == "float32":
+            assert request.output_token_ids == plain_greedy(config, weights, prompt, 6)
+        # the logits of the whole sequence in one step
+        tokens = prompt + request.output_token_ids
+        sequence = engine.cache.new_sequence()
+        assert engine.cache.append(sequence, 0, len(tokens))
+        got = engine.runner.step([StepEntry(sequence, tokens, 0, list(range(len(tokens))))]).float().cpu()
+        engine.cache.free_sequence(sequence)
+        want = qwen2_logits(config, weights, tokens)
+        tolerance = dict(rtol=2e-4, atol=2e-5) if dtype == "float32" else dict(rtol=5e-2, atol=3e-2)  # (those of the whole-prompt tests)
+        torch.testing.assert_close(got, want, **tolerance)
+
+
 def test_graph_decode_equals_eager_decode_and_preemption_keeps_tokens(tmp_path):
     """float32: every kernel is this repository's own and sums in a fixed order, so the tokens must be identical."""
     dtype = "float32"
@@ -262,8 +295,12 @@ def test_batches_of_every_size_class_with_layers_of_the_real_size(tmp_path):
         assert engine.runner.num_graph_replays >= replays + 4
         for request, prompt in list(zip(done, prompts))[::max(1, count // 6)]:
             logits = qwen2_logits(config, weights, prompt + request.output_token_ids[:-1])[len(prompt) - 1:]
+            # a bfloat16 run's logits differ from the plain model's by at most 1.75% of their spread in the root mean square
+            # (the bound the replayed logits at these widths are held to).  The engine's best token can then stand below
+            # the plain best by the errors of two logits: six such deviations are allowed, far out for two chosen logits
+            margin = 6 * 0.0175 * float(logits.std())
             for step, token in enumerate(request.output_token_ids):
-                assert logits[step][token] >= logits[step].max() - 0.2, (count, request.request_id, step)
+                assert logits[step][token] >= logits[step].max() - margin, (count, request.request_id, step, margin)
     engine.cache.assert_consistent([])
 
 

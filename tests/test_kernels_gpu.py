@@ -651,10 +651,12 @@ def test_sampling_keeps_exactly_the_tokens_the_filters_allow(ops, vocab, spread)
     """The threshold of top-k / top-p at the real vocabulary size, flat and peaked rows, ties across the threshold: over many
     draws per row, every drawn token is one the plain filter keeps, and the tokens at the filter's edge (the last kept ones)
     are drawn as well, so the kept set is neither too small nor too large.  A row's draw does not depend on its place."""
-    settings = [(0.8, 0.9, 0), (1.0, 1.0, 7), (0.7, 0.5, 50), (1.3, 0.95, 1000), (1.0, 0.999, 0), (0.5, 0.3, 3), (1.0, 1.0, 0), (2.0, 0.6, 20000)]
+    settings = [(0.8, 0.9, 0), (1.0, 1.0, 7), (0.7, 0.5, 50), (1.3, 0.95, 1000), (1.0, 0.999, 0), (0.5, 0.3, 3), (1.0, 1.0, 0), (2.0, 0.6, 20000),
+                (1.0, 1e-20, 0), (1.0, 1.0, 2)]  # a share of the mass so small that it rounds to nothing: the best token is still kept
     base = rand((len(settings), vocab), torch.float32, 77, spread)
     base[2, 5] = base[2, 11] = base[2, vocab - 1] = float(base[2].max()) + 0.5  # three equal tokens at the top
     base[5, :40] = float(base[5].max())  # forty equal tokens: rank 0 for all of them, so top_k = 3 keeps all forty
+    base[9, 3], base[9, 8], base[9, 100], base[9, vocab - 2] = (float(base[9].max()) + x for x in (1.0, 0.5, 0.5, 0.5))  # top_k = 2 with three tokens tied at the cut
     draws = 300
     logits = base.repeat_interleave(draws, 0).contiguous()
     options = np.zeros((len(settings) * draws, 6), dtype=np.int32)
@@ -681,6 +683,10 @@ def test_sampling_keeps_exactly_the_tokens_the_filters_allow(ops, vocab, spread)
         for j in (0, 1, draws - 1):
             token, scores = TorchOps.sample_row(base[r].cpu().numpy(), options[r * draws + j])
             assert scores[drawn[j]] >= scores.max() - 1e-3, (r, j, int(drawn[j]), token)
+    # stated without the plain filter: a share of the mass of nothing keeps the one best token, and a cut of top-k that falls
+    # into a run of equal logits keeps the whole run (the reference keeps exactly k by sorted position, engine/sampler.py:218-221)
+    assert set(got[8 * draws:9 * draws]) == {int(base[8].argmax())}
+    assert set(got[9 * draws:10 * draws]) == {3, 8, 100, vocab - 2}
     # the same rows in another order and beside other rows: the same tokens
     order = torch.randperm(len(settings) * draws, generator=torch.Generator().manual_seed(5))[:97]
     again = ops.sample(logits[order.cuda()].contiguous(), torch.from_numpy(options[order.numpy()]).cuda()).cpu().numpy()
@@ -693,7 +699,8 @@ def test_sampling_with_rows_cut_into_chunks_gives_the_same_tokens(ops, vocab, sp
     added up in global memory: the tokens are those of the one-workgroup kernel, bit for bit, for every number of chunks
     (chunks that end inside the last quad, chunks beyond the row's end, rows that start off a 16-byte boundary), for
     greedy rows, rows without a filter and rows with one, side by side."""
-    settings = [(0.8, 0.9, 0), (1.0, 1.0, 7), (0.0, 1.0, 0), (0.7, 0.5, 50), (1.3, 0.95, 1000), (1.0, 0.999, 0), (0.5, 0.3, 3), (1.0, 1.0, 0), (2.0, 0.6, 20000)]
+    settings = [(0.8, 0.9, 0), (1.0, 1.0, 7), (0.0, 1.0, 0), (0.7, 0.5, 50), (1.3, 0.95, 1000), (1.0, 0.999, 0), (0.5, 0.3, 3), (1.0, 1.0, 0), (2.0, 0.6, 20000),
+                (1.0, 1e-20, 0)]
     base = rand((len(settings), vocab), torch.float32, 78, spread)
     base[3, 5] = base[3, 11] = base[3, vocab - 1] = float(base[3].max()) + 0.5
     base[6, :40] = float(base[6].max())
@@ -711,6 +718,7 @@ def test_sampling_with_rows_cut_into_chunks_gives_the_same_tokens(ops, vocab, sp
     device_options = torch.from_numpy(options).cuda()
     whole = ops.sample(logits, device_options, chunks=1).cpu().numpy()
     assert whole[2 * draws] == 17
+    assert set(whole[9 * draws:10 * draws]) == {int(base[9].argmax())}  # top_p of nothing: the best token, not an id outside the vocabulary
     for chunks in (None, 2, 3, 7, 16, 64):
         got = ops.sample(logits, device_options, chunks=chunks).cpu().numpy()
         assert (got == whole).all(), (chunks, np.flatnonzero(got != whole)[:10], got[got != whole][:10], whole[got != whole][:10])

@@ -110,3 +110,102 @@ def test_tied_head_uses_the_embedding_table(tmp_path):
     weights2 = dict(weights)
     weights2["lm_head.weight"] = weights["model.embed_tokens.weight"]
     torch.testing.assert_close(qwen2_logits(untied, weights2, tokens, torch.float64), qwen2_logits(config, weights, tokens, torch.float64))
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_without_the_sub_layers_outputs_the_model_is_norm_of_the_embedding_times_head(tmp_path, name):
+    """With every o_proj and down_proj zero the sub-layers add nothing, and what is left fixes the residual's frame:
+    logits = final_norm(E[ids]) @ head^T.  A post-norm block (the residual itself normed), a residual that carries the
+    normed input on, or a scale on the embeddings would each leave something behind."""
+    folder = make_folder(tmp_path, name)
+    config, weights = read_model_folder(folder, torch.float64)
+    for key in weights:
+        if key.endswith("o_proj.weight") or key.endswith("down_proj.weight"):
+            weights[key] = torch.zeros_like(weights[key])
+    tokens = random_tokens(config["vocab_size"], 12, seed=8)
+    table = weights["model.embed_tokens.weight"]
+    head = table if config["tie_word_embeddings"] else weights["lm_head.weight"]
+    want = F.rms_norm(table[torch.tensor(tokens)], (config["hidden_size"],), weights["model.norm.weight"], config["rms_norm_eps"]) @ head.T
+    torch.testing.assert_close(qwen2_logits(config, weights, tokens, torch.float64), want, rtol=1e-10, atol=1e-12)
+    # and the feed-forward reads the NORMED residual: with the norm before it weighted zero it sees zeros and gives
+    # down(silu(0) * 0) = 0, as if its down_proj were zero
+    _, full = read_model_folder(folder, torch.float64)
+    silenced = dict(full)
+    for key in full:
+        if key.endswith("post_attention_layernorm.weight"):
+            silenced[key] = torch.zeros_like(full[key])
+    no_mlp = dict(full)
+    for key in full:
+        if key.endswith("down_proj.weight"):
+            no_mlp[key] = torch.zeros_like(full[key])
+    torch.testing.assert_close(qwen2_logits(config, silenced, tokens, torch.float64), qwen2_logits(config, no_mlp, tokens, torch.float64), rtol=1e-10, atol=1e-12)
+
+
+def test_one_layer_put_together_from_library_routines_only():
+    """One layer of the third tiny configuration (6 heads of 48 channels on a width of 80: head_dim is not width / heads)
+    assembled from ``F.rms_norm``, ``F.linear``, ``F.silu``, ``F.scaled_dot_product_attention`` with its DEFAULT scale
+    (1 / sqrt of the last dimension = 48) and the rotation pinned above.  It fixes what the reading alone fixed: the order
+    norm -> sub-layer -> add (twice), and the scale head_dim^-0.5 (width / heads = 13.3 would differ)."""
+    config = dict(CONFIGS["C"], num_hidden_layers=1)
+    hidden, nh, nkv, d, inner, vocab = 80, 6, 2, 48, 150, 263
+    generator = torch.Generator().manual_seed(5)
+
+    def draw(*shape, around=0.0):
+        return around + 0.02 * torch.randn(*shape, generator=generator, dtype=torch.float64)
+
+    p = "model.layers.0."
+    w = {"model.embed_tokens.weight": draw(vocab, hidden), "lm_head.weight": draw(vocab, hidden), "model.norm.weight": draw(hidden, around=1.0),
+         p + "input_layernorm.weight": draw(hidden, around=1.0), p + "post_attention_layernorm.weight": draw(hidden, around=1.0),
+         p + "self_attn.q_proj.weight": 8 * draw(nh * d, hidden), p + "self_attn.q_proj.bias": 8 * draw(nh * d),
+         p + "self_attn.k_proj.weight": 8 * draw(nkv * d, hidden), p + "self_attn.k_proj.bias": 8 * draw(nkv * d),
+         p + "self_attn.v_proj.weight": draw(nkv * d, hidden), p + "self_attn.v_proj.bias": draw(nkv * d),
+         p + "self_attn.o_proj.weight": draw(hidden, nh * d), p + "mlp.gate_proj.weight": draw(inner, hidden),
+         p + "mlp.up_proj.weight": draw(inner, hidden), p + "mlp.down_proj.weight": draw(hidden, inner)}
+    tokens = random_tokens(vocab, 17, seed=4)
+    t = len(tokens)
+    eps = config["rms_norm_eps"]
+    cos, sin = rope_tables(d, config["rope_theta"], t, factor=2.0, dtype=torch.float64)
+    positions = torch.arange(t)
+
+    h = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+    a = F.rms_norm(h, (hidden,), w[p + "input_layernorm.weight"], eps)
+    q = apply_rope(F.linear(a, w[p + "self_attn.q_proj.weight"], w[p + "self_attn.q_proj.bias"]).view(t, nh, d), cos, sin, positions)
+    k = apply_rope(F.linear(a, w[p + "self_attn.k_proj.weight"], w[p + "self_attn.k_proj.bias"]).view(t, nkv, d), cos, sin, positions)
+    v = F.linear(a, w[p + "self_attn.v_proj.weight"], w[p + "self_attn.v_proj.bias"]).view(t, nkv, d)
+    heads = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.repeat_interleave(nh // nkv, 1).transpose(0, 1)[None],
+                                           v.repeat_interleave(nh // nkv, 1).transpose(0, 1)[None], is_causal=True)[0].transpose(0, 1)
+    h = h + F.linear(heads.reshape(t, nh * d), w[p + "self_attn.o_proj.weight"])
+    m = F.rms_norm(h, (hidden,), w[p + "post_attention_layernorm.weight"], eps)
+    h = h + F.linear(F.silu(F.linear(m, w[p + "mlp.gate_proj.weight"])) * F.linear(m, w[p + "mlp.up_proj.weight"]), w[p + "mlp.down_proj.weight"])
+    want = F.linear(F.rms_norm(h, (hidden,), w["model.norm.weight"], eps), w["lm_head.weight"])
+
+    got = qwen2_logits(config, w, tokens, torch.float64)
+    torch.testing.assert_close(got, want, rtol=1e-9, atol=1e-11)
+    # the scores are large enough (q and k scaled up) for another scale to show: width / heads in place of head_dim
+    other = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.repeat_interleave(nh // nkv, 1).transpose(0, 1)[None],
+                                           v.repeat_interleave(nh // nkv, 1).transpose(0, 1)[None], is_causal=True, scale=(hidden / nh) ** -0.5)[0].transpose(0, 1)
+    assert float((other - heads).abs().max()) > 1e-4
+
+
+def test_what_the_filters_keep_when_logits_are_equal_at_the_cut():
+    """The plain sampler the kernels are compared with, on cases small enough to state by hand.  Tokens of equal value
+    share rank and mass, so a cut inside a run of equal logits keeps the whole run: top_k = 2 over [3, 2, 2, 2, 1] keeps four
+    tokens.  The reference keeps exactly k, whichever of the equal ones its sort puts first (engine/sampler.py:218-221)."""
+    import numpy as np
+    from torch_ops import TorchOps
+
+    def kept(row, temperature, top_p, top_k):
+        option = np.zeros(6, dtype=np.int32)
+        option.view(np.float32)[0:2] = (temperature, top_p)
+        option[2:] = (top_k, 11, 22, 0)
+        return sorted(np.flatnonzero(np.isfinite(TorchOps.sample_row(np.asarray(row, dtype=np.float32), option)[1])))
+
+    assert kept([3, 2, 2, 2, 1], 1.0, 1.0, 2) == [0, 1, 2, 3]
+    assert kept([3, 2, 2, 2, 1], 1.0, 1.0, 1) == [0]
+    assert kept([1, 2, 5, 2, 4], 1.0, 1.0, 2) == [2, 4]
+    # top-p: a token is kept while the mass of the strictly larger ones is below p; the best one always is
+    p = np.exp([3.0, 2, 2, 2, 1]) / np.exp([3.0, 2, 2, 2, 1]).sum()
+    assert kept([3, 2, 2, 2, 1], 1.0, float(p[0]) * 0.99, 0) == [0]
+    assert kept([3, 2, 2, 2, 1], 1.0, float(p[0]) * 1.01, 0) == [0, 1, 2, 3]
+    assert kept([3, 2, 2, 2, 1], 1.0, 1e-20, 0) == [0]
+    assert kept([3, 2, 2, 2, 1], 1.0, 1.0, 0) == [0, 1, 2, 3, 4]

@@ -177,3 +177,52 @@ def test_index_file_that_names_a_shard_that_is_not_there(tmp_path):
     os.unlink(os.path.join(folder, "model-00002-of-00002.safetensors"))
     with pytest.raises(FileNotFoundError, match="model-00002-of-00002.safetensors"):
         _load(folder)
+
+
+def test_random_weights_in_memory_go_through_the_binder_of_folders(tmp_path):
+    """``bind_random`` is the folder's binder fed from a stream of random tensors: fused rows, the tied head, held dtypes
+    and the values themselves are the folder's, and reading a bound model back by checkpoint name gives the folder's file."""
+    import velox_amd.weights.random_init as random_init
+    from velox_amd.weights import RandomSource, named_tensors
+
+    assert "setattr" not in open(random_init.__file__).read()
+    for name, config in (("A", TINY_A), ("B", TINY_B)):
+        folder = write_random_model(config, str(tmp_path / name), 11, "bfloat16")
+        raw = load_file(os.path.join(folder, "model.safetensors"))
+        for run_dtype in (torch.float32, torch.bfloat16):
+            from_folder = _load(folder, run_dtype)
+            in_memory = build_model(load_config(folder), run_dtype, "cpu")
+            bind_random(in_memory, 11, run_dtype, "cpu", storage_dtype=torch.bfloat16)
+            back = dict(named_tensors(in_memory))
+            assert sorted(back) == sorted(raw)
+            for key, stored in raw.items():
+                assert torch.equal(back[key].float(), stored.float()), key
+            for (_, a), (_, b) in zip(named_tensors(from_folder), named_tensors(in_memory)):
+                assert a.dtype == b.dtype and torch.equal(a, b)
+        tied = in_memory.head.weight.data_ptr() == in_memory.embedding.table.data_ptr()
+        assert tied == bool(config["tie_word_embeddings"])
+    # the stream has one generator: tensors out of the order of declaration are refused, not drawn from the wrong state
+    source = RandomSource(build_model(load_config(folder), torch.float32, "cpu"), 3)
+    with pytest.raises(RuntimeError, match="order of declaration"):
+        source.tensor("model.norm.weight")
+
+
+def test_unexpected_tensors_are_an_error_unless_told_to_ignore_them(tmp_path, capsys):
+    folder = make_folder(tmp_path, "A")
+    path = os.path.join(folder, "model.safetensors")
+    raw = load_file(path)
+    raw["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    save_file(raw, path)
+    with pytest.raises(WeightsError) as err:
+        _load(folder)
+    assert err.value.unexpected == ["model.layers.0.self_attn.rotary_emb.inv_freq"] and "ignore_unexpected_weights=True" in str(err.value)
+    model = build_model(load_config(folder), torch.float32, "cpu")
+    bind_from_checkpoint(model, folder, torch.float32, "cpu", ignore_unexpected=True)
+    assert "ignoring 1 tensors" in capsys.readouterr().out
+    assert torch.equal(model.final_norm.weight, raw["model.norm.weight"])
+    # a missing tensor is an error whatever is ignored
+    del raw["model.norm.weight"]
+    save_file(raw, path)
+    with pytest.raises(WeightsError) as err:
+        bind_from_checkpoint(model, folder, torch.float32, "cpu", ignore_unexpected=True)
+    assert err.value.missing == ["model.norm.weight"] and err.value.unexpected == ["model.layers.0.self_attn.rotary_emb.inv_freq"]

@@ -73,6 +73,9 @@ class EngineConfig:
     # time the same shapes again: "auto" = beside the built kernel libraries, None = nowhere (not a reference option)
     library_tuning_file: Optional[str] = "auto"
     watermark: float = 0.01
+    # tensors of the model folder that the model has no place for: False = an error that lists them, True = their number
+    # is printed and they are ignored (what the reference always does, ``src/weight_loader.py:131-136``)
+    ignore_unexpected_weights: bool = False
 
     seed: Optional[int] = None
 
@@ -80,20 +83,24 @@ class EngineConfig:
         return resolve_dtype(self.dtype)
 
     def validate(self) -> None:
-        # reference engine/config.py:61-75
-        if self.max_num_seqs < 1:
-            raise ValueError("max_num_seqs must be at least 1")
-        if self.max_num_batched_tokens < self.max_prefill_chunk_size:
-            raise ValueError("max_num_batched_tokens must be at least max_prefill_chunk_size")
-        if self.max_num_batched_tokens < self.max_num_seqs:
-            raise ValueError("max_num_batched_tokens must leave room for one token per running sequence")
-        if not 0.0 < self.gpu_memory_utilization <= 1.0:
-            raise ValueError("gpu_memory_utilization must be in (0, 1]")
-        if self.block_size <= 0 or (self.block_size & (self.block_size - 1)) != 0:
-            raise ValueError("block_size must be a power of two")
-        if self.max_prefill_chunk_size < 1 or self.max_model_len < 2:
-            raise ValueError("max_prefill_chunk_size must be at least 1 and max_model_len at least 2")
-        if (self.kv_cache_dtype or "auto").lower() not in ("auto", str(self.dtype).lower()):
-            raise ValueError(f"kv_cache_dtype={self.kv_cache_dtype!r}: the cache holds the run dtype; quantized caches are not built")
-        if self.quantization not in (None, "", "none"):
-            raise ValueError(f"quantization={self.quantization!r}: weight quantization is not built")
+        """Refuses option values that cannot work together (the limits are the reference's, ``engine/config.py:61-75``)."""
+        def power_of_two(n: int) -> bool:
+            return n > 0 and n & (n - 1) == 0
+
+        checks = (
+            (self.max_num_seqs >= 1, f"max_num_seqs={self.max_num_seqs}: at least one request runs at a time"),
+            (self.max_prefill_chunk_size >= 1, f"max_prefill_chunk_size={self.max_prefill_chunk_size}: a portion has at least one token"),
+            (self.max_model_len >= 2, f"max_model_len={self.max_model_len}: a prompt token and a generated one need two positions"),
+            (self.max_num_batched_tokens >= self.max_prefill_chunk_size,
+             f"max_num_batched_tokens={self.max_num_batched_tokens} is less than one portion of a prompt (max_prefill_chunk_size={self.max_prefill_chunk_size})"),
+            (self.max_num_batched_tokens >= self.max_num_seqs,
+             f"max_num_batched_tokens={self.max_num_batched_tokens} is less than a decode step of max_num_seqs={self.max_num_seqs} requests"),
+            (0.0 < self.gpu_memory_utilization <= 1.0, f"gpu_memory_utilization={self.gpu_memory_utilization}: a share of the memory, above 0 and at most 1"),
+            (power_of_two(self.block_size), f"block_size={self.block_size}: pages hold a power of two of tokens"),
+            ((self.kv_cache_dtype or "auto").lower() in ("auto", str(self.dtype).lower()),
+             f"kv_cache_dtype={self.kv_cache_dtype!r}: the cache holds the run dtype; quantized caches are not built"),
+            (self.quantization in (None, "", "none"), f"quantization={self.quantization!r}: weight quantization is not built"),
+        )
+        failed = [message for ok, message in checks if not ok]
+        if failed:
+            raise ValueError("engine options: " + "; ".join(failed))

@@ -438,7 +438,8 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_kernel(const float* __r
       const unsigned long long my_total = add_to_tables(row, vocab, 0, quads, o, mx, level, prefix, counts, masses);
       if (level == 0 && o.use_mass) atomicAdd(&total_mass, my_total);
       __syncthreads();
-      if (level == 0) mass_limit = (unsigned long long)((double)o.top_p * (double)total_mass);
+      // (at least 1: the largest token is kept however small top_p is)
+      if (level == 0) mass_limit = max(1ull, (unsigned long long)((double)o.top_p * (double)total_mass));
       const int digit = select_digit(counts, masses, bins, o.top_k, o.use_mass, mass_limit, above, &found_digit, &found_above);
       prefix |= (uint32_t)digit << level_shift(level);
       __syncthreads();  // the tables are free again
@@ -544,7 +545,7 @@ __device__ __forceinline__ uint32_t finished_digit(const ChunkedScratch& s, int 
   const size_t base = ((size_t)r * 3 + level) * SELECT_BINS;
   for (int b = threadIdx.x; b < bins; b += blockDim.x) { counts[b] = s.counts[base + b]; masses[b] = s.masses[base + b]; }
   __syncthreads();
-  const unsigned long long mass_limit = (unsigned long long)((double)o.top_p * (double)s.search[r].total_mass);
+  const unsigned long long mass_limit = max(1ull, (unsigned long long)((double)o.top_p * (double)s.search[r].total_mass));
   const int digit = select_digit(counts, masses, bins, o.top_k, o.use_mass, mass_limit, above, found_digit, found_above);
   __syncthreads();  // the tables are free again
   return prefix_before | ((uint32_t)digit << level_shift(level));

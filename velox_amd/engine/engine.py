@@ -108,7 +108,7 @@ class Engine:
         config.validate()
         model_config = load_config(config.model)
         eos = read_generation_eos(config.model)
-        return cls._assemble(config, model_config, ops, eos, lambda model, dtype, device: bind_from_checkpoint(model, config.model, dtype, device))
+        return cls._assemble(config, model_config, ops, eos, lambda model, dtype, device: bind_from_checkpoint(model, config.model, dtype, device, ignore_unexpected=config.ignore_unexpected_weights))
 
     @classmethod
     def from_random(cls, model_config_dict: dict, seed: int, config: Optional[EngineConfig] = None, ops=None, generator_device: str = "cpu", **overrides) -> "Engine":

@@ -144,15 +144,21 @@ class Scheduler:
 
     def _drop_finished(self) -> None:
         """Requests that ended since the last decision leave ``running``; their pages and slot go back only now, so a step
-        that was still in flight when they ended wrote into pages that were still theirs."""
+        that was still in flight when they ended wrote into pages that were still theirs.  A request may also end while it
+        WAITS: it was preempted with a token still in flight, and that token turned out to be its last.  It holds nothing,
+        and must not be admitted again."""
         ended = [r for r in self.running if r.finished]
-        if not ended:
+        ended_waiting = [r for r in self.waiting if r.finished]
+        if not ended and not ended_waiting:
             return
-        for request in ended:
+        for request in ended + ended_waiting:
             self._give_back(request)
             self.requests.pop(request.request_id, None)
-        self.num_finished += len(ended)
-        self.running = [r for r in self.running if not r.finished]
+        self.num_finished += len(ended) + len(ended_waiting)
+        if ended:
+            self.running = [r for r in self.running if not r.finished]
+        if ended_waiting:
+            self.waiting = deque(r for r in self.waiting if not r.finished)
 
     def _preempt(self, victim: Request, plan: Optional[StepPlan] = None) -> None:
         """Recompute preemption: everything the victim holds goes back, it waits at the front of the queue and is later

@@ -13,6 +13,7 @@ a library has no call for.  bfloat16 x bfloat16 products go to the library behin
 from __future__ import annotations
 
 import ctypes
+import logging
 import os
 import tempfile
 from typing import Tuple, Dict, Optional
@@ -21,6 +22,8 @@ import torch
 
 from ..parts.base import DeferredNorm, ResidualSink
 from . import build
+
+logger = logging.getLogger(__name__)
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 _P = ctypes.c_void_p
@@ -225,7 +228,17 @@ class HipOps:
         if tunable.get_filename() != results_file:
             tunable.set_filename(results_file)
             if os.path.isfile(results_file) and not tunable.read_file(results_file):
-                os.remove(results_file)  # made with other versions of the libraries: start again
+                # made with other versions of the libraries, or half written: start again.  Only a file of the engine's
+                # own (beside its kernel libraries, or the temporary one) is removed; a caller's file is left alone and
+                # what is found now goes to a new name beside it
+                own = results_file == self.tuning_file() or os.path.dirname(results_file) == tempfile.gettempdir()
+                if own:
+                    os.remove(results_file)
+                else:
+                    fresh = f"{results_file}.{os.getpid()}"
+                    logger.warning("the timings in %s cannot be read by this version of the matrix library; leaving it and writing to %s", results_file, fresh)
+                    results_file = fresh
+                    tunable.set_filename(results_file)
         tunable.set_max_tuning_duration(int(seconds_per_shape * 1000))
         tunable.tuning_enable(True)
         done = 0

@@ -1,7 +1,8 @@
-"""Per-request sampling options, with the reference's names, defaults and checks
-(``engine/utils.py:9-47``)."""
+"""Per-request sampling options.  Names, defaults and the ranges that are accepted are the reference's
+(``engine/utils.py:9-47``): they are the schema callers write against."""
 from __future__ import annotations
 
+import math
 from dataclasses import dataclass, field
 from typing import List, Optional
 
@@ -21,18 +22,21 @@ class SamplingParams:
     stop_token_ids: List[int] = field(default_factory=list)
 
     def __post_init__(self) -> None:
+        problems = []
         if self.n != 1:
-            raise ValueError("only n=1 is supported")
-        if self.temperature < 0.0:
-            raise ValueError("temperature must be non-negative")
+            problems.append(f"n={self.n}: one sequence is generated per request")
+        if not self.temperature >= 0.0 or math.isinf(self.temperature):
+            problems.append(f"temperature={self.temperature}: a finite number >= 0 (0 = greedy)")
         if not 0.0 < self.top_p <= 1.0:
-            raise ValueError("top_p must be in (0, 1]")
+            problems.append(f"top_p={self.top_p}: a share of the probability mass, above 0 and at most 1")
         if self.top_k < 0:
-            raise ValueError("top_k must be non-negative (0 disables the filter)")
-        if self.repetition_penalty <= 0.0:
-            raise ValueError("repetition_penalty must be positive")
+            problems.append(f"top_k={self.top_k}: a count of tokens to keep, 0 = no limit")
+        if not self.repetition_penalty > 0.0:
+            problems.append(f"repetition_penalty={self.repetition_penalty}: a factor above 0 (1 = none)")
         if self.max_tokens < 1:
-            raise ValueError("max_tokens must be at least 1")
+            problems.append(f"max_tokens={self.max_tokens}: a request generates at least one token")
+        if problems:
+            raise ValueError("sampling options out of range: " + "; ".join(problems))
 
     @property
     def is_greedy(self) -> bool:
@@ -40,4 +44,4 @@ class SamplingParams:
 
     @property
     def has_penalties(self) -> bool:
-        return self.repetition_penalty != 1.0 or self.presence_penalty != 0.0 or self.frequency_penalty != 0.0
+        return (self.repetition_penalty, self.presence_penalty, self.frequency_penalty) != (1.0, 0.0, 0.0)

@@ -42,22 +42,25 @@ class WeightsError(RuntimeError):
             lines.append(f"  missing tensors ({len(missing)}): " + ", ".join(missing))
         if unexpected:
             lines.append(f"  unexpected tensors ({len(unexpected)}): " + ", ".join(unexpected))
+            lines.append("    (tensors the model has no place for are refused, so that a misnamed weight cannot go unnoticed; an export that "
+                         "carries buffers of no use loads with ignore_unexpected_weights=True, which prints their number and goes on)")
         if wrong_shape:
             lines.append(f"  wrong shapes ({len(wrong_shape)}): " + "; ".join(wrong_shape))
         super().__init__("\n".join(lines))
 
 
 def list_weight_files(model_dir: str) -> List[str]:
-    index_path = os.path.join(model_dir, _INDEX_FILE)
-    if os.path.exists(index_path):
-        with open(index_path, "r", encoding="utf-8") as handle:
-            index = json.load(handle)
-        names = sorted(set(index["weight_map"].values()))
-        return [os.path.join(model_dir, name) for name in names]
-    single_path = os.path.join(model_dir, _SINGLE_FILE)
-    if os.path.exists(single_path):
-        return [single_path]
-    raise FileNotFoundError(f"no safetensors weights found in {model_dir}")
+    """The folder's safetensors files: the shards its index names, else the single file (reference
+    ``src/weight_loader.py:31-47``)."""
+    indexed = os.path.join(model_dir, _INDEX_FILE)
+    if os.path.isfile(indexed):
+        with open(indexed, "r", encoding="utf-8") as handle:
+            shards = set(json.load(handle)["weight_map"].values())
+        return [os.path.join(model_dir, shard) for shard in sorted(shards)]
+    whole = os.path.join(model_dir, _SINGLE_FILE)
+    if not os.path.isfile(whole):
+        raise FileNotFoundError(f"{model_dir} holds neither {_SINGLE_FILE} nor {_INDEX_FILE}")
+    return [whole]
 
 
 class _Checkpoint:
@@ -107,10 +110,46 @@ def expected_names(parts: List[Part]) -> List[Tuple[Part, str, Param, List[str]]
     return rows
 
 
+def named_tensors(model):
+    """The binder's inverse: every tensor a bound model holds, under its checkpoint name (fused rows cut apart again,
+    a shared tensor named once), in the dtype it is held in."""
+    seen = set()
+    for part, attr, param, names in expected_names(model.all_parts()):
+        held = getattr(part, attr)
+        row = 0
+        for name, shape in zip(names, param.source_shapes):
+            n = shape[0] if len(shape) > 0 else 1
+            piece = held[row:row + n].reshape(shape)
+            row += n
+            if name not in seen and param.alias_of is None:
+                seen.add(name)
+                yield name, piece
+
+
+class TensorSource:
+    """Where a binder takes tensors from, by checkpoint name.  ``names()``: every name it holds; ``shape(name)``;
+    ``tensor(name)``: the tensor, on any device, in the dtype it is stored in.  The binder asks for tensors in the order
+    the model's parts declare them."""
+
+    def names(self):
+        raise NotImplementedError
+
+    def __contains__(self, name: str) -> bool:
+        return name in self.names()
+
+    def shape(self, name: str) -> Tuple[int, ...]:
+        raise NotImplementedError
+
+    def tensor(self, name: str) -> torch.Tensor:
+        raise NotImplementedError
+
+
 @torch.no_grad()
-def bind_from_checkpoint(model, model_dir: str, run_dtype: torch.dtype, device) -> int:
-    """Fills every declared tensor of ``model`` from the folder's safetensors; returns the parameter count."""
-    checkpoint = _Checkpoint(list_weight_files(model_dir))
+def bind(model, source, run_dtype: torch.dtype, device, ignore_unexpected: bool = False) -> int:
+    """Fills every declared tensor of ``model`` from ``source`` (files of a folder, or tensors drawn at random: anything
+    with ``names``, ``shape`` and ``tensor``); returns the parameter count.  The one place where rows are concatenated,
+    a tied tensor is shared and held dtypes are decided."""
+    checkpoint = source
     device = torch.device(device)
     rows = expected_names(model.all_parts())
 
@@ -141,6 +180,10 @@ def bind_from_checkpoint(model, model_dir: str, run_dtype: torch.dtype, device) 
     aliased = {part.prefix + s for part, _, param, names in plan if names is None for s in param.sources}
     tolerated = {n for n in unexpected if n in aliased}
     unexpected = [n for n in unexpected if n not in tolerated]
+    if unexpected and ignore_unexpected and not missing and not wrong:
+        # (as the reference does, src/weight_loader.py:131-136)
+        print(f"[weights] ignoring {len(unexpected)} tensors the model has no place for: {', '.join(unexpected[:8])}{' ...' if len(unexpected) > 8 else ''}")
+        unexpected = []
     if missing or unexpected or wrong:
         raise WeightsError(sorted(missing), unexpected, wrong)
 
@@ -162,6 +205,7 @@ def bind_from_checkpoint(model, model_dir: str, run_dtype: torch.dtype, device) 
             n = piece.shape[0] if piece.dim() > 0 else 1
             target[row:row + n].copy_(piece.to(dtype))
             row += n
+        del pieces
         setattr(part, attr, target)
         if len(names) == 1:
             bound[names[0]] = target
@@ -173,3 +217,8 @@ def bind_from_checkpoint(model, model_dir: str, run_dtype: torch.dtype, device) 
     for part in model.all_parts():
         part.finalize(device, run_dtype)
     return count
+
+
+def bind_from_checkpoint(model, model_dir: str, run_dtype: torch.dtype, device, ignore_unexpected: bool = False) -> int:
+    """``bind`` from the folder's safetensors files."""
+    return bind(model, _Checkpoint(list_weight_files(model_dir)), run_dtype, device, ignore_unexpected=ignore_unexpected)
