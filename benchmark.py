@@ -1,6 +1,7 @@
 #!/usr/bin/env python3
 """End-to-end benchmark of the engine from the command line, in the manner of the reference's
-``benchmark.py`` (its options ``:349-388``, its step loop ``:160-182``, its report ``:232-276``).
+``benchmark.py``: its options (``:349-388``), the quantities it reports and the keys of its JSON
+(``:184-223,232-276``).
 
 The engine is token-in / token-out, so where the reference tokenises hand-written chat prompts
 (``:17-47,149-153``) this program draws seeded random token ids of the workload's lengths.
@@ -34,18 +35,26 @@ WORKLOAD_LENGTHS = {"short": (16, 64), "long": (256, 1024)}
 
 
 def summarise(values: List[float]) -> Dict[str, float]:
-    if not values:
-        return {"n": 0, "mean": 0.0, "p50": 0.0, "p90": 0.0, "p99": 0.0, "max": 0.0}
+    """Count, mean and nearest-rank percentiles of a list of numbers (zeros for an empty list)."""
     ordered = sorted(values)
+    count = len(ordered)
+    out = {"n": count, "mean": statistics.fmean(ordered) if count else 0.0}
+    for name, share in (("p50", 0.5), ("p90", 0.9), ("p99", 0.99), ("max", 1.0)):
+        out[name] = ordered[min(count - 1, int(share * count))] if count else 0.0
+    return out
 
-    def pct(q: float) -> float:
-        return ordered[min(len(ordered) - 1, int(q * len(ordered)))]
 
-    return {"n": len(values), "mean": statistics.fmean(values), "p50": pct(0.5), "p90": pct(0.9), "p99": pct(0.99), "max": ordered[-1]}
+def heading(title: str) -> None:
+    bar = "=" * 78
+    print(f"\n{bar}\n  {title}\n{bar}")
 
 
-def rule(title: str = "") -> None:
-    print("\n" + "=" * 78 + f"\n  {title}\n" + "=" * 78 if title else "-" * 78)
+def print_table(columns, rows, indent: str = "  ") -> None:
+    """``columns``: (title, width, format) per column, the first left-aligned; ``rows``: one tuple of values per line."""
+    print(indent + "".join(f"{title:<{width}}" if index == 0 else f"{title:>{width}}" for index, (title, width, _) in enumerate(columns)))
+    for row in rows:
+        cells = [format(value, fmt) for value, (_, _, fmt) in zip(row, columns)]
+        print(indent + "".join(f"{cell:<{width}}" if index == 0 else f"{cell:>{width}}" for index, (cell, (_, width, _)) in enumerate(zip(cells, columns))))
 
 
 SHARED_PREFIX_TOKENS = 96  # stands in for the reference's shared system prompt (``benchmark.py:42-47``, about 90 tokens)
@@ -70,77 +79,120 @@ def build_prompts(workload: str, count: int, vocab: int, limit: int, fixed_len: 
     return prompts
 
 
+class Measurement:
+    """Times of one workload, taken where the engine announces them: every request's token and finish listeners note the
+    clock (``Request.subscribe``), so a token counts when the engine hands it over, not when a poll notices it."""
+
+    def __init__(self, requests) -> None:
+        self.begin = time.perf_counter()
+        self.token_times: Dict[str, List[float]] = {r.request_id: [] for r in requests}
+        self.finished_at: Dict[str, float] = {}
+        self.peak_running = self.peak_pages = 0
+        for request in requests:
+            request.subscribe(on_token=self._token, on_finish=self._finish)
+
+    def _token(self, request, _token_id) -> None:
+        self.token_times[request.request_id].append(time.perf_counter())
+
+    def _finish(self, request, _reason) -> None:
+        self.finished_at[request.request_id] = time.perf_counter()
+
+    def after_step(self, engine) -> None:
+        self.peak_running = max(self.peak_running, engine.scheduler.num_running)
+        self.peak_pages = max(self.peak_pages, engine.cache.num_used_pages())
+
+    def first_token_delays(self) -> List[float]:
+        return [times[0] - self.begin for times in self.token_times.values() if times]
+
+    def gaps_between_tokens_ms(self) -> List[float]:
+        return [(later - earlier) * 1000 for times in self.token_times.values() for earlier, later in zip(times, times[1:])]
+
+    def per_request(self, requests) -> List[Dict]:
+        """One record per request, as the reference's JSON holds them (``benchmark.py:208-218``)."""
+        records = []
+        for request in requests:
+            times = self.token_times[request.request_id]
+            done = self.finished_at.get(request.request_id)
+            records.append({
+                "id": request.request_id, "prompt_tokens": request.num_prompt_tokens, "generated_tokens": len(request.output_token_ids),
+                "ttft": times[0] - self.begin if times else None, "end_to_end": done - self.begin if done is not None else None,
+                "cached_prompt_tokens": request.num_cached_tokens,  # (of a preempted request: at its last admission)
+            })
+        return records
+
+
 def run_workload(engine, prompts, sampling, label: str) -> Dict:
+    """Queues every prompt at once and steps the engine until nothing is left.  The result's keys are the reference's
+    (``benchmark.py:184-223``): scripts that read its JSON read this one."""
     import torch
 
     from velox_amd import Request
 
-    requests = [Request(f"{label}-{i}", p, sampling(i)) for i, p in enumerate(prompts)]
-    token_times: Dict[str, List[float]] = {r.request_id: [] for r in requests}
-    seen = {r.request_id: 0 for r in requests}
-    start = time.perf_counter()
+    requests = [Request(f"{label}-{index}", prompt, sampling(index)) for index, prompt in enumerate(prompts)]
+    measured = Measurement(requests)
     for request in requests:
         engine.add_request(request)
-    log = []
     while engine.has_work():
         engine.step()
-        now = time.perf_counter()
-        log.append((engine.scheduler.num_running, engine.scheduler.num_waiting, engine.cache.num_used_pages()))
-        for request in requests:
-            produced = len(request.output_token_ids)
-            if produced > seen[request.request_id]:
-                token_times[request.request_id].extend([now] * (produced - seen[request.request_id]))
-                seen[request.request_id] = produced
+        measured.after_step(engine)
     torch.cuda.synchronize()
-    wall = time.perf_counter() - start
-    ttft = [times[0] - start for times in token_times.values() if times]
-    itl = [(b - a) * 1000 for times in token_times.values() for a, b in zip(times, times[1:])]
-    generated = sum(len(r.output_token_ids) for r in requests)
-    prompt_tokens = sum(len(p) for p in prompts)
-    cached_tokens = sum(r.num_cached_tokens for r in requests)  # (of a preempted request: at its last admission)
+    wall = time.perf_counter() - measured.begin
+    records = measured.per_request(requests)
+    prompt_tokens = sum(r["prompt_tokens"] for r in records)
+    generated = sum(r["generated_tokens"] for r in records)
+    per_second = (lambda tokens: tokens / wall) if wall > 0 else (lambda tokens: 0.0)
     return {
-        "label": label, "wall_seconds": wall, "num_requests": len(requests), "prompt_tokens": prompt_tokens,
-        "generated_tokens": generated, "decode_throughput": generated / wall if wall else 0.0,
-        "total_throughput": (prompt_tokens + generated) / wall if wall else 0.0,
-        "ttft": summarise(ttft), "itl_ms": summarise(itl), "steps": engine.num_steps,
-        "preemptions": engine.scheduler.num_preemptions, "cached_prompt_tokens": cached_tokens,
-        "max_running": max((entry[0] for entry in log), default=0), "max_blocks_used": max((entry[2] for entry in log), default=0),
+        "label": label, "wall_seconds": wall, "num_requests": len(requests),
+        "prompt_tokens": prompt_tokens, "generated_tokens": generated, "cached_prompt_tokens": sum(r["cached_prompt_tokens"] for r in records),
+        "decode_throughput": per_second(generated), "total_throughput": per_second(prompt_tokens + generated),
+        "ttft": summarise(measured.first_token_delays()), "itl_ms": summarise(measured.gaps_between_tokens_ms()),
+        "steps": engine.num_steps, "preemptions": engine.scheduler.num_preemptions,
+        "max_running": measured.peak_running, "max_blocks_used": measured.peak_pages,
+        "requests": records,
         "outputs": {r.request_id: r.output_token_ids for r in requests},
     }
+
+
+_PERCENTILES = (("mean", "mean"), ("p50", "p50"), ("p90", "p90"), ("p99", "p99"), ("max", "max"))
 
 
 def report(result: Dict, engine, show_outputs: bool) -> None:
     import torch
 
-    rule(f"RESULTS: {result['label']}")
-    print(f"  Requests              : {result['num_requests']}")
-    print(f"  Wall time             : {result['wall_seconds']:.3f} s")
-    print(f"  Engine steps          : {result['steps']}")
-    print(f"  Prompt tokens         : {result['prompt_tokens']}")
-    print(f"  Generated tokens      : {result['generated_tokens']}")
-    print(f"  Decode throughput     : {result['decode_throughput']:.2f} tok/s")
-    print(f"  End-to-end throughput : {result['total_throughput']:.2f} tok/s")
-    print(f"  Peak running requests : {result['max_running']}")
-    print(f"  Peak KV blocks in use : {result['max_blocks_used']}")
-    print(f"  Preemptions           : {result['preemptions']}")
-    share = 100.0 * result['cached_prompt_tokens'] / max(1, result['prompt_tokens'])
-    print(f"  Prompt tokens cached  : {result['cached_prompt_tokens']} ({share:.1f}%, prefix caching {'on' if engine.cache.prefix is not None else 'off'})")
-    ttft, itl = result["ttft"], result["itl_ms"]
-    print(f"\n  TTFT (s)   mean={ttft['mean']:.3f}  p50={ttft['p50']:.3f}  p90={ttft['p90']:.3f}  p99={ttft['p99']:.3f}  max={ttft['max']:.3f}")
-    print(f"  ITL (ms)   mean={itl['mean']:.2f}  p50={itl['p50']:.2f}  p90={itl['p90']:.2f}  p99={itl['p99']:.2f}  max={itl['max']:.2f}")
-    rule()
+    heading(f"RESULTS: {result['label']}")
+    cached_share = result["cached_prompt_tokens"] / max(1, result["prompt_tokens"])
+    facts = [
+        ("Requests", f"{result['num_requests']}"),
+        ("Wall time", f"{result['wall_seconds']:.3f} s"),
+        ("Engine steps", f"{result['steps']}"),
+        ("Prompt tokens", f"{result['prompt_tokens']}"),
+        ("Generated tokens", f"{result['generated_tokens']}"),
+        ("Decode throughput", f"{result['decode_throughput']:.2f} tok/s"),
+        ("End-to-end throughput", f"{result['total_throughput']:.2f} tok/s"),
+        ("Peak running requests", f"{result['max_running']}"),
+        ("Peak KV blocks in use", f"{result['max_blocks_used']}"),
+        ("Preemptions", f"{result['preemptions']}"),
+        ("Prompt tokens cached", f"{result['cached_prompt_tokens']} ({cached_share:.1%}, prefix caching {'on' if engine.cache.prefix is not None else 'off'})"),
+    ]
+    for name, value in facts:
+        print(f"  {name:<22}: {value}")
+    print()
+    for title, key, digits in (("TTFT (s)", "ttft", 3), ("ITL (ms)", "itl_ms", 2)):
+        print(f"  {title:<10} " + "  ".join(f"{name}={result[key][field]:.{digits}f}" for name, field in _PERCENTILES))
+    print("-" * 78)
     print("  Per-step breakdown (ms)")
-    print(f"  {'stage':<20}{'n':>7}{'mean':>10}{'p50':>10}{'p90':>10}{'p99':>10}{'total(s)':>11}")
+    stage_rows = []
     for stage, values in engine.stats.items():
-        s = summarise(values)
-        print(f"  {stage:<20}{s['n']:>7}{s['mean']:>10.3f}{s['p50']:>10.3f}{s['p90']:>10.3f}{s['p99']:>10.3f}{sum(values) / 1000:>11.3f}")
-    gpu_ms = sum(engine.stats.get("gpu_ms", []))
-    busy = gpu_ms / 1000 / result["wall_seconds"] if result["wall_seconds"] else 0.0
-    print(f"\n  GPU busy      : {gpu_ms / 1000:.3f} s  ({busy:.1%} of wall time)")
+        numbers = summarise(values)
+        stage_rows.append((stage, numbers["n"], numbers["mean"], numbers["p50"], numbers["p90"], numbers["p99"], sum(values) / 1000))
+    print_table((("stage", 20, ""), ("n", 7, "d"), ("mean", 10, ".3f"), ("p50", 10, ".3f"), ("p90", 10, ".3f"), ("p99", 10, ".3f"), ("total(s)", 11, ".3f")), stage_rows)
+    device_seconds = sum(engine.stats.get("gpu_ms", [])) / 1000
+    busy_share = device_seconds / result["wall_seconds"] if result["wall_seconds"] else 0.0
+    print(f"\n  GPU busy      : {device_seconds:.3f} s  ({busy_share:.1%} of wall time)")
     print(f"  HIP graphs    : {'on' if engine.runner.uses_graphs else 'off'}")
     print(f"  Peak GPU alloc: {torch.cuda.max_memory_allocated() / 1e9:.3f} GB")
     if show_outputs:
-        rule("SAMPLE OUTPUTS (token ids)")
+        heading("SAMPLE OUTPUTS (token ids)")
         for request_id, tokens in list(result["outputs"].items())[:4]:
             print(f"  [{request_id}] {tokens[:32]}")
 
@@ -228,7 +280,7 @@ def main(argv=None) -> int:
             raise SystemExit("--max-tokens leaves no room for a prompt under --max-model-len")
         length_range = tuple(int(v) for v in args.prompt_len_range.split(",")) if args.prompt_len_range else None
         prompts = build_prompts(args.workload, args.num_requests, vocab, limit, args.prompt_len, args.seed, args.shared_system_prompt, length_range)
-        rule("ENGINE BENCHMARK")
+        heading("ENGINE BENCHMARK")
         print(f"  Model            : {args.model or args.shape + ' (random weights)'}")
         print(f"  PyTorch / HIP    : {torch.__version__} / {torch.version.hip}")
         print(f"  GPU              : {torch.cuda.get_device_name(0)}")
@@ -239,22 +291,22 @@ def main(argv=None) -> int:
             torch.cuda.reset_peak_memory_stats()
             result = run_workload(engine, prompts, sampling, f"engine(max_num_seqs={max_num_seqs})" + (f" round={round_index + 1}" if args.rounds > 1 else ""))
             result["kv_blocks"] = engine.cache.num_total_pages
+            result["max_num_seqs"] = max_num_seqs
             report(result, engine, args.show_outputs and round_index == 0)
             results.append(result)
         del engine
         torch.cuda.empty_cache()
     if len(sizes) > 1:
-        rule("BATCH SIZE SWEEP")
-        print(f"  {'max_num_seqs':>14}{'kv_blocks':>11}{'peak_used':>11}{'wall(s)':>10}{'tok/s':>10}{'TTFT p50':>11}{'ITL p50':>10}{'preempt':>9}")
-        for size, result in zip(sizes, results):
-            print(f"  {size:>14}{result['kv_blocks']:>11}{result['max_blocks_used']:>11}{result['wall_seconds']:>10.2f}"
-                  f"{result['decode_throughput']:>10.2f}{result['ttft']['p50']:>11.3f}{result['itl_ms']['p50']:>10.2f}{result['preemptions']:>9}")
+        heading("BATCH SIZE SWEEP")
+        columns = (("max_num_seqs", 14, "d"), ("kv_blocks", 11, "d"), ("peak_used", 11, "d"), ("wall(s)", 10, ".2f"), ("tok/s", 10, ".2f"),
+                   ("TTFT p50", 11, ".3f"), ("ITL p50", 10, ".2f"), ("preempt", 9, "d"))
+        print_table(columns, [(r["max_num_seqs"], r["kv_blocks"], r["max_blocks_used"], r["wall_seconds"], r["decode_throughput"], r["ttft"]["p50"],
+                               r["itl_ms"]["p50"], r["preemptions"]) for r in results])
     if args.output_json:
-        for result in results:
-            result.pop("outputs", None)
-        os.makedirs(os.path.dirname(os.path.abspath(args.output_json)), exist_ok=True)
+        folder = os.path.dirname(os.path.abspath(args.output_json))
+        os.makedirs(folder, exist_ok=True)
         with open(args.output_json, "w", encoding="utf-8") as handle:
-            json.dump(results, handle, indent=2)
+            json.dump([{key: value for key, value in r.items() if key != "outputs"} for r in results], handle, indent=2)
         print(f"\nWrote {args.output_json}")
     return 0
 

@@ -1,24 +1,25 @@
-import os
+"""Test set-up: the repository root and this folder on the import path; tests marked ``gpu`` are skipped where
+no GPU is visible (the marker itself is registered in pytest.ini)."""
+import pathlib
 import sys
 
 import pytest
 
-ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-if ROOT not in sys.path:
-    sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+HERE = pathlib.Path(__file__).resolve().parent
+for folder in (HERE, HERE.parent):
+    if str(folder) not in sys.path:
+        sys.path.insert(0, str(folder))
+
+_gpu_visible = None
 
 
-def pytest_configure(config):
-    config.addinivalue_line("markers", "gpu: needs an MI355X (run with -m gpu on the GPU box)")
-
-
-def pytest_collection_modifyitems(config, items):
-    import torch
-
-    if torch.cuda.is_available():
+def pytest_runtest_setup(item):
+    global _gpu_visible
+    if item.get_closest_marker("gpu") is None:
         return
-    skip = pytest.mark.skip(reason="no GPU in this process")
-    for item in items:
-        if "gpu" in item.keywords:
-            item.add_marker(skip)
+    if _gpu_visible is None:
+        import torch
+
+        _gpu_visible = torch.cuda.is_available()
+    if not _gpu_visible:
+        pytest.skip("needs a GPU")

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from velox_amd.cache import NULL_PAGE, CacheManager, PoolExhausted, PageAllocator
-from velox_amd.parts.base import PagedNeed, StateNeed
+from velox_amd.parts import PagedNeed, StateNeed, kv_pages
 
 
 def test_allocator_order_and_errors():
@@ -60,9 +60,9 @@ def _manager(needs, pages=9, page=4, seqs=4, max_len=None):
 
 
 def test_growth_and_release():
-    need = PagedNeed(2, 16)
+    need = kv_pages(2, 16)
     m = _manager([need, need, need])
-    assert len(m.groups) == 1 and m.groups[0].keys.shape == (3, 9, 2, 4, 16) and m.groups[0].values.shape == (3, 9, 2, 16, 4)
+    assert len(m.groups) == 1 and m.groups[0].tensors["k"].shape == (3, 9, 2, 4, 16) and m.groups[0].tensors["v"].shape == (3, 9, 2, 16, 4)
     assert m.max_model_len == 32
     s = m.new_sequence()
     assert m.append(s, 0, 5) and s.tables[0] == [1, 2]
@@ -86,8 +86,8 @@ def test_growth_and_release():
 
 
 def test_groups_by_need_and_window_release():
-    full = PagedNeed(2, 16)
-    windowed = PagedNeed(2, 16, window=6)
+    full = kv_pages(2, 16)
+    windowed = kv_pages(2, 16, window=6)
     m = _manager([full, windowed, full, windowed, None], pages=12)
     assert len(m.groups) == 2 and m.entry_group[0] == (0, 0) and m.entry_group[2] == (0, 1) and m.entry_group[3] == (1, 1)
     s = m.new_sequence()
@@ -108,7 +108,7 @@ def test_groups_by_need_and_window_release():
 
 def test_state_slots_are_zeroed_on_take():
     need = StateNeed((("sum", (3,), torch.float32), ("count", (), None)))
-    m = _manager([PagedNeed(1, 16), need], seqs=2)
+    m = _manager([kv_pages(1, 16), need], seqs=2)
     a, b = m.new_sequence(), m.new_sequence()
     assert m.new_sequence() is None and {a.slot, b.slot} == {0, 1}
     view = m.view(1, [None])
@@ -128,7 +128,7 @@ def test_state_slots_are_zeroed_on_take():
 def test_random_orders_of_requests(seed):
     rng = random.Random(seed)
     windowed = seed % 2 == 1
-    needs = [PagedNeed(1, 16), PagedNeed(1, 16, window=9) if windowed else PagedNeed(1, 16)]
+    needs = [kv_pages(1, 16), kv_pages(1, 16, window=9) if windowed else kv_pages(1, 16)]
     m = _manager(needs, pages=14, page=4, seqs=5)
     live = {}
     for step in range(600):
@@ -173,5 +173,5 @@ def test_pool_size_from_free_memory():
         pages_that_fit(per_page, 1 << 20, 0.5, 1 << 20)
     with pytest.raises(RuntimeError, match="even one cache page"):
         pages_that_fit(per_page, per_page + 10, 1.0, 0)
-    m = CacheManager([PagedNeed(4, 128)] * 28, 16, 2, 4, torch.bfloat16, "cpu", allocate_tensors=False)
+    m = CacheManager([kv_pages(4, 128)] * 28, 16, 2, 4, torch.bfloat16, "cpu", allocate_tensors=False)
     assert m.bytes_per_page() == per_page

@@ -52,6 +52,34 @@ def test_mixed_batch_with_page_reuse(tmp_path):
     assert h.cache.num_used_pages() == 0
 
 
+def test_a_step_padded_up_to_a_timed_number_of_rows_keeps_its_logits(tmp_path):
+    """A step of portions a little short of a row count the matrix library was timed for gets rows of a sequence on the
+    null page: with every slot but one decoding beside the portions (the padding is then one sequence more than
+    ``max_num_seqs``), the logits are those of the same step unpadded, and the null page is all the padding wrote to."""
+    name = "B"
+    folder = make_folder(tmp_path, name)
+    config, weights = read_model_folder(folder)
+    prompts = {rid: random_tokens(config["vocab_size"], n, seed=50 + i) for i, (rid, n) in enumerate([("a", 12), ("b", 9), ("c", 15), ("d", 40)])}
+
+    def run(tuned):
+        h = Harness(folder, TorchOps(), torch.float32, "cpu", PAGE_SIZE[name], num_pages=32, max_num_seqs=4, max_num_tokens=64)
+        h.runner.tuned_row_counts = tuned
+        for rid in "abc":  # three of the four slots decode
+            h.feed([(rid, prompts[rid][:-1], [])])
+        batch = [(rid, prompts[rid][-1:], [0]) for rid in "abc"] + [("d", prompts["d"], [0, 39])]
+        out = h.feed(batch)
+        return h, out
+
+    plain, want = run([])
+    padded, got = run([48])  # 43 rows -> 48: five rows more, within the 12% that a step may grow by
+    assert padded.runner.num_padded_steps == 1 and plain.runner.num_padded_steps == 0
+    torch.testing.assert_close(got, want, rtol=0, atol=0)
+    torch.testing.assert_close(got[-1], qwen2_logits(config, weights, prompts["d"])[-1], rtol=1e-4, atol=1e-5)
+    for mine, theirs in zip(padded.cache.groups, plain.cache.groups):
+        for name in mine.tensors:
+            assert torch.equal(mine.tensors[name][:, 1:], theirs.tensors[name][:, 1:])  # everything but the null page
+
+
 def test_a_fixed_workspace_refuses_to_replace_a_buffer():
     import pytest
     import torch

@@ -62,7 +62,8 @@ def test_the_cache_holds_the_first_layers_rotated_keys_and_values(tmp_path, ops,
     p = "model.layers.0.self_attn."
     keys = apply_rope((x @ weights[p + "k_proj.weight"].T + weights[p + "k_proj.bias"]).view(-1, nkv, d), cos, sin, torch.arange(len(tokens)))
     values = (x @ weights[p + "v_proj.weight"].T + weights[p + "v_proj.bias"]).view(-1, nkv, d)
-    got_keys, got_values = h.cache.gather_sequence(0, h.live["a"][0], len(tokens))
+    held = h.cache.gather_sequence(0, h.live["a"][0], len(tokens))
+    got_keys, got_values = held["k"], held["v"]  # [tokens, kv_heads, head_dim] both: the token dimension comes first
     torch.testing.assert_close(got_keys.float().cpu(), keys, rtol=2e-5, atol=2e-6)
     torch.testing.assert_close(got_values.float().cpu(), values, rtol=2e-5, atol=2e-6)
     assert len(set(h.live["a"][0].tables[0]) & set(h.live["b"][0].tables[0])) == 0

@@ -109,7 +109,7 @@ def test_captured_steps_behind_few_keys_and_behind_many(tmp_path):
     """With a long context allowed, a bucket has two captures: one whose attention splits the keys as the longest context
     needs, one for steps whose sequences all hold few keys (one workgroup per sequence and KV head).  A request that grows
     past the bound moves from the one to the other; tokens as without graphs (float32: bit for bit)."""
-    from velox_amd.engine.runner import SHORT_CONTEXT_KEYS
+    from velox_amd.parts.attention import SHORT_CONTEXT_KEYS
 
     folder = make_folder(tmp_path, "B", "float32")
     config, _ = read_model_folder(folder)
@@ -118,7 +118,7 @@ def test_captured_steps_behind_few_keys_and_behind_many(tmp_path):
     options = dict(max_model_len=1024, max_num_batched_tokens=512, max_prefill_chunk_size=256, num_gpu_blocks=400)
     eager = engine_for(folder, "B", "float32", **options).generate(greedy(prompts, 30))
     engine = engine_for(folder, "B", "float32", enable_cuda_graphs=True, **options)
-    assert sorted(engine.runner._short_graphs) == [1, 2, 4]
+    assert sorted(engine.runner._bounded_graphs) == [1, 2, 4] and all([b for b, _ in v] == [SHORT_CONTEXT_KEYS] for v in engine.runner._bounded_graphs.values())
     graphed = engine.generate(greedy(prompts, 30))
     assert [r.output_token_ids for r in graphed] == [r.output_token_ids for r in eager]
     assert 10 <= engine.runner.num_short_graph_replays <= 20 and engine.runner.num_graph_replays >= 29
@@ -501,3 +501,7 @@ def test_command_line(tmp_path):
     result = json.loads(out.read_text())[0]
     assert result["num_requests"] == 5 and result["generated_tokens"] == 30 and result["prompt_tokens"] == 55
     assert "Decode throughput" in process.stdout and "TTFT" in process.stdout
+    records = result["requests"]  # one per request, as in the reference's JSON
+    assert len(records) == 5 and all(r["prompt_tokens"] == 11 and r["generated_tokens"] == 6 for r in records)
+    assert all(0 < r["ttft"] <= r["end_to_end"] <= result["wall_seconds"] for r in records) and "outputs" not in result
+    assert sorted(records[0]) == ["cached_prompt_tokens", "end_to_end", "generated_tokens", "id", "prompt_tokens", "ttft"]

@@ -660,3 +660,154 @@ def test_stateful_toy_architecture_through_the_engine_with_preemption(tmp_path, 
         assert (engine.scheduler.num_preemptions > 0) == expect_preemption
         assert [r.output_token_ids for r in requests] == want
         assert engine.cache.num_used_pages() == 0 and engine.cache.state.num_free == 4
+
+
+# ----------------------------------------------------------------------------------------------------
+# a fourth toy architecture: a mixer that keeps ONE latent vector per token in pages (no keys and values, no heads) and
+# attends over the latents themselves, beside an ordinary attention layer.  Its need names its own page tensor; the
+# cache manager, the step function and replay learn of it from that need alone.
+# ----------------------------------------------------------------------------------------------------
+class LatentMixer(Mixer):
+    """c_t = W_c x_t is written to the request's pages; y_t = W_o sum_j softmax_j(q_t . c_j / sqrt(r)) c_j over j <= t,
+    with q_t = W_q x_t: keys and values are one and the same cached vector of ``rank`` numbers."""
+
+    graph_safe = False  # forward reads the step's lengths on the host
+
+    def __init__(self, prefix: str, hidden_size: int, rank: int) -> None:
+        super().__init__(prefix)
+        self.hidden_size, self.rank = hidden_size, rank
+        self.w_c = self.w_q = self.w_o = None
+
+    def params(self):
+        h, r = self.hidden_size, self.rank
+        return {"w_c": single("compress.weight", (r, h)), "w_q": single("query.weight", (r, h)), "w_o": single("expand.weight", (h, r))}
+
+    def cache_need(self):
+        from velox_amd.parts import PAGE, PagedNeed
+
+        return PagedNeed((("latent", (PAGE, self.rank), torch.float32),))
+
+    def forward(self, x, ctx, cache, owns_cache=True):
+        latents = cache.tensors["latent"]  # [pages, page size, rank]
+        meta = cache.batch
+        c = x.float() @ self.w_c.float().T
+        q = x.float() @ self.w_q.float().T
+        if owns_cache:
+            latents.view(-1, self.rank)[meta.slot_mapping.long()] = c
+        out = torch.empty((x.shape[0], self.hidden_size), dtype=torch.float32, device=x.device)
+        at = 0
+        for b, n in enumerate(ctx.q_lens):
+            held = int(meta.kv_lens[b])
+            pages = meta.block_tables[b, : (held + cache.block_size - 1) // cache.block_size].long()
+            past = latents[pages].reshape(-1, self.rank)[:held]
+            scores = q[at:at + n] @ past.T / math.sqrt(self.rank)
+            seen = torch.arange(held, device=x.device)[None, :] <= ctx.positions[at:at + n, None]
+            weights = torch.softmax(scores.masked_fill(~seen, float("-inf")), dim=-1)
+            out[at:at + n] = (weights @ past) @ self.w_o.float().T
+            at += n
+        return out.to(x.dtype)
+
+
+def latent_spec(config, max_position=None) -> ModelSpec:
+    raw = config.raw
+    h = raw["hidden_size"]
+    norm = PartSpec.of("rmsnorm", hidden_size=h, eps=raw["eps"])
+    ff = PartSpec.of("gated_mlp", hidden_size=h, intermediate_size=raw["inter"])
+    layers = [
+        LayerSpec("layers.0.", PartSpec.of("toy_latent", hidden_size=h, rank=raw["rank"]), ff, norm, norm, **dict(HF_NAMES, mixer_prefix="mixer.")),
+        LayerSpec("layers.1.", PartSpec.of("attention", hidden_size=h, num_heads=4, num_kv_heads=2, head_dim=16, qkv_bias=True), ff, norm, norm, position="rope", **HF_NAMES),
+        LayerSpec("layers.2.", PartSpec.of("toy_latent", hidden_size=h, rank=raw["rank"]), ff, norm, norm, **dict(HF_NAMES, mixer_prefix="mixer.")),
+    ]
+    return ModelSpec(vocab_size=raw["vocab_size"], hidden_size=h, max_position=max_position or 256, layers=layers, schedule=[ScheduleEntry(i) for i in range(3)],
+                     final_norm=norm, positions={"rope": PartSpec.of("rotary", rotary_dim=16, theta=10000.0, max_position=max_position or 256)}, tie_head=True, **HF_ENDS)
+
+
+def plain_latent(tensors, raw, tokens):
+    eps, n, r = raw["eps"], len(tokens), raw["rank"]
+    cos, sin = rope_tables(16, 10000.0, n)
+    x = tensors["model.embed_tokens.weight"][torch.tensor(tokens)]
+    causal = torch.arange(n)[None, :] <= torch.arange(n)[:, None]
+    for layer in range(3):
+        p = f"layers.{layer}."
+        a = rms_norm(x, tensors[p + "input_layernorm.weight"], eps)
+        if layer == 1:
+            q = apply_rope((a @ tensors[p + "self_attn.q_proj.weight"].T + tensors[p + "self_attn.q_proj.bias"]).reshape(n, 4, 16), cos, sin, torch.arange(n))
+            k = apply_rope((a @ tensors[p + "self_attn.k_proj.weight"].T + tensors[p + "self_attn.k_proj.bias"]).reshape(n, 2, 16), cos, sin, torch.arange(n))
+            v = (a @ tensors[p + "self_attn.v_proj.weight"].T + tensors[p + "self_attn.v_proj.bias"]).reshape(n, 2, 16)
+            mixed = causal_attention(q, k, v, 0.25).reshape(n, 64) @ tensors[p + "self_attn.o_proj.weight"].T
+        else:
+            c = a @ tensors[p + "mixer.compress.weight"].T
+            scores = (a @ tensors[p + "mixer.query.weight"].T) @ c.T / math.sqrt(r)
+            mixed = (torch.softmax(scores.masked_fill(~causal, float("-inf")), dim=-1) @ c) @ tensors[p + "mixer.expand.weight"].T
+        x = x + mixed
+        x = x + gated_mlp(rms_norm(x, tensors[p + "post_attention_layernorm.weight"], eps), tensors[p + "mlp.gate_proj.weight"],
+                          tensors[p + "mlp.up_proj.weight"], tensors[p + "mlp.down_proj.weight"])
+    return rms_norm(x, tensors["model.norm.weight"], eps) @ tensors["model.embed_tokens.weight"].T
+
+
+def test_toy_architecture_with_one_latent_tensor_per_page_stepped_and_replayed(tmp_path, ops):
+    """A paged mixer that is no attention: its need names one float32 tensor ``(PAGE, rank)``.  The cache manager gives it
+    a pool of its own beside the attention layer's (two groups, two block tables per request), the step function runs
+    it in portions and single tokens with pages used again, and the replay program drives the same model from a folder."""
+    import numpy as np
+
+    from velox_amd.engine.replay import Replayer
+    from velox_amd.weights import write_random_model
+
+    register_part("mixer", "toy_latent", LatentMixer)
+    register_architecture("LatentToyForCausalLM", lambda raw: ModelConfig(architecture_name(raw), dict(raw)), latent_spec)
+    raw = {"architectures": ["LatentToyForCausalLM"], "hidden_size": 64, "inter": 96, "vocab_size": 83, "eps": 1e-5, "rank": 12}
+    model = build_model(config_from_dict(raw), torch.float32, "cuda")
+    needs = model.cache_needs()
+    assert [n.tensors[0][0] for n in needs] == ["latent", "k", "latent"]
+    bind_random(model, 6, torch.float32, "cuda", storage_dtype=torch.float32)
+    tensors = dict(random_tensors(model, 6))
+    for name in tensors:  # sharper scores, so that a latent read from a wrong page shows
+        if name.endswith("query.weight") or name.endswith("compress.weight"):
+            tensors[name] = tensors[name] * 12
+    for block in (model.blocks[0], model.blocks[2]):
+        block.mixer.w_c.mul_(12)
+        block.mixer.w_q.mul_(12)
+    ops.prepare(model, torch.float32)
+    cache = CacheManager(needs, 4, 20, 3, torch.float32, "cuda")
+    assert len(cache.groups) == 2 and [g.entries for g in cache.groups] == [[0, 2], [1]]
+    assert cache.groups[0].tensors["latent"].shape == (2, 20, 4, 12) and set(cache.groups[1].tensors) == {"k", "v"}
+    assert cache.bytes_per_page() == 2 * 4 * 12 * 4 + 2 * 4 * 2 * 16 * 4
+    runner = ModelRunner(model, cache, ops, torch.float32, "cuda", 128, 3)
+    g = torch.Generator().manual_seed(3)
+    prompts = {k: torch.randint(0, 83, (n,), generator=g).tolist() for k, n in (("p", 29), ("q", 12), ("r", 40))}
+    # 19 usable pages of 4 tokens for 81 tokens in all: q ends and r takes its pages
+    seqs, done, got = {}, {k: 0 for k in prompts}, {k: [] for k in prompts}
+    plan = [({"p": 5, "q": 12}, ["q"]), ({"p": 2, "r": 17}, []), ({"p": 22, "r": 1}, ["p"]), ({"r": 2}, []), ({"r": 20}, ["r"])]
+    for cuts, ended in plan:
+        entries = []
+        for k, n in cuts.items():
+            if k not in seqs:
+                seqs[k] = cache.new_sequence()
+            assert cache.append(seqs[k], done[k], n)
+            entries.append(StepEntry(seqs[k], prompts[k][done[k]:done[k] + n], done[k], list(range(n))))
+        logits = runner.step(entries).cpu()
+        at = 0
+        for k, n in cuts.items():
+            got[k].append(logits[at:at + n])
+            at += n
+            done[k] += n
+        for k in ended:
+            cache.free_sequence(seqs.pop(k))
+        cache.assert_consistent(list(seqs.values()))
+    for k, tokens in prompts.items():
+        torch.testing.assert_close(torch.cat(got[k]), plain_latent(tensors, raw, tokens), rtol=2e-4, atol=2e-5)
+    assert cache.num_used_pages() == 0
+
+    # the same architecture from a folder through the replay program's class
+    folder = write_random_model(raw, str(tmp_path / "latent"), seed=6, dtype="float32")
+    from safetensors.torch import load_file
+
+    stored = load_file(f"{folder}/model.safetensors")
+    replayer = Replayer(folder, "float32", max_tokens=64, block_size=4, ops=ops)
+    tokens = prompts["r"]
+    first = replayer.step({"step": 0, "entries": [{"id": "a", "tokens": tokens[:23], "want": [22]}, {"id": "b", "tokens": prompts["q"], "want": [11]}], "end": ["b"]})
+    rest = [replayer.step({"step": 1 + i, "entries": [{"id": "a", "tokens": [tokens[23 + i]], "want": [0]}], "end": []}) for i in range(17)]
+    want = plain_latent(stored, raw, tokens)
+    torch.testing.assert_close(torch.from_numpy(np.concatenate([first[:1]] + rest)), want[22:], rtol=2e-4, atol=2e-5)
+    torch.testing.assert_close(torch.from_numpy(first[1:2].copy()), plain_latent(stored, raw, prompts["q"])[-1:], rtol=2e-4, atol=2e-5)

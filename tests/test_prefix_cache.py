@@ -15,7 +15,7 @@ from velox_amd.cache.allocator import PageAllocator
 from velox_amd.cache.prefix import PrefixCache
 from velox_amd.engine.request import RequestStatus
 from velox_amd.engine.scheduler import Scheduler, SchedulerConfig
-from velox_amd.parts.base import PagedNeed, StateNeed
+from velox_amd.parts import PagedNeed, StateNeed, kv_pages
 
 
 # -- the trie alone ------------------------------------------------------------------------------------------------------
@@ -54,6 +54,22 @@ def test_publish_match_and_eviction_order():
     trie.assert_consistent()
     allocator.verify()
     assert trie.hit_rate == pytest.approx((4 + 4) / (6 + 6))
+
+
+def test_a_page_with_a_token_still_in_flight_is_not_published():
+    """A request's newest token may be a place holder while the step that draws it runs: a page that holds it is offered
+    only once the value is there, and the request goes on publishing then."""
+    from velox_amd.engine.request import PENDING_TOKEN
+
+    allocator = PageAllocator(8)
+    trie = PrefixCache([allocator], page_size=2)
+    pages = allocator.take_many(3)
+    tokens = [1, 2, 3, PENDING_TOKEN, 5, 6]
+    assert trie.publish(tokens, [pages], 0, 3) == (1, True) and trie.num_nodes == 1
+    assert trie.match([1, 2, 3, PENDING_TOKEN, 5], max_pages=2)[-1].pages == (pages[0],)
+    tokens[3] = 4
+    assert trie.publish(tokens, [pages], 1, 3) == (3, True) and trie.num_nodes == 3
+    trie.assert_consistent()
 
 
 def test_least_recently_used_leaf_goes_first_and_a_held_leaf_stays():
@@ -111,15 +127,15 @@ def test_nodes_hold_one_page_per_group():
 
 # -- the cache manager with it ---------------------------------------------------------------------------------------------
 def manager(pages=9, page=4, seqs=4, needs=None, **kwargs):
-    return CacheManager(needs or [PagedNeed(1, 16)], page, pages, seqs, torch.float32, "cpu", allocate_tensors=False, prefix_caching=True, **kwargs)
+    return CacheManager(needs or [kv_pages(1, 16)], page, pages, seqs, torch.float32, "cpu", allocate_tensors=False, prefix_caching=True, **kwargs)
 
 
 def test_only_models_whose_requests_hold_their_whole_past_share_prefixes():
     assert manager().prefix is not None
-    assert manager(needs=[PagedNeed(1, 16), PagedNeed(2, 32)]).prefix is not None
-    assert manager(needs=[PagedNeed(1, 16), PagedNeed(1, 16, window=8)]).prefix is None
-    assert manager(needs=[PagedNeed(1, 16), StateNeed((("s", (4,), None),))]).prefix is None
-    assert CacheManager([PagedNeed(1, 16)], 4, 9, 4, torch.float32, "cpu", allocate_tensors=False).prefix is None
+    assert manager(needs=[kv_pages(1, 16), kv_pages(2, 32)]).prefix is not None
+    assert manager(needs=[kv_pages(1, 16), kv_pages(1, 16, window=8)]).prefix is None
+    assert manager(needs=[kv_pages(1, 16), StateNeed((("s", (4,), None),))]).prefix is None
+    assert CacheManager([kv_pages(1, 16)], 4, 9, 4, torch.float32, "cpu", allocate_tensors=False).prefix is None
 
 
 def test_matched_pages_enter_the_table_and_one_token_is_left_to_compute():
@@ -214,7 +230,7 @@ def test_random_orders_of_requests_with_common_prefixes(seed):
 
 # -- the scheduler's admissions ----------------------------------------------------------------------------------------------
 def scheduler(pages=33, page=4, seqs=4, budget=16, chunk=8, max_len=128, watermark=0.01):
-    cache = CacheManager([PagedNeed(1, 16)], page, pages, seqs, torch.float32, "cpu", max_model_len=max_len, allocate_tensors=False, prefix_caching=True)
+    cache = CacheManager([kv_pages(1, 16)], page, pages, seqs, torch.float32, "cpu", max_model_len=max_len, allocate_tensors=False, prefix_caching=True)
     return Scheduler(cache, SchedulerConfig(max_num_seqs=seqs, max_num_batched_tokens=budget, max_prefill_chunk_size=chunk, max_model_len=max_len, watermark=watermark))
 
 

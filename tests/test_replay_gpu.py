@@ -217,6 +217,32 @@ OTHER_REAL_WIDTHS = {
 }
 
 
+def test_a_prompt_of_2048_tokens_in_true_32_bit_at_the_real_width(tmp_path):
+    """float32 at the widths of Qwen2.5-7B and at the prompt length the measurements use: ONE portion of 2,048 tokens (the
+    exact product with 2,048 rows and inner sizes of 3584 and 18944, the 32-bit attention kernel with a head size of 128
+    over a 2,048-row portion), then eight single tokens.  Two layers; the vocabulary is cut down and made odd.  The
+    yardstick is the plain model in float64: the engine has to be as close to it as three times the plain float32
+    model's own rounding."""
+    from velox_amd.weights import write_random_model
+
+    config = dict(QWEN25_7B_TWO_LAYERS, vocab_size=32003)
+    folder = write_random_model(config, str(tmp_path / "real_width"), 5, dtype="float32")
+    config, weights = read_model_folder(folder)
+    tokens = random_tokens(config["vocab_size"], 2056, seed=15)
+    places = [0, 1, 15, 16, 17, 511, 1023, 1024, 2031, 2032, 2046, 2047]  # of the portion: page edges, tile edges, the ends
+    exact = qwen2_logits(config, weights, tokens, dtype=torch.float64)
+    plain = qwen2_logits(config, weights, tokens)
+    rounding = float((plain.double() - exact).abs().max())
+    assert 1e-6 < rounding < 2e-4, rounding
+    replayer = Replayer(folder, "float32", 2112, block_size=16)
+    first = replayer.step({"step": 0, "entries": [{"id": "a", "tokens": tokens[:2048], "want": places}], "end": []})
+    rest = [replayer.step({"step": 1 + i, "entries": [{"id": "a", "tokens": [tokens[2048 + i]], "want": [0]}], "end": []}) for i in range(8)]
+    got = torch.from_numpy(np.concatenate([first] + rest)).double()
+    want = torch.cat([exact[places], exact[2048:]])
+    assert float((got - want).abs().max()) < 3 * rounding, (float((got - want).abs().max()), rounding)
+    assert float(want.std()) > 100 * rounding  # (the logits' spread: the bound is a small share of it)
+
+
 @pytest.mark.parametrize("shape", sorted(OTHER_REAL_WIDTHS))
 def test_layers_of_the_other_real_sizes(tmp_path, shape):
     """bfloat16, two layers with the widths of Qwen2.5-1.5B and of Qwen2.5-32B: the products' kernels are picked by width and

@@ -5,12 +5,12 @@ import torch
 from velox_amd.cache import CacheManager
 from velox_amd.engine.request import FinishReason, Request, RequestStatus
 from velox_amd.engine.scheduler import Scheduler, SchedulerConfig
-from velox_amd.parts.base import PagedNeed
+from velox_amd.parts import kv_pages
 from velox_amd.sampling import SamplingParams
 
 
 def make(pages=33, page=4, seqs=4, budget=16, chunk=8, max_len=128, watermark=0.01):
-    cache = CacheManager([PagedNeed(1, 16)], page, pages, seqs, torch.float32, "cpu", max_model_len=max_len, allocate_tensors=False)
+    cache = CacheManager([kv_pages(1, 16)], page, pages, seqs, torch.float32, "cpu", max_model_len=max_len, allocate_tensors=False)
     return Scheduler(cache, SchedulerConfig(max_num_seqs=seqs, max_num_batched_tokens=budget, max_prefill_chunk_size=chunk, max_model_len=max_len, watermark=watermark))
 
 

@@ -10,10 +10,9 @@ a ``StateNeed`` get one row per request in fixed-size tensors, indexed by the re
 *slot* (the reference's ``seq_index``, ``engine/scheduler.py:58,113-129``); slot rows are zeroed
 when a request takes the slot.
 
-Page layout, per entry of a group: keys ``[pages, kv_heads, page_size, head_dim]``, values
-``[pages, kv_heads, head_dim, page_size]`` (values are stored transposed inside a page so
-that the attention kernels read a run of consecutive keys for one channel in one
-contiguous access).
+What a page holds is the need's to say (``PagedNeed.tensors``: names, shapes per page and
+dtypes): per entry of a group every named tensor is ``[pages, *shape of one page]``, with the
+page size where the shape says ``PAGE``.  The manager knows nothing of keys or values.
 
 Growth rule per group (reference ``src/block_manager.py:74-99``): a request that has
 ``num_computed`` tokens in the cache and is given ``n`` more needs
@@ -28,7 +27,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
-from ..parts.base import PagedNeed, StateNeed
+from ..parts.base import PAGE, PagedNeed, StateNeed
 from .allocator import NULL_PAGE, PoolExhausted, PageAllocator
 from .prefix import PrefixCache
 
@@ -63,16 +62,26 @@ class PageGroup:
         self.page_size = int(page_size)
         self.allocator = PageAllocator(num_pages, scatter=scatter_pages)
         self.dtype = dtype
-        self.keys: Optional[torch.Tensor] = None
-        self.values: Optional[torch.Tensor] = None
+        # name -> (shape of one page, the dimension of it that runs over the page's tokens, dtype)
+        self.layout: Dict[str, Tuple[Tuple[int, ...], int, torch.dtype]] = {}
+        for name, shape, tensor_dtype in need.tensors:
+            shape = tuple(int(n) for n in shape)
+            axis = shape.index(PAGE)
+            self.layout[name] = (shape[:axis] + (self.page_size,) + shape[axis + 1:], axis, tensor_dtype or dtype)
+        # name -> [entries of the group, pages, *shape of one page]
+        self.tensors: Dict[str, torch.Tensor] = {}
         if allocate_tensors:
-            n, h, d = len(entries), need.num_kv_heads, need.head_dim
-            self.keys = torch.zeros((n, num_pages, h, page_size, d), dtype=dtype, device=device)
-            self.values = torch.zeros((n, num_pages, h, d, page_size), dtype=dtype, device=device)
+            for name, (shape, _, tensor_dtype) in self.layout.items():
+                self.tensors[name] = torch.zeros((len(entries), num_pages, *shape), dtype=tensor_dtype, device=device)
 
     def bytes_per_page(self) -> int:
-        element = torch.empty((), dtype=self.dtype).element_size()
-        return 2 * self.page_size * self.need.num_kv_heads * self.need.head_dim * element * len(self.entries)
+        per_entry = 0
+        for shape, _, tensor_dtype in self.layout.values():
+            numel = 1
+            for n in shape:
+                numel *= n
+            per_entry += numel * torch.empty((), dtype=tensor_dtype).element_size()
+        return per_entry * len(self.entries)
 
     def table_entries_for(self, num_tokens: int) -> int:
         return (num_tokens + self.page_size - 1) // self.page_size
@@ -131,10 +140,10 @@ class StateSlots:
 
 @dataclass
 class PagedView:
-    """What a mixer with a ``PagedNeed`` is handed for one schedule entry and one step."""
+    """What a mixer with a ``PagedNeed`` is handed for one schedule entry and one step: its page tensors by the names its
+    need gave them, each ``[pages, *shape of one page]``."""
 
-    k: torch.Tensor
-    v: torch.Tensor
+    tensors: Dict[str, torch.Tensor]
     block_size: int
     batch: object  # engine.batch.GroupBatch of this step
 
@@ -342,22 +351,26 @@ class CacheManager:
         if entry in self.entry_group:
             g, position = self.entry_group[entry]
             group = self.groups[g]
-            return PagedView(group.keys[position], group.values[position], group.page_size, group_batches[g])
+            return PagedView({name: tensor[position] for name, tensor in group.tensors.items()}, group.page_size, group_batches[g])
         if entry in self.state_entries:
             return StateView(self.state.tensors[entry])
         return None
 
-    def gather_sequence(self, entry: int, seq: SequenceCache, length: int):
-        """Contiguous keys and values ``[length, kv_heads, head_dim]`` of one request (a debugging aid,
-        reference ``src/paged_kv_cache.py:125-150``)."""
+    def gather_sequence(self, entry: int, seq: SequenceCache, length: int) -> Dict[str, torch.Tensor]:
+        """What the first ``length`` tokens of one request hold in the entry's page tensors, token by token: per tensor
+        ``[length, *shape of one page without its token dimension]`` (a debugging aid, reference
+        ``src/paged_kv_cache.py:125-150``)."""
         g, position = self.entry_group[entry]
         group = self.groups[g]
         index = torch.arange(length)
         pages = torch.tensor(seq.tables[g], dtype=torch.long)[index // group.page_size].to(self.device)
         offsets = (index % group.page_size).to(self.device)
-        keys = group.keys[position][pages, :, offsets, :]
-        values = group.values[position][pages, :, :, offsets]
-        return keys, values
+        out = {}
+        for name, tensor in group.tensors.items():
+            axis = group.layout[name][1]
+            per_page = tensor[position].movedim(1 + axis, 1)  # [pages, page_size, ...]
+            out[name] = per_page[pages, offsets]
+        return out
 
     # -- invariants ---------------------------------------------------------------------
     def assert_consistent(self, live: Sequence[SequenceCache] = ()) -> None:

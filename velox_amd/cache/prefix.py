@@ -126,6 +126,10 @@ class PrefixCache:
             node = node.children[tuple(tokens[index * self.page_size:(index + 1) * self.page_size])]
         for index in range(first, last):
             key = tuple(tokens[index * self.page_size:(index + 1) * self.page_size])
+            if any(token < 0 for token in key):
+                # a place holder for a token that a step in flight is still drawing: its value is not known, so the page
+                # cannot be found by its tokens; it is offered once the value has arrived
+                return index, True
             child = node.children.get(key)
             pages = tuple(table[index] for table in tables)
             if child is not None:

@@ -54,6 +54,12 @@ logger = logging.getLogger(__name__)
 _STAGES = ("scheduler_ms", "prepare_ms", "forward_ms", "sampling_ms", "cpu_sync_wait_ms", "step_ms", "gpu_ms")
 
 
+def model_position_limit(model_config) -> int:
+    """The most positions the architecture itself allows: ``ModelSpec.max_position`` of the spec made without a limit of
+    the caller's (every architecture's ``make_spec`` fills it from whatever its configuration calls it)."""
+    return int(get_architecture(model_config.architecture).make_spec(model_config, None).max_position)
+
+
 def build_model(model_config, dtype: torch.dtype, device, max_position: Optional[int] = None) -> DecoderModel:
     spec = get_architecture(model_config.architecture).make_spec(model_config, max_position)
     return DecoderModel(spec)
@@ -129,8 +135,7 @@ class Engine:
             from ..kernels import load_ops
 
             ops = load_ops(device)
-        max_position = getattr(model_config, "max_position_embeddings", None)
-        max_model_len = min(config.max_model_len, max_position) if max_position else config.max_model_len
+        max_model_len = min(config.max_model_len, model_position_limit(model_config))
         config.max_model_len = max_model_len
         model = build_model(model_config, dtype, device, max_position=max_model_len)
         bind(model, dtype, device)
@@ -303,6 +308,14 @@ class Engine:
         dest_rows: List[int] = []
         source_rows: List[int] = []
         source_of = {id(r): row for row, r in enumerate(pending.sampled)} if pending is not None else {}
+
+        def source_row(request: Request) -> int:
+            # a pending token belongs to the step just before this one: nothing else can still be in flight
+            row = source_of.get(id(request))
+            if row is None:
+                raise RuntimeError(f"request {request.request_id!r} has a token in flight, but the step before this one did not sample it")
+            return row
+
         at = 0  # rows of the step so far
         # decode rows first, then prompt portions; only rows that complete their tokens are sampled
         for request in plan.decodes:
@@ -310,7 +323,7 @@ class Engine:
             token = request.all_token_ids[start]
             if token == PENDING_TOKEN:
                 dest_rows.append(at)
-                source_rows.append(source_of[id(request)])
+                source_rows.append(source_row(request))
             entries.append(StepEntry(request.cache, [token], start, [0]))
             sampled.append(request)
             at += 1
@@ -319,7 +332,7 @@ class Engine:
             tokens = request.all_token_ids[start:start + count]
             if tokens[-1] == PENDING_TOKEN:  # (only a request's newest token can be pending)
                 dest_rows.append(at + count - 1)
-                source_rows.append(source_of[id(request)])
+                source_rows.append(source_row(request))
             entries.append(StepEntry(request.cache, tokens, start, [count - 1] if portion.completes else []))
             if portion.completes:
                 sampled.append(request)

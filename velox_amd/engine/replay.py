@@ -26,7 +26,7 @@ from ..config.engine_config import resolve_dtype
 from ..config.registry import load_config
 from ..weights import bind_from_checkpoint
 from .batch import StepEntry
-from .engine import build_model
+from .engine import build_model, model_position_limit
 from .runner import ModelRunner
 
 
@@ -51,8 +51,7 @@ class Replayer:
         if pages < 1:
             raise TraceError("--max-tokens must be positive")
         capacity = pages * block_size
-        limit = getattr(self.config, "max_position_embeddings", capacity)
-        self.max_model_len = min(capacity, limit)
+        self.max_model_len = min(capacity, model_position_limit(self.config))
         self.model = build_model(self.config, self.dtype, self.device, max_position=self.max_model_len)
         bind_from_checkpoint(self.model, model_dir, self.dtype, self.device)
         ops.prepare(self.model, self.dtype)

@@ -12,7 +12,13 @@ A batch in which every entry has one token may be replayed from a captured HIP g
 graphs are captured per batch-size bucket 1, 2, 4, ... (reference
 ``engine/model_runner.py:19-26,331-368``), rows beyond the batch are padded with one-token
 rows that read and write the reserved null page, and the step's tensors live at fixed
-addresses that the host refreshes before each replay.
+addresses that the host refreshes before each replay.  A capture fixes how its kernels are
+launched; a part whose kernels would be launched differently behind short contexts says so
+(``Part.capture_key_bounds``) and gets further captures of the same bucket, each for steps whose
+sequences all stay within a bound on their length; a step replays the tightest capture that
+covers it.  The captured activations live in the pool of the framework's graph allocator
+(``torch.cuda.graph_pool_handle``), shared by all captures; the step's inputs and the parts'
+scratch are the runner's own buffers.
 """
 from __future__ import annotations
 
@@ -36,11 +42,6 @@ def decode_buckets(max_num_seqs: int) -> List[int]:
     return buckets
 
 
-# A captured decode step fixes how many workgroups share a sequence's keys (the split count is part of the launch).
-# Chosen for the longest context the engine allows, that count is too many behind few keys, where one workgroup per
-# sequence and KV head is quicker than splits and their merge; so steps whose sequences all hold at most this many
-# keys have a capture of their own.
-SHORT_CONTEXT_KEYS = 384
 
 
 class ModelRunner:
@@ -81,7 +82,8 @@ class ModelRunner:
         # a model with a part that reads the host while it runs (``Part.graph_safe`` False) is never captured
         self.enable_graphs = bool(enable_graphs) and self.device.type == "cuda" and model.allows_capture()
         self._graphs: Dict[int, Tuple[object, torch.Tensor, torch.Tensor]] = {}
-        self._short_graphs: Dict[int, Tuple[object, torch.Tensor, torch.Tensor]] = {}  # the same buckets behind few keys
+        # the same buckets again for steps whose sequences are all short: bucket -> [(bound on keys, capture)], tightest first
+        self._bounded_graphs: Dict[int, List[Tuple[int, Tuple[object, torch.Tensor, torch.Tensor]]]] = {}
         self._graph_buffers: Dict[int, torch.Tensor] = {}
         self._graph_pool = None
         self.num_graph_replays = 0
@@ -151,13 +153,16 @@ class ModelRunner:
             return
         buckets = list(buckets) if buckets is not None else decode_buckets(self.max_num_seqs)
         self._graph_pool = torch.cuda.graph_pool_handle()
-        self._short_graphs.clear()
+        self._bounded_graphs.clear()
+        parts = self.model.all_parts()
+        longest = self.cache.max_model_len
         for bucket in buckets:
             capacity = self.builder.section_total(bucket, bucket, bucket, self.builder.width)
             self._graph_buffers[bucket] = torch.zeros(capacity, dtype=torch.int32, device=self.device)
-            self._graphs[bucket] = self._capture(self._graph_context(bucket, self.cache.max_model_len), warmup_iters)
-            if self.cache.max_model_len > SHORT_CONTEXT_KEYS and self._splits_differ(bucket):
-                self._short_graphs[bucket] = self._capture(self._graph_context(bucket, SHORT_CONTEXT_KEYS), warmup_iters)
+            self._graphs[bucket] = self._capture(self._graph_context(bucket, longest), warmup_iters)
+            bounds = sorted({int(b) for part in parts for b in part.capture_key_bounds(self.ops, bucket, longest) if 0 < int(b) < longest})
+            if bounds:
+                self._bounded_graphs[bucket] = [(bound, self._capture(self._graph_context(bucket, bound), warmup_iters)) for bound in bounds]
         torch.cuda.synchronize()
 
     def _capture(self, ctx: StepContext, warmup_iters: int):
@@ -172,18 +177,6 @@ class ModelRunner:
         with torch.cuda.graph(graph, pool=self._graph_pool):
             logits = self._forward(ctx)
         return graph, logits, ctx
-
-    def _splits_differ(self, bucket: int) -> bool:
-        """Whether any paged group's attention would split the keys of a ``bucket``-row step behind the longest context
-        but not behind a short one (only then is a second capture worth its memory)."""
-        choose = getattr(self.ops, "choose_splits", None)
-        if choose is None:
-            return False
-        for group in self.cache.groups:
-            heads = group.need.num_kv_heads
-            if choose(bucket, heads, 1, self.cache.max_model_len, True) != choose(bucket, heads, 1, SHORT_CONTEXT_KEYS, True):
-                return True
-        return False
 
     def _graph_context(self, bucket: int, max_kv_len: int) -> StepContext:
         """A context of ``bucket`` padded rows only (all on the null page), laid out in the bucket's buffer."""
@@ -217,9 +210,13 @@ class ModelRunner:
 
     def _replay(self, bucket: int, entries: Sequence[StepEntry], device_ids: Optional[tuple] = None) -> torch.Tensor:
         graph, logits, _ = self._graphs[bucket]
-        if bucket in self._short_graphs and all(e.start < SHORT_CONTEXT_KEYS for e in entries):
-            graph, logits, _ = self._short_graphs[bucket]
-            self.num_short_graph_replays += 1
+        if bucket in self._bounded_graphs:
+            keys = max(e.start for e in entries) + 1  # the longest sequence of the step, this token's key included
+            for bound, capture in self._bounded_graphs[bucket]:
+                if keys <= bound:
+                    graph, logits, _ = capture
+                    self.num_short_graph_replays += 1
+                    break
         self._padded_entries_context(bucket, entries, device_ids)  # refreshes the bucket's buffer in place
         graph.replay()
         self.num_graph_replays += 1

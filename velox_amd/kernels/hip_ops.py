@@ -153,13 +153,13 @@ class HipOps:
         return lib
 
     def prepare(self, model, dtype) -> None:
-        """Builds (at first use) and loads what this model's mixers need, and lets every part register the weights
-        that decode-sized products read (``Part.prepare_kernels``)."""
-        for need in model.cache_needs():
-            if need is not None and hasattr(need, "head_dim"):
-                self.attention_library(need.head_dim)
+        """Lets every part get what it needs of the kernels before the first step (``Part.prepare_kernels``): the weights
+        that decode-sized products read are registered, and libraries that are built per size (attention, per head
+        size) are built and loaded by the parts that use them."""
         for part in model.all_parts():
             part.prepare_kernels(self)
+        if dtype == torch.bfloat16 and self.use_library_gemm and self._mm_out_dtype_ok is None:
+            self._decide_float32_out_route()
 
     def prepare_weight(self, weight: torch.Tensor, stacked: int = 1, rotary_heads: Optional[Tuple[int, int, int]] = None,
                        handle: Optional[PreparedWeight] = None) -> Optional[PreparedWeight]:
@@ -407,14 +407,25 @@ class HipOps:
         if self.use_library_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and bias is None:
             if out_dtype == torch.bfloat16:
                 return torch.nn.functional.linear(x, weight)
-            if out_dtype == torch.float32 and self._mm_out_dtype_ok is not False:
-                try:
-                    out = torch.mm(x, weight.t(), out_dtype=torch.float32)
-                    self._mm_out_dtype_ok = True
-                    return out
-                except (RuntimeError, TypeError):
-                    self._mm_out_dtype_ok = False
+            if out_dtype == torch.float32:
+                if self._mm_out_dtype_ok is None:
+                    self._decide_float32_out_route()
+                return torch.mm(x, weight.t(), out_dtype=torch.float32)
         return self.gemm_fma(x, weight, bias, out_dtype)
+
+    def _decide_float32_out_route(self) -> None:
+        """Decides once how a bfloat16 product with a float32 result and more rows than the skinny kernels take (the
+        head over many wanted rows) is computed: by the library with a float32 output, if this PyTorch has that call.
+        If it has not, that is an error here, at load time, and not a silent fall to the exact FMA kernel, which is some
+        two hundred times slower at such sizes."""
+        probe = torch.zeros((32, 64), dtype=torch.bfloat16, device=self.device)
+        try:
+            torch.mm(probe, probe.t(), out_dtype=torch.float32)
+            self._mm_out_dtype_ok = True
+        except (RuntimeError, TypeError) as err:
+            self._mm_out_dtype_ok = False
+            raise KernelError("this PyTorch's matrix library has no bfloat16 product with a float32 result (torch.mm(..., out_dtype=)); "
+                              f"logits of many rows at once need it in a bfloat16 run: {err}") from err
 
     def _linear_into_residual(self, x: torch.Tensor, weight: torch.Tensor, sink: ResidualSink, waves: Optional[int] = None, row_tiles: Optional[int] = None,
                               packed: Optional[torch.Tensor] = None) -> Optional[DeferredNorm]:
@@ -743,7 +754,9 @@ class HipOps:
     def attention_scratch_elems(self, num_heads: int, num_kv_heads: int, head_dim: int, max_num_tokens: int, max_num_seqs: int, max_model_len: int) -> Tuple[int, int]:
         """The most float32 elements ``paged_attention`` asks its workspace for (partial outputs, partial log-sums) in
         any step of at most ``max_num_tokens`` tokens and ``max_num_seqs`` sequences behind at most ``max_model_len`` keys,
-        with the splits that ``choose_splits`` and ``choose_portion_splits`` pick."""
+        with the splits that ``choose_splits`` and ``choose_portion_splits`` pick.  The bound counts TOKENS, not sequences:
+        the sequence on the null page that pads a step up to a timed number of rows (one more than ``max_num_seqs``) brings
+        tokens within ``max_num_tokens`` like any other and is covered."""
         group = num_heads // num_kv_heads
         rows = 0  # splits x the rows the partial results are counted by
         for count in range(1, max_num_seqs + 1):  # single tokens, alone or before portions

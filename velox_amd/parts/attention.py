@@ -17,7 +17,18 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import Mixer, PagedNeed, Param, PositionEncoding, fused_rows, register_part, single
+from .base import PAGE, Mixer, PagedNeed, Param, PositionEncoding, fused_rows, register_part, single
+
+# Behind this many keys a decode step's attention runs without splitting a sequence's keys over workgroups (splits and
+# their merge cost about as much as one workgroup's walk over that many keys): captured steps exist a second time for
+# steps whose sequences are all that short, when the two would be launched differently.
+SHORT_CONTEXT_KEYS = 384
+
+
+def kv_pages(num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> PagedNeed:
+    """What attention keeps per page: keys ``[kv_heads, page, head_dim]`` and values transposed, ``[kv_heads, head_dim,
+    page]`` (a run of consecutive keys for one channel is then one contiguous access for the kernels' second product)."""
+    return PagedNeed((("k", (int(num_kv_heads), PAGE, int(head_dim)), None), ("v", (int(num_kv_heads), int(head_dim), PAGE), None)), window)
 
 
 class AttentionMixer(Mixer):
@@ -69,17 +80,27 @@ class AttentionMixer(Mixer):
         return out
 
     def cache_need(self):
-        return PagedNeed(self.num_kv_heads, self.head_dim, self.window)
+        return kv_pages(self.num_kv_heads, self.head_dim, self.window)
 
     def _rotary_tables(self):
         tables = self.position.rotary_tables() if self.position is not None else None
         return tables if tables is not None else (None, None)
 
     def prepare_kernels(self, ops) -> None:
+        load = getattr(ops, "attention_library", None)
+        if load is not None:
+            load(self.head_dim)  # built at first use for this head size; a missing compiler fails here, not in a step
         cos, _ = self._rotary_tables()
         whole_heads = cos is not None and 2 * cos.shape[1] == self.head_dim
         self.prepare_weight(ops, "qkv_weight", rotary_heads=(self.num_heads, self.num_kv_heads, self.head_dim) if whole_heads else None)
         self.prepare_weight(ops, "o_weight")
+
+    def capture_key_bounds(self, ops, batch: int, max_model_len: int):
+        choose = getattr(ops, "choose_splits", None)
+        if choose is None or max_model_len <= SHORT_CONTEXT_KEYS:
+            return ()
+        differs = choose(batch, self.num_kv_heads, 1, max_model_len, True) != choose(batch, self.num_kv_heads, 1, SHORT_CONTEXT_KEYS, True)
+        return (SHORT_CONTEXT_KEYS,) if differs else ()
 
     def workspace_needs(self, ops, limits):
         sizes = getattr(ops, "attention_scratch_elems", None)
@@ -100,12 +121,12 @@ class AttentionMixer(Mixer):
             x, self.operand("qkv_weight"), self.qkv_bias_vec if self.qkv_bias else None,
             self.num_heads, self.num_kv_heads, self.head_dim,
             ctx.positions, cos, sin,
-            meta.slot_mapping, cache.k, cache.v, cache.block_size,
+            meta.slot_mapping, cache.tensors["k"], cache.tensors["v"], cache.block_size,
             write_kv=owns_cache,
         )
         attn = ops.paged_attention(
             q, self.num_heads, self.num_kv_heads, self.head_dim,
-            cache.k, cache.v, cache.block_size,
+            cache.tensors["k"], cache.tensors["v"], cache.block_size,
             meta.block_tables, ctx.cu_q, meta.kv_lens,
             ctx.max_q_len, meta.max_kv_len, self.scale, self.window,
             ctx.all_decode, ctx.workspace,

@@ -124,6 +124,13 @@ class Part:
                                "call ops.prepare(model, dtype) again")
         return handle
 
+    def capture_key_bounds(self, ops, batch: int, max_model_len: int):
+        """Context lengths below ``max_model_len`` for which a captured step of ``batch`` one-token rows should exist a
+        second time, because this part's kernels would be launched differently when every sequence is that short (a
+        capture fixes launch shapes; the step function replays the capture with the smallest bound that covers the
+        step).  Default: none."""
+        return ()
+
     def workspace_needs(self, ops, limits) -> Dict[str, int]:
         """Scratch this part may ask ``ctx.workspace`` for: buffer name -> the most float32 elements, for any step within
         ``limits`` (``max_num_tokens``, ``max_num_seqs``, ``max_model_len``).  The step function reserves these before it
@@ -134,18 +141,34 @@ class Part:
 # ----------------------------------------------------------------------------------------
 # what a mixer needs of the cache manager
 # ----------------------------------------------------------------------------------------
+PAGE = -1  # stands in a page tensor's shape for the dimension that runs over the tokens of a page
+
+
 @dataclass(frozen=True)
 class PagedNeed:
-    """Keys and values that grow by one entry per token, kept in pages.
+    """Memory that grows by one entry per token, kept in pages.
 
-    ``window`` = None keeps every key; an integer keeps the last ``window`` keys
-    (a query at position p reads keys p-window+1 .. p), so pages wholly behind
-    the window can be given back while the request is still running.
+    ``tensors``: what a page holds, ``(name, shape of one page, dtype)`` per tensor; ``PAGE`` in a shape marks the
+    dimension that runs over the page's tokens (its size is the page size, which the cache manager decides), dtype
+    None = the run dtype.  The mixer decides the layout: attention keeps keys as ``(kv_heads, PAGE, head_dim)`` and
+    values transposed (``parts.attention.kv_pages``); a mixer that caches one latent vector per token would name a
+    single ``(PAGE, width)`` tensor.  Entries of the schedule with equal needs share a pool of pages.
+
+    ``window`` = None keeps every token; an integer keeps the last ``window`` of them (a query at position p reads
+    positions p-window+1 .. p), so pages wholly behind the window can be given back while the request is still running.
     """
 
-    num_kv_heads: int
-    head_dim: int
+    tensors: Tuple[Tuple[str, Tuple[int, ...], Optional[torch.dtype]], ...]
     window: Optional[int] = None
+
+    def __post_init__(self) -> None:
+        if not self.tensors:
+            raise ValueError("a PagedNeed names at least one tensor per page")
+        for name, shape, _ in self.tensors:
+            if tuple(shape).count(PAGE) != 1:
+                raise ValueError(f"page tensor {name!r}: its shape {tuple(shape)} must hold PAGE exactly once")
+        if self.window is not None and self.window < 1:
+            raise ValueError(f"window={self.window} must be at least 1")
 
 
 @dataclass(frozen=True)
