@@ -61,7 +61,7 @@ def test_an_engine_over_weights_drawn_on_the_device_computes_the_plain_models_lo
 
     config = CONFIGS[name]
     engine = Engine.from_random(config, seed=21, config=EngineConfig(
-        dtype=dtype, device="cuda", max_model_len=160, max_num_seqs=4, max_num_batched_tokens=32, max_prefill_chunk_size=7,
+        dtype=dtype, device="cuda", max_model_len=160, max_num_seqs=4, max_num_batched_tokens=64, max_prefill_chunk_size=7,
         block_size=PAGE_SIZE[name], num_gpu_blocks=96, enable_cuda_graphs=False, seed=0, enable_prefix_caching=False), generator_device="cuda")
     weights = {key: value.float().cpu() for key, value in named_tensors(engine.model)}
     assert ("lm_head.weight" in weights) != bool(config["tie_word_embeddings"])
