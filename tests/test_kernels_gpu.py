@@ -574,6 +574,50 @@ def test_paged_attention_window(ops, ref, dtype, nh, nkv, d, page, window):
     torch.testing.assert_close(got, want, **(dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)))
 
 
+@pytest.mark.parametrize("nh,nkv,d,page", [(28, 4, 128, 16), (12, 2, 128, 8), (8, 8, 64, 64), (6, 3, 64, 16), (5, 1, 128, 32)])
+@pytest.mark.parametrize("window", [None, 300])
+def test_paged_attention_with_tiles_loaded_straight_into_lds(ops, ref, nh, nkv, d, page, window):
+    """The kernel for portions of prompts whose tiles of keys and values reach LDS by direct loads (bfloat16, head sizes 64
+    and 128, pages of 8 tokens and more), made to run wherever it can, beside the kernel it stands in for: whole prompts
+    whose lengths are no multiple of a tile or of a piece of eight keys, portions behind longer contexts, short
+    entries beside them, pages in no order, and loud garbage in every slot beyond the sequences' ends (values there must
+    not reach the output, not even multiplied with a probability of zero) and on the null page."""
+    from velox_amd.engine.batch import Workspace
+
+    lib = ops.attention_library(d)
+    seqs = [(1100, 1100), (700, 1301), (1, 97), (300, 300), (2, 40), (67, 67), (130, 1003)]
+    case = _attention_case(torch.bfloat16, nh, nkv, d, page, seqs, seed=d + nh + 7)
+    dirty = _attention_case(torch.bfloat16, nh, nkv, d, page, seqs, seed=d + nh + 7, garbage=True)
+    dirty["qkv"], dirty["tables"] = case["qkv"], case["tables"]
+    tables = case["tables"].cpu()
+    used = torch.zeros(dirty["k_cache"].shape[0], page, dtype=torch.bool)
+    for b, (_, kv_len) in enumerate(seqs):
+        for n in range(kv_len):
+            used[int(tables[b, n // page]), n % page] = True
+    keep = used.cuda()
+    dirty["k_cache"] = torch.where(keep[:, None, :, None], case["k_cache"], dirty["k_cache"] * float("inf"))  # +-inf where no key lives
+    dirty["v_cache"] = torch.where(keep[:, None, None, :], case["v_cache"], dirty["v_cache"] * float("inf"))
+    tolerance = dict(rtol=2e-2, atol=2e-2)
+    want = _run_attention(ref, case, nh, nkv, d, page, window=window)
+    try:
+        results = {}
+        for choice in (1, 2):
+            lib.velox_attention_portion_kernel(choice)
+            results[choice] = _run_attention(ops, case, nh, nkv, d, page, window=window)
+            torch.testing.assert_close(results[choice], want, **tolerance)
+            assert torch.equal(_run_attention(ops, dirty, nh, nkv, d, page, window=window), results[choice])
+        assert not torch.equal(results[1], results[2])  # two kernels did run (they add a row's keys in different orders)
+        # split keys (few tokens behind many keys) through the same kernel, and the partial results merged
+        lib.velox_attention_portion_kernel(2)
+        far = _attention_case(torch.bfloat16, nh, nkv, d, page, [(150, 4400), (90, 90), (2, 4200)], seed=d + nh + 8)
+        workspace = Workspace(torch.device("cuda"))
+        for splits in (1, 3, 4):
+            got = _run_attention(ops, far, nh, nkv, d, page, window=window, splits=splits, workspace=workspace)
+            torch.testing.assert_close(got, _run_attention(ref, far, nh, nkv, d, page, window=window), **tolerance)
+    finally:
+        lib.velox_attention_portion_kernel(0)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 4), (28, 4, 128, 16), (3, 1, 32, 8), (2, 1, 256, 16)])
 def test_decode_split_keys_equals_one_pass(ops, ref, dtype, nh, nkv, d, page):

@@ -547,6 +547,306 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
   }
 }
 
+// ---- portions of prompts, bfloat16, tiles brought into LDS by the memory system itself ---------------------------------
+// The same arithmetic as the general kernel with CT row tiles per wave, for head sizes of 64 and 128 channels and pages
+// of at least 8 tokens.  What differs is how a tile of 64 keys gets into LDS: every lane asks for 16 bytes of the
+// cache with a load that writes LDS directly (no registers, no LDS write instructions, no address arithmetic on the
+// way back), a whole tile AHEAD of the one being multiplied, into the other of two tile buffers.  One barrier per tile
+// is left: behind it every wave has read the buffer that the next loads overwrite and this tile has landed.
+//
+// Such a load puts lane l's 16 bytes at (wave-uniform base) + 16 l, so an instruction fills one contiguous kilobyte
+// and what lies where in LDS is decided by which piece of the cache each lane asks for.  Pieces are placed so that
+// the operand reads are free of bank conflicts without padding: a K row (2 D bytes) keeps its place and its 16-byte
+// pieces are exchanged among themselves, piece c of key k sits at place c ^ f(k) with f(k) = (k & 3) | ((k >> 3) & 1) << 2;
+// a V^T row (128 bytes: 64 keys of one channel) likewise, piece c of channel d sits at place c ^ (d & 7).  Any eight
+// lanes that read together (consecutive rows, the same piece) then touch eight different places.
+//
+// S^T tiles take their keys in another order than the general kernel: tile u of key block b (32 keys), row 4 q + j
+// (q = 0..3, j = 0..3) is key 32 b + 8 q + 4 u + j.  Lane group g then holds, over the block's two tiles, the scores
+// of keys 8 g .. 8 g + 7 of the block: eight consecutive keys, which is one 16-byte piece of a V^T row in its natural
+// order.  (The general kernel reorders V^T instead, in pieces of 8 bytes; a direct load cannot.)  For such a row of K
+// f(k) is i & 7 for lane i: a constant of the lane.
+template <int CT, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, WAVES > 4 ? 4 : 2))) direct_attention_kernel(
+    const bf16_t* __restrict__ qkv, int qkv_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
+    bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
+    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens, int slots) {
+  typedef bf16_t T;
+  typedef Block<T> B;
+  typedef typename B::Operand Operand;
+  static_assert(CT > 0 && (D == 64 || D == 128), "head sizes whose rows are a power of two of 16-byte pieces, at least eight");
+  constexpr int BN = 64, KB = 32, VEC = 8;
+  constexpr int NT = BN / 16, NQB = D / KB, NKB = BN / KB, NC = D / 16;
+  constexpr int CPR = D / 8;                        // 16-byte pieces of a K row
+  constexpr int TILE_BYTES = BN * D * 2;            // K tile and V^T tile alike
+  constexpr int LOADS = TILE_BYTES / 1024;          // load instructions per tile and operand
+  static_assert(LOADS % WAVES == 0, "every wave issues the same number of loads");
+  constexpr int LPW = LOADS / WAVES;
+  constexpr int ROWS_PER_BLOCK = 16 * WAVES * CT;
+  __shared__ __attribute__((aligned(1024))) char smem[2][2 * TILE_BYTES];
+  __shared__ int page_ids[PREFILL_PAGE_IDS];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = lane >> 4, i = lane & 15;
+  const int group = nh / nkv;
+  const int b = blockIdx.z / splits, split = blockIdx.z % splits;
+  const int page_size = 1 << page_shift;
+
+  const int q_start = cu_q[b];
+  const int q_len = cu_q[b + 1] - q_start;
+  const int kv_len = kv_lens[b];
+  const int ctx = kv_len - q_len;
+  const int rows_total = q_len * group;
+  // (which rows and which KV head: as in the general kernel, the longest units first, then the shortest, ...)
+  const int blocks_here = (rows_total + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
+  const int units = blocks_here * nkv;
+  const int launch_index = blockIdx.x + gridDim.x * blockIdx.y;
+  if (launch_index >= units) return;
+  const int round = launch_index / slots, within = launch_index % slots;
+  const int rank = (round & 1) ? units - 1 - ((round >> 1) * slots + within) : (round >> 1) * slots + within;  // 0 = longest
+  const int kvh = rank % nkv;
+  const int r0 = (blocks_here - 1 - rank / nkv) * ROWS_PER_BLOCK;
+
+  bool row_ok[CT];
+  int tok[CT], head[CT], pos[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int r = r0 + (wave * CT + ct) * 16 + i;
+    row_ok[ct] = r < rows_total;
+    tok[ct] = row_ok[ct] ? r / group : 0;
+    head[ct] = kvh * group + (row_ok[ct] ? r % group : 0);
+    pos[ct] = ctx + tok[ct];
+  }
+  const int first_tok = r0 / group;
+  const int last_row = (r0 + ROWS_PER_BLOCK - 1 < rows_total - 1) ? r0 + ROWS_PER_BLOCK - 1 : rows_total - 1;
+  const int last_tok = last_row / group;
+  int n_end = ctx + last_tok + 1;
+  if (n_end > kv_len) n_end = kv_len;
+  int n_begin = 0;
+  if (window > 0) {
+    n_begin = ctx + first_tok - window + 1;
+    if (n_begin < 0) n_begin = 0;
+    n_begin = n_begin / BN * BN;
+  }
+  const int tiles_total = (n_end - n_begin + BN - 1) / BN;
+  const int tiles_per_split = (tiles_total + splits - 1) / splits;
+  const int tile_lo = split * tiles_per_split;
+  int tile_hi = tile_lo + tiles_per_split;
+  if (tile_hi > tiles_total) tile_hi = tiles_total;
+
+  int wave_last_pos = -1, wave_first_pos = 0x7fffffff;
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    if (row_ok[ct] && pos[ct] > wave_last_pos) wave_last_pos = pos[ct];
+    if (row_ok[ct] && pos[ct] < wave_first_pos) wave_first_pos = pos[ct];
+  }
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) {
+    const int hi = __shfl_xor(wave_last_pos, offset, VELOX_WAVE);
+    const int lo = __shfl_xor(wave_first_pos, offset, VELOX_WAVE);
+    wave_last_pos = hi > wave_last_pos ? hi : wave_last_pos;
+    wave_first_pos = lo < wave_first_pos ? lo : wave_first_pos;
+  }
+
+  // page ids of the keys this workgroup visits, a window of PREFILL_PAGE_IDS pages at a time
+  const int* table = block_tables + (size_t)b * table_width;
+  const int last_key = n_begin + tile_hi * BN < kv_len ? n_begin + tile_hi * BN : kv_len;
+  const int last_page = tile_hi > tile_lo ? (last_key - 1) >> page_shift : -1;
+  int first_page = (n_begin + tile_lo * BN) >> page_shift;
+  auto load_page_ids = [&]() {
+    const int num_pages = last_page - first_page + 1;
+    for (int p = tid; p < num_pages && p < PREFILL_PAGE_IDS; p += 64 * WAVES) page_ids[p] = table[first_page + p];
+  };
+  load_page_ids();
+  auto page_of = [&](int n) -> size_t { return (size_t)page_ids[(n >> page_shift) - first_page]; };
+
+  Operand qf[CT][NQB];
+  float m_i[CT], l_i[CT];
+  float4_t acc_o[CT][NC];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const T* qp = qkv + (size_t)(q_start + tok[ct]) * qkv_stride + (size_t)head[ct] * D + VEC * g;
+#pragma unroll
+    for (int cb = 0; cb < NQB; ++cb)
+      qf[ct][cb] = row_ok[ct] ? load_operand<T>(qp + KB * cb) : __builtin_bit_cast(Operand, float4_t{0.f, 0.f, 0.f, 0.f});
+    m_i[ct] = -INFINITY;
+    l_i[ct] = 0.f;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) acc_o[ct][c] = float4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  const float scale_eff = scale * Softmax<T>::SCALE;
+
+  // ---- what each lane asks for: load instruction q = wave + WAVES * m of a tile fills bytes [1024 q, 1024 q + 1024) of
+  // the K part (or the V^T part) of a buffer; lane l's 16 bytes are piece s = 64 q + l of the tile
+  int k_key[LPW], k_col[LPW], v_chan[LPW];
+  int v_key;
+#pragma unroll
+  for (int m = 0; m < LPW; ++m) {
+    const int s = 64 * (wave + WAVES * m) + lane;
+    const int key = s / CPR, place = s % CPR;
+    k_key[m] = key;
+    k_col[m] = 8 * (place ^ ((key & 3) | (((key >> 3) & 1) << 2)));
+    v_chan[m] = s / 8;
+  }
+  v_key = 8 * ((lane & 7) ^ ((lane >> 3) & 7));  // (the channel's low bits are the lane's: 64 q is a multiple of 8 channels)
+  auto issue = [&](int n0, int buffer) {
+    char* const k_dst = smem[buffer];
+    char* const v_dst = smem[buffer] + TILE_BYTES;
+#pragma unroll
+    for (int m = 0; m < LPW; ++m) {
+      int nk = n0 + k_key[m];
+      nk = nk < kv_len ? nk : kv_len - 1;  // (a key beyond the sequence: any valid address; its scores are masked)
+      const T* src = k_cache + (((page_of(nk) * nkv + kvh) << page_shift) + (nk & (page_size - 1))) * D + k_col[m];
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(k_dst + 1024 * (wave + WAVES * m)), 16, 0, 0);
+    }
+#pragma unroll
+    for (int m = 0; m < LPW; ++m) {
+      int nv = n0 + v_key;
+      nv = nv < kv_len ? nv : (kv_len - 1) & ~7;
+      const T* src = v_cache + (((page_of(nv) * nkv + kvh) * D + v_chan[m]) << page_shift) + (nv & (page_size - 1));
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(v_dst + 1024 * (wave + WAVES * m)), 16, 0, 0);
+    }
+  };
+
+  // ---- where each lane reads its operands.  K: row 8 (i / 4) + (i % 4) of a key block (+ 4 u for tile u, + 32 b for
+  // block b), piece (4 cb + g) ^ (i & 7) = 4 (cb ^ h) + (g ^ (i & 3)) with h = (i / 4) & 1.  V^T: row i of a channel
+  // tile, piece (4 kb + g) ^ (i & 7) likewise.
+  const int h = (i >> 2) & 1;
+  const int k_row_bytes = (8 * (i >> 2) + (i & 3)) * (2 * D) + 16 * (g ^ (i & 3));
+  const int k_even = k_row_bytes + 64 * h, k_odd = k_row_bytes + 64 * (1 - h);           // cb even / odd: + 128 (cb / 2)
+  const int v_row_bytes = TILE_BYTES + i * 128 + 16 * (g ^ (i & 3));
+  const int v_first = v_row_bytes + 64 * h, v_second = v_row_bytes + 64 * (1 - h);       // kb = 0 / 1
+
+  __syncthreads();  // page ids are in place
+  if (tile_lo < tile_hi) issue(n_begin + tile_lo * BN, 0);
+  int buffer = 0;
+  for (int tile = tile_lo; tile < tile_hi; ++tile, buffer ^= 1) {
+    const int n0 = n_begin + tile * BN;
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces of the tile have landed
+    __syncthreads();                      // everybody's have, and everybody is done with the other buffer
+    if (tile + 1 < tile_hi) {
+      const int next = n0 + BN;
+      if (((next + BN - 1) >> page_shift) - first_page >= PREFILL_PAGE_IDS) {  // the same for every thread
+        first_page = next >> page_shift;
+        __syncthreads();
+        load_page_ids();
+        __syncthreads();
+      }
+      issue(next, buffer ^ 1);
+    }
+    if (n0 > wave_last_pos) continue;  // nothing this wave may read
+    const char* const tile_base = smem[buffer];
+
+    // ---- S^T = K Q^T: tile t = 2 b + u of the 64 keys ----------------------------------------
+    float4_t s[CT][NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int tile_bytes = (32 * (t >> 1) + 4 * (t & 1)) * (2 * D);
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) s[ct][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int cb = 0; cb < NQB; ++cb) {
+        const Operand kf = __builtin_bit_cast(Operand, *reinterpret_cast<const float4_t*>(tile_base + ((cb & 1) ? k_odd : k_even) + 128 * (cb >> 1) + tile_bytes));
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) s[ct][t] = B::mma(kf, qf[ct][cb], s[ct][t]);
+      }
+    }
+    // ---- scale, mask (only where the tile crosses a row's limits), running maximum ----------
+    const bool whole = n0 + BN <= kv_len && n0 + BN - 1 <= wave_first_pos && (window <= 0 || n0 > wave_last_pos - window);
+    float alpha[CT];
+    Operand pf[CT][NKB];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      float mx = -INFINITY;
+      if (whole) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) mx = fmaxf(mx, s[ct][t][j]);
+      } else {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int n = n0 + 32 * (t >> 1) + 8 * g + 4 * (t & 1) + j;
+            const bool keep = row_ok[ct] && n < kv_len && n <= pos[ct] && (window <= 0 || n > pos[ct] - window);
+            s[ct][t][j] = keep ? s[ct][t][j] : -INFINITY;
+            mx = fmaxf(mx, s[ct][t][j]);
+          }
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, VELOX_WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, VELOX_WAVE));
+      const float m_new = fmaxf(m_i[ct], mx * scale_eff);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      alpha[ct] = (m_i[ct] == -INFINITY) ? 0.f : Softmax<T>::exp_of(m_i[ct] - m_safe);
+      float psum = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb) {
+        Vec16<T> packed;
+        T* e = reinterpret_cast<T*>(&packed.v);
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float p = Softmax<T>::exp_of(fmaf(s[ct][kb * 2 + u][j], scale_eff, -m_safe));
+            psum += p;
+            e[4 * u + j] = from_f32<T>(p);
+          }
+        pf[ct][kb] = __builtin_bit_cast(Operand, packed.v);
+      }
+      l_i[ct] = l_i[ct] * alpha[ct] + psum;
+      m_i[ct] = m_new;
+    }
+    // ---- O^T = O^T * alpha + V^T P^T --------------------------------------------------------
+    const bool tail = n0 + BN > kv_len;  // values beyond the sequence are whatever the page holds: they are zeroed
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      Operand vf[NKB];
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb) {
+        Vec16<T> x;
+        x.v = *reinterpret_cast<const float4_t*>(tile_base + (kb ? v_second : v_first) + 2048 * c);
+        if (tail) mask_tail(x, kv_len - (n0 + 32 * kb + 8 * g));
+        vf[kb] = __builtin_bit_cast(Operand, x.v);
+      }
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) acc_o[ct][c] = acc_o[ct][c] * alpha[ct];
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) acc_o[ct][c] = B::mma(vf[kb], pf[ct][kb], acc_o[ct][c]);
+    }
+  }
+
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    float l = l_i[ct];
+    l += __shfl_xor(l, 16, VELOX_WAVE);
+    l += __shfl_xor(l, 32, VELOX_WAVE);
+    if (!row_ok[ct]) continue;
+    const float inv = l > 0.f ? 1.f / l : 1.f;
+    const size_t token = (size_t)(q_start + tok[ct]);
+    if (splits == 1) {
+      T* dst = out + (token * nh + head[ct]) * D + 4 * g;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[16 * c + j] = from_f32<T>(acc_o[ct][c][j] * inv);
+      }
+    } else {
+      const size_t slot = ((size_t)split * total_tokens + token) * nh + head[ct];
+      float* dst = part_o + slot * D + 4 * g;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) *reinterpret_cast<float4_t*>(dst + 16 * c) = acc_o[ct][c] * inv;
+      if (g == 0) part_lse[slot] = l > 0.f ? m_i[ct] * Softmax<T>::LN_UNIT + logf(l) : -INFINITY;
+    }
+  }
+}
+
 // Zeroes the elements of a 4-key fragment whose key index is not below `valid`.
 __device__ __forceinline__ void mask_frag(Frag<float>& f, int valid) {
 #pragma unroll
@@ -825,6 +1125,11 @@ __global__ void merge_splits_kernel(const float* __restrict__ part_o, const floa
   }
 }
 
+// Which kernel portions of prompts take: 0 = chosen by shape; 1 = never the kernel with direct loads; 2 = that kernel
+// wherever it can run (for tests and measurements).
+static int portion_kernel_choice = 0;
+extern "C" void velox_attention_portion_kernel(int choice) { portion_kernel_choice = choice; }
+
 static int compute_units() {
   static int cached = 0;  // (the same value whichever thread gets here first)
   if (cached == 0) {
@@ -861,6 +1166,23 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
     merge_splits_kernel<T><<<dim3(total_tokens, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens, 0);
     return (int)hipGetLastError();
   }
+  // The kernel whose tiles reach LDS by direct loads: bfloat16, head sizes 64 and 128, pages of at least 8 tokens.
+  constexpr bool HAS_DIRECT = sizeof(T) == 2 && (D == 64 || D == 128);
+  const bool direct_ok = HAS_DIRECT && page_shift >= 3 && portion_kernel_choice != 1;
+  auto launch_direct = [&]() -> int {
+    if constexpr (HAS_DIRECT) {
+      dim3 grid((max_q_len * group + 127) / 128, nkv, num_seqs * splits);
+      direct_attention_kernel<2, 4><<<grid, 256, 0, stream>>>(
+          (const bf16_t*)qkv, qkv_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width, cu_q, kv_lens, (bf16_t*)out,
+          part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+    }
+    int status = (int)hipGetLastError();
+    if (status != 0 || splits == 1) return status;
+    merge_splits_kernel<T><<<dim3(total_tokens - first_token, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens,
+                                                                                                 first_token);
+    return (int)hipGetLastError();
+  };
+  if (direct_ok && portion_kernel_choice == 2 && max_q_len * group > 64) return launch_direct();
   // Eight waves per workgroup when bfloat16 portions are long enough to fill their rows and the step brings enough rows
   // that the larger workgroups still fill the GPU.  Behind few keys (a causal step's longest workgroup decides how
   // long the step takes, and short streams of keys leave LDS idle) a wave takes one row tile, 128 rows per workgroup;
@@ -879,6 +1201,10 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
       // over 8.  With fewer workgroups the eight waves hide more of a short stream's latency (12 heads over 2, two
       // sequences of 2,048: 61.5 / 75.8).
       const long long workgroups = (long long)grid.x * grid.y * grid.z;
+      // From 2.5 workgroups per compute unit on, the kernel with direct loads is the faster of the two with four waves of
+      // two row tiles (two prompts of 2,048 tokens 113 -> 107 us, four 205 -> 191, 28 heads over 4; 40 heads over 8: 149 ->
+      // 141 and 278 -> 255; one prompt of 2,048 tokens, 448 workgroups: 76 against 78 the other way).
+      if (direct_ok && rows >= 256 && workgroups * 2 >= 5LL * compute_units()) return launch_direct();
       if (rows >= 256 && workgroups * 4 >= 7LL * compute_units()) {
         paged_attention_kernel<T, BN, 2, 1, 4><<<grid, 256, 0, stream>>>(
             (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
@@ -889,6 +1215,10 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
             part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
       }
     } else {
+      // Behind many keys: 128 rows per workgroup with direct loads where that kernel runs (2,048 tokens behind 2,048 keys
+      // 163 -> 148 us, 4 x 512 tokens behind 7,680 keys 348 -> 335, 8,192 tokens from an empty cache 657 -> 641; with 12
+      // heads over 2 KV heads 4,096 tokens 160 -> 145, 8,192 tokens 322 -> 296), else 256 rows in eight waves.
+      if (direct_ok) return launch_direct();
       dim3 grid((rows + 255) / 256, nkv, num_seqs * splits);
       paged_attention_kernel<T, BN, WIDE, 1, 8><<<grid, 512, 0, stream>>>(
           (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,

@@ -147,6 +147,8 @@ class HipOps:
             lib.velox_paged_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P]
             lib.velox_paged_attention.restype = _I
             lib.velox_attention_head_dim.restype = _I
+            lib.velox_attention_portion_kernel.argtypes = [_I]
+            lib.velox_attention_portion_kernel.restype = None
             if lib.velox_attention_head_dim() != head_dim:
                 raise KernelError(f"attention library for head_dim={head_dim} reports {lib.velox_attention_head_dim()}")
             self._attention[head_dim] = lib
