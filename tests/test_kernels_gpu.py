@@ -81,7 +81,7 @@ def test_rmsnorm_eps_is_inside_the_root(ops):
     (torch.float32, torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16, torch.bfloat16),
     (torch.bfloat16, torch.float32, torch.bfloat16), (torch.bfloat16, torch.bfloat16, torch.float32),
 ])
-@pytest.mark.parametrize("m,n,k", [(1, 320, 96), (7, 263, 80), (65, 130, 150), (130, 64, 224), (3, 70, 37)])
+@pytest.mark.parametrize("m,n,k", [(1, 320, 96), (7, 263, 80), (65, 130, 150), (130, 64, 224), (3, 70, 37), (16, 1001, 3584), (9, 3584, 18944), (2, 13, 260)])
 def test_gemm_fma(ops, ref, a_dtype, w_dtype, out_dtype, m, n, k):
     x = rand((m, k), a_dtype, 5)
     w = rand((n, k), w_dtype, 6, 0.05)
@@ -89,7 +89,18 @@ def test_gemm_fma(ops, ref, a_dtype, w_dtype, out_dtype, m, n, k):
     for b in (None, bias):
         got = ops.gemm_fma(x, w, b, out_dtype)
         want = ref.linear(x, w, b, out_dtype)
+        if k >= 1024 and out_dtype == torch.float32:
+            # sums of thousands of terms round differently in every order of adding: the yardstick is the exact product
+            # (float64), and the kernel has to be as close to it as the library's float32 product is, within a factor of two
+            exact = x.double() @ w.double().T + (b.double() if b is not None else 0)
+            library = (x.float() @ w.float().T + (b if b is not None else 0)).double()
+            assert float((got.double() - exact).abs().max()) <= 2 * float((library - exact).abs().max()) + 1e-7
+            continue
         torch.testing.assert_close(got.float(), want.float(), **tol(out_dtype))
+    if m <= 16 and m > 1:
+        # few rows take a kernel of their own: a row's sum depends on that row alone, to the bit, whatever else is in the batch
+        alone = ops.gemm_fma(x[m - 1:].contiguous(), w, None, out_dtype)
+        assert torch.equal(alone[0], ops.gemm_fma(x, w, None, out_dtype)[m - 1])
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 320, 96), (8, 152064 // 8, 512), (64, 1000, 3584), (300, 4608, 3584)])

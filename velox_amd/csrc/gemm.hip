@@ -102,6 +102,64 @@ __global__ void __launch_bounds__(256) gemm_fma_kernel(const TA* __restrict__ a,
   }
 }
 
+// The same product for few rows (M <= 16), where it is bound by reading W once: the decode steps of a float32 run.
+// A wave owns SKINNY_ROWS consecutive rows of W and all of K; lane l takes indices 4 l .. 4 l + 3 of every block of
+// 256, so a wave's load of a row's block is one contiguous kilobyte (float32) and the activations (from L2) are used
+// for SKINNY_ROWS rows of W at once.  A lane adds its terms in the order of k, the 64 lanes' sums are added in a fixed
+// tree: an element's sum depends on nothing but its own row of A and row of W.
+#define SKINNY_ROWS 4
+
+template <typename TA, typename TW, typename TO, int MT>
+__global__ void __launch_bounds__(256) skinny_fma_kernel(const TA* __restrict__ a, const TW* __restrict__ w, const float* __restrict__ bias,
+                                                         TO* __restrict__ out, int m, int n, int k) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n0 = (blockIdx.x * 4 + wave) * SKINNY_ROWS;
+  if (n0 >= n) return;
+  float acc[SKINNY_ROWS][MT];
+#pragma unroll
+  for (int r = 0; r < SKINNY_ROWS; ++r)
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[r][i] = 0.f;
+  size_t w_off[SKINNY_ROWS], a_off[MT];
+#pragma unroll
+  for (int r = 0; r < SKINNY_ROWS; ++r) w_off[r] = (size_t)(n0 + r < n ? n0 + r : n0) * k;  // (a row beyond N: row n0 again, never stored)
+#pragma unroll
+  for (int i = 0; i < MT; ++i) a_off[i] = (size_t)(i < m ? i : 0) * k;
+  for (int k0 = 4 * lane; k0 < k; k0 += 256) {
+    float wv[SKINNY_ROWS][4], av[MT][4];
+#pragma unroll
+    for (int r = 0; r < SKINNY_ROWS; ++r) load4<TW>(w, w_off[r], k0, k, true, true, wv[r]);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) load4<TA>(a, a_off[i], k0, k, true, true, av[i]);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int r = 0; r < SKINNY_ROWS; ++r)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) acc[r][i] = fmaf(av[i][e], wv[r][e], acc[r][i]);
+  }
+#pragma unroll
+  for (int r = 0; r < SKINNY_ROWS; ++r)
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const float total = wave_sum(acc[r][i]);
+      if (lane == 0 && i < m && n0 + r < n) out[(size_t)i * n + n0 + r] = from_f32<TO>(total + (bias ? bias[n0 + r] : 0.f));
+    }
+}
+
+template <typename TA, typename TW, typename TO>
+static void launch_skinny_fma(const void* a, const void* w, const float* bias, void* out, int m, int n, int k, hipStream_t stream) {
+  const int waves = (n + SKINNY_ROWS - 1) / SKINNY_ROWS;
+  dim3 grid((waves + 3) / 4);
+#define SKINNY(MT) skinny_fma_kernel<TA, TW, TO, MT><<<grid, 256, 0, stream>>>((const TA*)a, (const TW*)w, bias, (TO*)out, m, n, k)
+  if (m <= 1) SKINNY(1);
+  else if (m <= 2) SKINNY(2);
+  else if (m <= 4) SKINNY(4);
+  else if (m <= 8) SKINNY(8);
+  else SKINNY(16);
+#undef SKINNY
+}
+
 extern "C" int velox_gemm_fma(const void* a, const void* w, const float* bias, void* out, int m, int n, int k,
                               int a_dtype, int w_dtype, int out_dtype, hipStream_t stream) {
   if (m <= 0 || n <= 0) return 0;
@@ -112,6 +170,20 @@ extern "C" int velox_gemm_fma(const void* a, const void* w, const float* bias, v
 #define LAUNCH(TA, TW, TO) \
   gemm_fma_kernel<TA, TW, TO><<<grid, 256, 0, stream>>>((const TA*)a, (const TW*)w, bias, (TO*)out, m, n, k, a_vec, w_vec)
   const int key = a_dtype * 4 + w_dtype * 2 + out_dtype;
+  if (m <= 16 && a_vec && w_vec) {  // (rows of whole 16-byte pieces: every load is a vector)
+    switch (key) {
+      case 0: launch_skinny_fma<float, float, float>(a, w, bias, out, m, n, k, stream); break;
+      case 1: launch_skinny_fma<float, float, bf16_t>(a, w, bias, out, m, n, k, stream); break;
+      case 2: launch_skinny_fma<float, bf16_t, float>(a, w, bias, out, m, n, k, stream); break;
+      case 3: launch_skinny_fma<float, bf16_t, bf16_t>(a, w, bias, out, m, n, k, stream); break;
+      case 4: launch_skinny_fma<bf16_t, float, float>(a, w, bias, out, m, n, k, stream); break;
+      case 5: launch_skinny_fma<bf16_t, float, bf16_t>(a, w, bias, out, m, n, k, stream); break;
+      case 6: launch_skinny_fma<bf16_t, bf16_t, float>(a, w, bias, out, m, n, k, stream); break;
+      case 7: launch_skinny_fma<bf16_t, bf16_t, bf16_t>(a, w, bias, out, m, n, k, stream); break;
+      default: return -1;
+    }
+    VELOX_RETURN_LAUNCH_STATUS();
+  }
   switch (key) {
     case 0: LAUNCH(float, float, float); break;
     case 1: LAUNCH(float, float, bf16_t); break;
