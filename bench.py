@@ -33,6 +33,14 @@ QWEN25_7B = {
     "intermediate_size": 18944, "vocab_size": 152064, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
     "tie_word_embeddings": False, "use_sliding_window": False, "max_position_embeddings": 32768,
 }
+# the other two shapes the reference is quoted on (--shape): the headline stays the 7B shape
+SHAPES = {
+    "7b": ("Qwen2.5-7B shape", QWEN25_7B),
+    "1.5b": ("Qwen2.5-1.5B shape", dict(QWEN25_7B, hidden_size=1536, num_attention_heads=12, num_key_value_heads=2, intermediate_size=8960,
+                                          vocab_size=151936, tie_word_embeddings=True)),
+    "32b": ("Qwen2.5-32B shape", dict(QWEN25_7B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=40, num_key_value_heads=8,
+                                        intermediate_size=27648, rms_norm_eps=1e-6)),
+}
 
 
 def linear_params_per_layer(c):
@@ -175,6 +183,40 @@ def time_prefill(engine, vocab, tokens, repeats=3, seed=1):
     return sum(times) / len(times), min(times)
 
 
+def far_points(model_config, layers, args) -> dict:
+    """Sizes beyond the headline's, each with its share of the roofline: decode behind a long context, a long prefill,
+    and the true 32-bit path's decode step.  Engines are built one after the other (the first is given up)."""
+    import gc
+
+    import torch
+
+    out = {}
+    vocab = model_config["vocab_size"]
+    elem = 2 if args.dtype == "bf16" else 4
+    gc.collect()
+    torch.cuda.empty_cache()
+    long_context = 32256
+    far = make_engine(model_config, args.dtype, 8, long_context, 8192, not args.no_graphs)
+    for batch in (1, 8):
+        each_s, mean_context = time_decode(far, vocab, batch, long_context, 16, 4)
+        out[f"decode_b{batch}_ctx{long_context}"] = round(batch / each_s, 2)
+        out[f"decode_b{batch}_ctx{long_context}_frac"] = round(decode_bytes(model_config, layers, batch, mean_context, elem) / each_s / 1e9 / PEAK_HBM_GBS, 4)
+    long_s, _ = time_prefill(far, vocab, 8192, repeats=2)
+    out["prefill_8192_tok_s"] = round(8192 / long_s, 1)
+    out["prefill_8192_frac"] = round(prefill_flops(model_config, layers, 8192) / long_s / PEAK_FLOPS[args.dtype], 4)
+    far.abort_all()
+    del far
+    gc.collect()
+    torch.cuda.empty_cache()
+    if args.dtype == "bf16":
+        exact = make_engine(model_config, "fp32", 8, args.context, 512, not args.no_graphs)
+        each_s, mean_context = time_decode(exact, vocab, 8, args.context, 16, 4)
+        out["decode_b8_fp32"] = round(8 / each_s, 2)
+        out["decode_b8_fp32_frac"] = round(decode_bytes(model_config, layers, 8, mean_context, 4) / each_s / 1e9 / PEAK_HBM_GBS, 4)
+        exact.abort_all()
+    return out
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -189,6 +231,9 @@ def main() -> int:
     parser.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     parser.add_argument("--no-tune", action="store_true", help="do not let the matrix library pick its kernels for the prefill shapes")
     parser.add_argument("--no-probes", action="store_true", help="skip the probes of what the card delivers (streaming read, bfloat16 matrix instructions)")
+    parser.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes: the headline is 7b; 1.5b and 32b are the reference's other two")
+    parser.add_argument("--far", action="store_true",
+                        help="further sizes under `points`: decode at batch 1 and 8 behind 32,256 tokens, a prefill of 8,192 tokens, and a decode step of a true float32 run (batch 8)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine (single-GPU tier)")
@@ -196,7 +241,8 @@ def main() -> int:
 
     import torch
 
-    model_config = dict(QWEN25_7B)
+    shape_name, shape = SHAPES[args.shape]
+    model_config = dict(shape)
     full_layers = model_config["num_hidden_layers"]
     layers = args.layers or full_layers
     model_config["num_hidden_layers"] = layers
@@ -247,7 +293,7 @@ def main() -> int:
         "dtype": args.dtype,
         "data": "synthetic: random weights N(0,0.02), uniform random token ids",
         "config": {
-            "model": "Qwen2.5-7B shape", "layers": layers, "layers_full": full_layers,
+            "model": shape_name, "layers": layers, "layers_full": full_layers,
             "hidden": model_config["hidden_size"], "heads": model_config["num_attention_heads"],
             "kv_heads": model_config["num_key_value_heads"], "head_dim": model_config["hidden_size"] // model_config["num_attention_heads"],
             "intermediate": model_config["intermediate_size"], "vocab": vocab,
@@ -274,6 +320,10 @@ def main() -> int:
         }
         if args.dtype == "bf16":
             result["probes"]["prefill_frac_of_mfma"] = round(flops / prefill_s / 1e12 / mfma_tflops, 4)
+    if args.far:
+        engine.abort_all()
+        engine = None  # (its weights and cache are given up before the next engines are built)
+        points.update(far_points(model_config, layers, args))
     print(json.dumps(result))
     return 0
 
