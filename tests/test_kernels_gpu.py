@@ -612,19 +612,21 @@ def test_paged_attention_with_tiles_loaded_straight_into_lds(ops, ref, nh, nkv, 
     want = _run_attention(ref, case, nh, nkv, d, page, window=window)
     try:
         results = {}
-        for choice in (1, 2):
+        for choice in (1, 2, 3):  # (the kernels it stands in for; direct loads; direct loads with two sets of waves)
             lib.velox_attention_portion_kernel(choice)
             results[choice] = _run_attention(ops, case, nh, nkv, d, page, window=window)
             torch.testing.assert_close(results[choice], want, **tolerance)
             assert torch.equal(_run_attention(ops, dirty, nh, nkv, d, page, window=window), results[choice])
-        assert not torch.equal(results[1], results[2])  # two kernels did run (they add a row's keys in different orders)
-        # split keys (few tokens behind many keys) through the same kernel, and the partial results merged
-        lib.velox_attention_portion_kernel(2)
+        # three kernels did run (they add a row's keys in different orders)
+        assert not torch.equal(results[1], results[2]) and not torch.equal(results[2], results[3])
+        # split keys (few tokens behind many keys) through the same kernels, and the partial results merged
         far = _attention_case(torch.bfloat16, nh, nkv, d, page, [(150, 4400), (90, 90), (2, 4200)], seed=d + nh + 8)
         workspace = Workspace(torch.device("cuda"))
-        for splits in (1, 3, 4):
-            got = _run_attention(ops, far, nh, nkv, d, page, window=window, splits=splits, workspace=workspace)
-            torch.testing.assert_close(got, _run_attention(ref, far, nh, nkv, d, page, window=window), **tolerance)
+        for choice in (2, 3):
+            lib.velox_attention_portion_kernel(choice)
+            for splits in (1, 3, 4):
+                got = _run_attention(ops, far, nh, nkv, d, page, window=window, splits=splits, workspace=workspace)
+                torch.testing.assert_close(got, _run_attention(ref, far, nh, nkv, d, page, window=window), **tolerance)
     finally:
         lib.velox_attention_portion_kernel(0)
 

@@ -31,6 +31,12 @@
 #endif
 
 constexpr int D = VELOX_HEAD_DIM;
+#ifndef VELOX_PV_AHEAD
+#define VELOX_PV_AHEAD 1
+#endif
+#ifndef VELOX_QK_AHEAD
+#define VELOX_QK_AHEAD 0
+#endif
 static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple of 16 between 16 and 256");
 
 template <typename T> struct Frag;
@@ -566,8 +572,14 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
 // of keys 8 g .. 8 g + 7 of the block: eight consecutive keys, which is one 16-byte piece of a V^T row in its natural
 // order.  (The general kernel reorders V^T instead, in pieces of 8 bytes; a direct load cannot.)  For such a row of K
 // f(k) is i & 7 for lane i: a constant of the lane.
-template <int CT, int WAVES>
-__global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, WAVES > 4 ? 4 : 2))) direct_attention_kernel(
+__device__ __attribute__((aligned(16))) const unsigned int zero_piece[4] = {0u, 0u, 0u, 0u};
+
+// KSPLIT = 2: two sets of WAVES waves own the same rows and take the key tiles alternately, each set with tile buffers of
+// its own; at the end the second set hands its running (maximum, sum, output) to the first through LDS.  The longest
+// workgroups of a causal step, the rows at the end of a prompt, which decide how long the step takes, then walk half
+// as many tiles one after the other.
+template <int CT, int WAVES, int KSPLIT = 1>
+__global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_waves_per_eu(2, 2))) direct_attention_kernel(
     const bf16_t* __restrict__ qkv, int qkv_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
@@ -584,10 +596,15 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
   static_assert(LOADS % WAVES == 0, "every wave issues the same number of loads");
   constexpr int LPW = LOADS / WAVES;
   constexpr int ROWS_PER_BLOCK = 16 * WAVES * CT;
-  __shared__ __attribute__((aligned(1024))) char smem[2][2 * TILE_BYTES];
+  constexpr int SETW = 64 * WAVES;                  // threads of a set of waves
+  constexpr int MERGE_BYTES = KSPLIT > 1 ? 4 * SETW * CT * (4 * NC + 2) : 0;  // what the second set hands over at the end
+  static_assert(MERGE_BYTES <= KSPLIT * 4 * TILE_BYTES, "the hand-over fits into the tile buffers");
+  __shared__ __attribute__((aligned(1024))) char smem_all[KSPLIT][2][2 * TILE_BYTES];
   __shared__ int page_ids[PREFILL_PAGE_IDS];
 
-  const int tid = threadIdx.x;
+  const int set = KSPLIT > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x / SETW) : 0;  // which set of waves
+  const int tid = KSPLIT > 1 ? threadIdx.x % SETW : threadIdx.x;                         // thread within the set
+  char (*const smem)[2 * TILE_BYTES] = smem_all[set];
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 4, i = lane & 15;
   const int group = nh / nkv;
@@ -657,7 +674,7 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
   int first_page = (n_begin + tile_lo * BN) >> page_shift;
   auto load_page_ids = [&]() {
     const int num_pages = last_page - first_page + 1;
-    for (int p = tid; p < num_pages && p < PREFILL_PAGE_IDS; p += 64 * WAVES) page_ids[p] = table[first_page + p];
+    for (int p = threadIdx.x; p < num_pages && p < PREFILL_PAGE_IDS; p += SETW * KSPLIT) page_ids[p] = table[first_page + p];
   };
   load_page_ids();
   auto page_of = [&](int n) -> size_t { return (size_t)page_ids[(n >> page_shift) - first_page]; };
@@ -699,16 +716,18 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
       int nk = n0 + k_key[m];
       nk = nk < kv_len ? nk : kv_len - 1;  // (a key beyond the sequence: any valid address; its scores are masked)
       const T* src = k_cache + (((page_of(nk) * nkv + kvh) << page_shift) + (nk & (page_size - 1))) * D + k_col[m];
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(k_dst + 1024 * (wave + WAVES * m)), 16, 0, 0);
+      load_to_lds_16(src, k_dst + 1024 * (wave + WAVES * m));
     }
 #pragma unroll
     for (int m = 0; m < LPW; ++m) {
-      int nv = n0 + v_key;
-      nv = nv < kv_len ? nv : (kv_len - 1) & ~7;
-      const T* src = v_cache + (((page_of(nv) * nkv + kvh) * D + v_chan[m]) << page_shift) + (nv & (page_size - 1));
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(v_dst + 1024 * (wave + WAVES * m)), 16, 0, 0);
+      // Values beyond the sequence are whatever the page holds, and even a probability of zero times an infinity is
+      // no zero: a piece that lies wholly beyond the sequence is taken from a piece of zeros instead (the piece that the
+      // sequence ends in is cleaned up in LDS, below)
+      const int nv = n0 + v_key;
+      const bool beyond = nv >= kv_len;
+      const int nc = beyond ? (kv_len - 1) & ~7 : nv;
+      const T* src = v_cache + (((page_of(nc) * nkv + kvh) * D + v_chan[m]) << page_shift) + (nc & (page_size - 1));
+      load_to_lds_16(beyond ? reinterpret_cast<const T*>(zero_piece) : src, v_dst + 1024 * (wave + WAVES * m));
     }
   };
 
@@ -721,39 +740,73 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
   const int v_row_bytes = TILE_BYTES + i * 128 + 16 * (g ^ (i & 3));
   const int v_first = v_row_bytes + 64 * h, v_second = v_row_bytes + 64 * (1 - h);       // kb = 0 / 1
 
+  // (the queries have arrived before the loop, said in a way the compiler sees: it would otherwise wait for them, and with
+  // them for every load in flight, at their first use in every round of the loop)
+  __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();  // page ids are in place
-  if (tile_lo < tile_hi) issue(n_begin + tile_lo * BN, 0);
+  // round `it` covers tiles tile_lo + it * KSPLIT .. + KSPLIT - 1, one per set (the last round may leave a set without one)
+  const int rounds = tile_hi > tile_lo ? (tile_hi - tile_lo + KSPLIT - 1) / KSPLIT : 0;
+  if (tile_lo + set < tile_hi) issue(n_begin + (tile_lo + set) * BN, 0);
   int buffer = 0;
-  for (int tile = tile_lo; tile < tile_hi; ++tile, buffer ^= 1) {
+  for (int it = 0; it < rounds; ++it, buffer ^= 1) {
+    const int tile = tile_lo + it * KSPLIT + set;
+    const bool have_tile = KSPLIT == 1 || tile < tile_hi;
     const int n0 = n_begin + tile * BN;
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces of the tile have landed
+    wait_for_loads<0>();                  // this wave's pieces of the tile have landed
     __syncthreads();                      // everybody's have, and everybody is done with the other buffer
-    if (tile + 1 < tile_hi) {
-      const int next = n0 + BN;
-      if (((next + BN - 1) >> page_shift) - first_page >= PREFILL_PAGE_IDS) {  // the same for every thread
-        first_page = next >> page_shift;
+    if (it + 1 < rounds) {
+      const int next_first = n_begin + (tile_lo + (it + 1) * KSPLIT) * BN;  // first key of the next round's tiles
+      if (((next_first + KSPLIT * BN - 1) >> page_shift) - first_page >= PREFILL_PAGE_IDS) {  // the same for every thread
+        first_page = next_first >> page_shift;
         __syncthreads();
         load_page_ids();
         __syncthreads();
       }
-      issue(next, buffer ^ 1);
+      if (tile + KSPLIT < tile_hi) issue(n0 + KSPLIT * BN, buffer ^ 1);
     }
+    // the sequence's last tile, if it is one of this round's and the sequence ends inside a piece of eight keys (the same
+    // answer for every thread; once per sequence and workgroup): what follows the last key in that piece is zeroed in LDS
+    const int last_tile = (kv_len - 1 - n_begin) / BN;
+    if ((kv_len & 7) != 0 && last_tile >= tile_lo + it * KSPLIT && last_tile < tile_lo + (it + 1) * KSPLIT && last_tile < tile_hi) {
+      if (tile == last_tile) {
+        const int piece = (kv_len - n0) >> 3, valid = (kv_len - n0) & 7;
+        for (int channel = tid; channel < D; channel += SETW) {
+          float4_t* const at = reinterpret_cast<float4_t*>(smem[buffer] + TILE_BYTES + channel * 128 + 16 * (piece ^ (channel & 7)));
+          Vec16<T> x;
+          x.v = *at;
+          mask_tail(x, valid);
+          *at = x.v;
+        }
+      }
+      __syncthreads();
+    }
+    if (!have_tile) continue;
     if (n0 > wave_last_pos) continue;  // nothing this wave may read
     const char* const tile_base = smem[buffer];
 
     // ---- S^T = K Q^T: tile t = 2 b + u of the 64 keys ----------------------------------------
     float4_t s[CT][NT];
+    constexpr int QK_AHEAD = VELOX_QK_AHEAD;
+    Operand kf[QK_AHEAD + 1][NQB];
+    auto read_keys = [&](int t, Operand (&into)[NQB]) {
+      const int tile_bytes = (32 * (t >> 1) + 4 * (t & 1)) * (2 * D);
+#pragma unroll
+      for (int cb = 0; cb < NQB; ++cb)
+        into[cb] = __builtin_bit_cast(Operand, *reinterpret_cast<const float4_t*>(tile_base + ((cb & 1) ? k_odd : k_even) + 128 * (cb >> 1) + tile_bytes));
+    };
+#pragma unroll
+    for (int a = 0; a < QK_AHEAD; ++a) read_keys(a, kf[a]);
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      const int tile_bytes = (32 * (t >> 1) + 4 * (t & 1)) * (2 * D);
+      if (QK_AHEAD == 0) read_keys(t, kf[0]);
+      else if (t + QK_AHEAD < NT) read_keys(t + QK_AHEAD, kf[(t + QK_AHEAD) % (QK_AHEAD + 1)]);
+      if constexpr (QK_AHEAD > 0) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) s[ct][t] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int cb = 0; cb < NQB; ++cb) {
-        const Operand kf = __builtin_bit_cast(Operand, *reinterpret_cast<const float4_t*>(tile_base + ((cb & 1) ? k_odd : k_even) + 128 * (cb >> 1) + tile_bytes));
+      for (int cb = 0; cb < NQB; ++cb)
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) s[ct][t] = B::mma(kf, qf[ct][cb], s[ct][t]);
-      }
+        for (int ct = 0; ct < CT; ++ct) s[ct][t] = B::mma(kf[t % (QK_AHEAD + 1)][cb], qf[ct][cb], s[ct][t]);
     }
     // ---- scale, mask (only where the tile crosses a row's limits), running maximum ----------
     const bool whole = n0 + BN <= kv_len && n0 + BN - 1 <= wave_first_pos && (window <= 0 || n0 > wave_last_pos - window);
@@ -802,23 +855,54 @@ __global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu
       m_i[ct] = m_new;
     }
     // ---- O^T = O^T * alpha + V^T P^T --------------------------------------------------------
-    const bool tail = n0 + BN > kv_len;  // values beyond the sequence are whatever the page holds: they are zeroed
+    constexpr int AHEAD = VELOX_PV_AHEAD;  // channel tiles whose operands are in flight ahead of the one being multiplied
+    Operand vf[AHEAD + 1][NKB];
+    auto read_values = [&](int c, Operand (&into)[NKB]) {
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb) into[kb] = __builtin_bit_cast(Operand, *reinterpret_cast<const float4_t*>(tile_base + (kb ? v_second : v_first) + 2048 * c));
+    };
+#pragma unroll
+    for (int a = 0; a < AHEAD; ++a) read_values(a, vf[a]);
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
-      Operand vf[NKB];
-#pragma unroll
-      for (int kb = 0; kb < NKB; ++kb) {
-        Vec16<T> x;
-        x.v = *reinterpret_cast<const float4_t*>(tile_base + (kb ? v_second : v_first) + 2048 * c);
-        if (tail) mask_tail(x, kv_len - (n0 + 32 * kb + 8 * g));
-        vf[kb] = __builtin_bit_cast(Operand, x.v);
-      }
+      if (c + AHEAD < NC) read_values(c + AHEAD, vf[(c + AHEAD) % (AHEAD + 1)]);
+      if constexpr (AHEAD > 0) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) acc_o[ct][c] = acc_o[ct][c] * alpha[ct];
 #pragma unroll
       for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) acc_o[ct][c] = B::mma(vf[kb], pf[ct][kb], acc_o[ct][c]);
+        for (int ct = 0; ct < CT; ++ct) acc_o[ct][c] = B::mma(vf[c % (AHEAD + 1)][kb], pf[ct][kb], acc_o[ct][c]);
+    }
+  }
+
+  if constexpr (KSPLIT > 1) {
+    // the second set's state goes through LDS (the tiles are no longer needed) and is folded into the first set's
+    __syncthreads();
+    float4_t* const hand_acc = reinterpret_cast<float4_t*>(&smem_all[0][0][0]);
+    float* const hand_ml = reinterpret_cast<float*>(&smem_all[0][0][0]) + SETW * CT * NC * 4;
+    if (set == 1) {
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) hand_acc[(ct * NC + c) * SETW + tid] = acc_o[ct][c];
+        hand_ml[ct * SETW + tid] = m_i[ct];
+        hand_ml[(CT + ct) * SETW + tid] = l_i[ct];
+      }
+    }
+    __syncthreads();
+    if (set == 1) return;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      const float m_other = hand_ml[ct * SETW + tid], l_other = hand_ml[(CT + ct) * SETW + tid];
+      const float m_new = fmaxf(m_i[ct], m_other);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float mine = (m_i[ct] == -INFINITY) ? 0.f : Softmax<T>::exp_of(m_i[ct] - m_safe);
+      const float theirs = (m_other == -INFINITY) ? 0.f : Softmax<T>::exp_of(m_other - m_safe);
+      l_i[ct] = l_i[ct] * mine + l_other * theirs;
+      m_i[ct] = m_new;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) acc_o[ct][c] = acc_o[ct][c] * mine + hand_acc[(ct * NC + c) * SETW + tid] * theirs;
     }
   }
 
@@ -1126,7 +1210,7 @@ __global__ void merge_splits_kernel(const float* __restrict__ part_o, const floa
 }
 
 // Which kernel portions of prompts take: 0 = chosen by shape; 1 = never the kernel with direct loads; 2 = that kernel
-// wherever it can run (for tests and measurements).
+// wherever it can run, 3 = the same with two sets of waves (for tests and measurements).
 static int portion_kernel_choice = 0;
 extern "C" void velox_attention_portion_kernel(int choice) { portion_kernel_choice = choice; }
 
@@ -1169,12 +1253,17 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
   // The kernel whose tiles reach LDS by direct loads: bfloat16, head sizes 64 and 128, pages of at least 8 tokens.
   constexpr bool HAS_DIRECT = sizeof(T) == 2 && (D == 64 || D == 128);
   const bool direct_ok = HAS_DIRECT && page_shift >= 3 && portion_kernel_choice != 1;
-  auto launch_direct = [&]() -> int {
+  auto launch_direct = [&](bool two_sets = false) -> int {
     if constexpr (HAS_DIRECT) {
       dim3 grid((max_q_len * group + 127) / 128, nkv, num_seqs * splits);
-      direct_attention_kernel<2, 4><<<grid, 256, 0, stream>>>(
-          (const bf16_t*)qkv, qkv_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width, cu_q, kv_lens, (bf16_t*)out,
-          part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+      if (two_sets)
+        direct_attention_kernel<2, 4, 2><<<grid, 512, 0, stream>>>(
+            (const bf16_t*)qkv, qkv_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width, cu_q, kv_lens, (bf16_t*)out,
+            part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+      else
+        direct_attention_kernel<2, 4><<<grid, 256, 0, stream>>>(
+            (const bf16_t*)qkv, qkv_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width, cu_q, kv_lens, (bf16_t*)out,
+            part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
     }
     int status = (int)hipGetLastError();
     if (status != 0 || splits == 1) return status;
@@ -1182,7 +1271,20 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
                                                                                                  first_token);
     return (int)hipGetLastError();
   };
-  if (direct_ok && portion_kernel_choice == 2 && max_q_len * group > 64) return launch_direct();
+  if (direct_ok && portion_kernel_choice >= 2 && max_q_len * group > 64) return launch_direct(portion_kernel_choice == 3);
+  if (direct_ok && max_q_len * group > 64) {
+    // Measured on MI355X over prompts and portions of 128 to 8,192 tokens behind up to 30,000 keys, with 28 heads over 4,
+    // 12 over 2 and 40 over 8 (us, the kernels below / direct loads / direct loads with two sets of waves).  From 1.5
+    // workgroups of 128 rows per compute unit on, the kernel with direct loads: 2 x 2,048 tokens 110 / 103 / 115, 4 x 512
+    // behind 512 keys 51.8 / 46.9 / 53.4, 8,192 tokens 631 / 608 / 618.  With fewer, down to 0.6 per compute unit and when the
+    // keys are not split over workgroups, two sets of waves share a workgroup's keys, which fills the compute units
+    // that one set would leave half empty: with 12 heads over 2, 4 x 512 tokens behind 1,536 keys 80.0 / 65.3 / 49.6, 16 x 128
+    // behind 1,920 keys 86.2 / 65.7 / 50.8, 4,096 tokens 123 / 123 / 89.9; with 28 over 4, 1,024 tokens 36.1 / 37.7 / 30.3 and
+    // 2,048 tokens 75.6 / 69.6 / 67.4.  Fewer workgroups still stay with the kernels below (512 tokens: 16.4 / 23.0 / 19.5).
+    const long long workgroups = (long long)((max_q_len * group + 127) / 128) * nkv * num_seqs * splits;
+    if (workgroups * 2 > 3LL * compute_units()) return launch_direct(false);
+    if (splits == 1 && workgroups * 5 >= 3LL * compute_units()) return launch_direct(true);
+  }
   // Eight waves per workgroup when bfloat16 portions are long enough to fill their rows and the step brings enough rows
   // that the larger workgroups still fill the GPU.  Behind few keys (a causal step's longest workgroup decides how
   // long the step takes, and short streams of keys leave LDS idle) a wave takes one row tile, 128 rows per workgroup;
@@ -1201,10 +1303,6 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
       // over 8.  With fewer workgroups the eight waves hide more of a short stream's latency (12 heads over 2, two
       // sequences of 2,048: 61.5 / 75.8).
       const long long workgroups = (long long)grid.x * grid.y * grid.z;
-      // From 2.5 workgroups per compute unit on, the kernel with direct loads is the faster of the two with four waves of
-      // two row tiles (two prompts of 2,048 tokens 113 -> 107 us, four 205 -> 191, 28 heads over 4; 40 heads over 8: 149 ->
-      // 141 and 278 -> 255; one prompt of 2,048 tokens, 448 workgroups: 76 against 78 the other way).
-      if (direct_ok && rows >= 256 && workgroups * 2 >= 5LL * compute_units()) return launch_direct();
       if (rows >= 256 && workgroups * 4 >= 7LL * compute_units()) {
         paged_attention_kernel<T, BN, 2, 1, 4><<<grid, 256, 0, stream>>>(
             (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
@@ -1215,10 +1313,6 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
             part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
       }
     } else {
-      // Behind many keys: 128 rows per workgroup with direct loads where that kernel runs (2,048 tokens behind 2,048 keys
-      // 163 -> 148 us, 4 x 512 tokens behind 7,680 keys 348 -> 335, 8,192 tokens from an empty cache 657 -> 641; with 12
-      // heads over 2 KV heads 4,096 tokens 160 -> 145, 8,192 tokens 322 -> 296), else 256 rows in eight waves.
-      if (direct_ok) return launch_direct();
       dim3 grid((rows + 255) / 256, nkv, num_seqs * splits);
       paged_attention_kernel<T, BN, WIDE, 1, 8><<<grid, 512, 0, stream>>>(
           (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,

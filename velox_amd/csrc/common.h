@@ -52,4 +52,18 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return total;
 }
 
+// 16 bytes per lane from global memory straight into LDS: lane l's piece lands at dst + 16 l, so one instruction fills a
+// contiguous kilobyte.  `dst` must be the same for the whole wave.  Written as assembly on purpose: of a load that the
+// compiler knows to write LDS it assumes that any later LDS read may touch what is still in flight, and waits for ALL
+// outstanding loads before the first read, which undoes a load issued ahead into another buffer.  The caller orders
+// things itself: `wait_for_loads<N>()` (at most N of the wave's loads still in flight) and a barrier before the reads.
+__device__ __forceinline__ void load_to_lds_16(const void* src, void* dst) {
+  const uint32_t at = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)dst;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(at), "v"(src) : "memory", "m0");
+}
+template <int N> __device__ __forceinline__ void wait_for_loads() {
+  static_assert(N >= 0 && N < 64, "the counter of loads in flight has six bits");
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
 #define VELOX_RETURN_LAUNCH_STATUS() return (int)hipGetLastError()
