@@ -627,6 +627,22 @@ def test_paged_attention_with_tiles_loaded_straight_into_lds(ops, ref, nh, nkv, 
             for splits in (1, 3, 4):
                 got = _run_attention(ops, far, nh, nkv, d, page, window=window, splits=splits, workspace=workspace)
                 torch.testing.assert_close(got, _run_attention(ref, far, nh, nkv, d, page, window=window), **tolerance)
+        # Scores that climb along the sequence, slowly (a row's best score moves up a little with every tile, so the
+        # reference of its exponents lags behind and catches up every few tiles) and in jumps (far above everything seen):
+        # the kernels with direct loads keep a reference that need not be the maximum
+        climbing = _attention_case(torch.bfloat16, nh, nkv, d, page, [(900, 900), (400, 1100)], seed=d + nh + 9)
+        direction = torch.randn(d, generator=torch.Generator().manual_seed(3))
+        direction = direction / direction.norm()
+        tables = climbing["tables"].cpu()
+        for b, kv_len in enumerate((900, 1100)):
+            for n in range(kv_len):
+                height = 0.07 * n + (40.0 if n in (300, 301, 777) else 0.0)
+                climbing["k_cache"][int(tables[b, n // page]), :, n % page, :] += (height * direction).to(torch.bfloat16).cuda()
+        climbing["qkv"][:, : nh * d] = (climbing["qkv"][:, : nh * d].float() * 0.3 + (direction * math.sqrt(d)).repeat(nh).cuda()).to(torch.bfloat16)
+        want = _run_attention(ref, climbing, nh, nkv, d, page, window=window)
+        for choice in (1, 2, 3):
+            lib.velox_attention_portion_kernel(choice)
+            torch.testing.assert_close(_run_attention(ops, climbing, nh, nkv, d, page, window=window), want, **tolerance)
     finally:
         lib.velox_attention_portion_kernel(0)
 

@@ -833,9 +833,17 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16, VELOX_WAVE));
       mx = fmaxf(mx, __shfl_xor(mx, 32, VELOX_WAVE));
-      const float m_new = fmaxf(m_i[ct], mx * scale_eff);
+      // The reference of a row's exponents need not be its maximum: any number the scores do not exceed by much will do,
+      // the sums and the output are relative to it all the same and the final division takes it out.  It is moved (and
+      // everything gathered so far rescaled) only when a score lies more than REFERENCE_SLACK above it, in units of the
+      // exponent (powers of two): probabilities then stay below 2^REFERENCE_SLACK, far inside the range of both number
+      // formats, and after a row's first tile the rescaling is the exception.
+      constexpr float REFERENCE_SLACK = 8.f;
+      const float top = mx * scale_eff;
+      const bool stays = top - m_i[ct] <= REFERENCE_SLACK;  // (false while the row has seen no key: -inf)
+      const float m_new = stays ? m_i[ct] : top;
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      alpha[ct] = (m_i[ct] == -INFINITY) ? 0.f : Softmax<T>::exp_of(m_i[ct] - m_safe);
+      alpha[ct] = stays ? 1.f : ((m_i[ct] == -INFINITY) ? 0.f : Softmax<T>::exp_of(m_i[ct] - m_safe));
       float psum = 0.f;
 #pragma unroll
       for (int kb = 0; kb < NKB; ++kb) {
@@ -863,12 +871,21 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     };
 #pragma unroll
     for (int a = 0; a < AHEAD; ++a) read_values(a, vf[a]);
+    // The kernel is bound by the vector instructions it issues, and the output's rescaling is 64 of a tile's 400: it is
+    // left out when no row of the wave saw its maximum move (nearly always, a few tiles into a row's keys).
+    bool moved = false;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) moved = moved || alpha[ct] != 1.f;
+    if (__ballot(moved) != 0ull) {
+#pragma unroll
+      for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) acc_o[ct][c] = acc_o[ct][c] * alpha[ct];
+    }
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       if (c + AHEAD < NC) read_values(c + AHEAD, vf[(c + AHEAD) % (AHEAD + 1)]);
       if constexpr (AHEAD > 0) __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct) acc_o[ct][c] = acc_o[ct][c] * alpha[ct];
 #pragma unroll
       for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
