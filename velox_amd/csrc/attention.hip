@@ -1299,8 +1299,17 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
     // behind 1,920 keys 86.2 / 65.7 / 50.8, 4,096 tokens 123 / 123 / 89.9; with 28 over 4, 1,024 tokens 36.1 / 37.7 / 30.3 and
     // 2,048 tokens 75.6 / 69.6 / 67.4.  Fewer workgroups still stay with the kernels below (512 tokens: 16.4 / 23.0 / 19.5).
     const long long workgroups = (long long)((max_q_len * group + 127) / 128) * nkv * num_seqs * splits;
+    // (one prompt alone from an empty cache is the step whose last rows decide its time: two sets up to 1.75 workgroups
+    // per compute unit, 2,048 tokens with 28 heads over 4: 68.7 us with one set, 64.2 with two; behind as many keys in the
+    // cache one set is quicker again, 129 against 136)
+    const long long two_sets_up_to = (num_seqs == 1 && max_kv_len <= max_q_len) ? 7LL * compute_units() / 4 : 3LL * compute_units() / 2;
+    if (splits == 1 && workgroups <= two_sets_up_to && workgroups * 5 >= 3LL * compute_units()) return launch_direct(true);
     if (workgroups * 2 > 3LL * compute_units()) return launch_direct(false);
-    if (splits == 1 && workgroups * 5 >= 3LL * compute_units()) return launch_direct(true);
+    // Keys split over workgroups (few tokens behind thousands of keys): direct loads throughout, 512 tokens behind 3,584
+    // keys 79.8 / 73.8 / 80.5 and behind 29,488 keys 397 / 357 / 378 with 28 heads over 4; with 12 over 2, 2,048 tokens behind
+    // 2,048 keys 110 / 95.8 / 95.0.  Two sets when even the splits leave compute units empty (12 over 2, 512 tokens behind
+    // 3,584 keys: 57.3 / 47.7 / 40.4).
+    if (splits > 1) return launch_direct(workgroups <= compute_units());
   }
   // Eight waves per workgroup when bfloat16 portions are long enough to fill their rows and the step brings enough rows
   // that the larger workgroups still fill the GPU.  Behind few keys (a causal step's longest workgroup decides how

@@ -135,6 +135,8 @@ class HipOps:
         c.velox_probe_read.restype = _I
         c.velox_probe_mfma.argtypes = [_I, _I, _P, _P]
         c.velox_probe_mfma.restype = _I
+        c.velox_probe_grid_barrier.argtypes = [_I, _I, _I, _P, _P, _P]
+        c.velox_probe_grid_barrier.restype = _I
         for fn in (c.velox_embed, c.velox_place_tokens, c.velox_add_rmsnorm, c.velox_silu_mul, c.velox_rope_kv_write, c.velox_gemm_fma,
                    c.velox_argmax, c.velox_sample, c.velox_sample_chunked, c.velox_apply_penalties, c.velox_count_tokens, c.velox_count_sampled,
                    c.velox_penalties_from_counts):
@@ -943,6 +945,21 @@ class HipOps:
         blocks = self.num_cus * 8
         seconds = self._timed(lambda: self._launched(self._core.velox_probe_read(_ptr(data), num_bytes, _ptr(sink), blocks, self._stream()), "probe_read"), repeats)
         return num_bytes / seconds * 1e-9
+
+    def probe_grid_barrier(self, fenced: bool, rounds: int = 2000, repeats: int = 3) -> float:
+        """Microseconds per barrier across one workgroup per compute unit inside one kernel: with relaxed agent-scope
+        counters only, or (``fenced``) with the release and acquire that ordinary stores and loads around it need."""
+        counters = torch.zeros(17 * 32, dtype=torch.int32, device=self.device)
+        failed = torch.zeros(1, dtype=torch.int32, device=self.device)
+
+        def launch() -> None:
+            counters.zero_()
+            self._launched(self._core.velox_probe_grid_barrier(self.num_cus, rounds, int(fenced), _ptr(counters), _ptr(failed), self._stream()), "probe_grid_barrier")
+
+        seconds = self._timed(launch, repeats)
+        if int(failed.item()) != 0:
+            raise KernelError("probe_grid_barrier: a workgroup gave up waiting for the others")
+        return seconds / rounds * 1e6
 
     def probe_mfma_rate(self, iterations: int = 20000, repeats: int = 5) -> float:
         """TFLOP/s of independent bfloat16 32x32x16 matrix instructions, two workgroups of four waves per compute unit."""
