@@ -1043,6 +1043,15 @@ def test_probes_report_rates_in_the_band_of_this_card(ops):
     assert 1250.0 < mfma <= 2600.0, mfma
 
 
+def test_grid_barrier_probe_ends_and_counts_every_round(ops):
+    """The probe of a barrier across one workgroup per compute unit runs all its rounds (nobody gives up waiting: that
+    would raise) in both forms, takes between 0.2 and 200 us per barrier, and the fenced form is the dearer one."""
+    relaxed = ops.probe_grid_barrier(False, rounds=200, repeats=2)
+    fenced = ops.probe_grid_barrier(True, rounds=200, repeats=2)
+    assert 0.2 < relaxed < 200.0 and 0.2 < fenced < 200.0, (relaxed, fenced)
+    assert fenced > relaxed, (relaxed, fenced)
+
+
 def test_place_tokens_puts_sampled_ids_into_a_steps_rows(ops, ref):
     from velox_amd.kernels.hip_ops import KernelError
 
