@@ -31,12 +31,6 @@
 #endif
 
 constexpr int D = VELOX_HEAD_DIM;
-#ifndef VELOX_PV_AHEAD
-#define VELOX_PV_AHEAD 1
-#endif
-#ifndef VELOX_QK_AHEAD
-#define VELOX_QK_AHEAD 0
-#endif
 static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple of 16 between 16 and 256");
 
 template <typename T> struct Frag;
@@ -583,7 +577,7 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     const bf16_t* __restrict__ qkv, int qkv_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
-    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens, int slots) {
+    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens) {
   typedef bf16_t T;
   typedef Block<T> B;
   typedef typename B::Operand Operand;
@@ -608,7 +602,13 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 4, i = lane & 15;
   const int group = nh / nkv;
-  const int b = blockIdx.z / splits, split = blockIdx.z % splits;
+  // The grid is (sequence and split, KV head, row block), and blockIdx.z counts a sequence's row blocks from its LAST
+  // rows, which read the most keys.  Workgroups are handed out in launch order, x fastest, each to the first compute
+  // unit with room: the longest of every sequence go first and the short ones fill in as compute units come free
+  // (against an order that paired long with short per compute unit, measured on MI355X: 2,048 tokens 62.4 -> 52.8 us,
+  // 4,096 tokens 169 -> 146, 8,192 tokens 559 -> 528).
+  const int b = blockIdx.x / splits, split = blockIdx.x % splits;
+  const int kvh = blockIdx.y;
   const int page_size = 1 << page_shift;
 
   const int q_start = cu_q[b];
@@ -616,15 +616,9 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
   const int kv_len = kv_lens[b];
   const int ctx = kv_len - q_len;
   const int rows_total = q_len * group;
-  // (which rows and which KV head: as in the general kernel, the longest units first, then the shortest, ...)
   const int blocks_here = (rows_total + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
-  const int units = blocks_here * nkv;
-  const int launch_index = blockIdx.x + gridDim.x * blockIdx.y;
-  if (launch_index >= units) return;
-  const int round = launch_index / slots, within = launch_index % slots;
-  const int rank = (round & 1) ? units - 1 - ((round >> 1) * slots + within) : (round >> 1) * slots + within;  // 0 = longest
-  const int kvh = rank % nkv;
-  const int r0 = (blocks_here - 1 - rank / nkv) * ROWS_PER_BLOCK;
+  if ((int)blockIdx.z >= blocks_here) return;
+  const int r0 = (blocks_here - 1 - (int)blockIdx.z) * ROWS_PER_BLOCK;
 
   bool row_ok[CT];
   int tok[CT], head[CT], pos[CT];
@@ -786,27 +780,19 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
 
     // ---- S^T = K Q^T: tile t = 2 b + u of the 64 keys ----------------------------------------
     float4_t s[CT][NT];
-    constexpr int QK_AHEAD = VELOX_QK_AHEAD;
-    Operand kf[QK_AHEAD + 1][NQB];
-    auto read_keys = [&](int t, Operand (&into)[NQB]) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      Operand kf[NQB > 0 ? NQB : 1];  // (the template is parsed for every head size, run for 64 and 128)
       const int tile_bytes = (32 * (t >> 1) + 4 * (t & 1)) * (2 * D);
 #pragma unroll
       for (int cb = 0; cb < NQB; ++cb)
-        into[cb] = __builtin_bit_cast(Operand, *reinterpret_cast<const float4_t*>(tile_base + ((cb & 1) ? k_odd : k_even) + 128 * (cb >> 1) + tile_bytes));
-    };
-#pragma unroll
-    for (int a = 0; a < QK_AHEAD; ++a) read_keys(a, kf[a]);
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      if (QK_AHEAD == 0) read_keys(t, kf[0]);
-      else if (t + QK_AHEAD < NT) read_keys(t + QK_AHEAD, kf[(t + QK_AHEAD) % (QK_AHEAD + 1)]);
-      if constexpr (QK_AHEAD > 0) __builtin_amdgcn_sched_barrier(0);
+        kf[cb] = __builtin_bit_cast(Operand, *reinterpret_cast<const float4_t*>(tile_base + ((cb & 1) ? k_odd : k_even) + 128 * (cb >> 1) + tile_bytes));
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) s[ct][t] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int cb = 0; cb < NQB; ++cb)
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) s[ct][t] = B::mma(kf[t % (QK_AHEAD + 1)][cb], qf[ct][cb], s[ct][t]);
+        for (int ct = 0; ct < CT; ++ct) s[ct][t] = B::mma(kf[cb], qf[ct][cb], s[ct][t]);
     }
     // ---- scale, mask (only where the tile crosses a row's limits), running maximum ----------
     const bool whole = n0 + BN <= kv_len && n0 + BN - 1 <= wave_first_pos && (window <= 0 || n0 > wave_last_pos - window);
@@ -863,7 +849,7 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
       m_i[ct] = m_new;
     }
     // ---- O^T = O^T * alpha + V^T P^T --------------------------------------------------------
-    constexpr int AHEAD = VELOX_PV_AHEAD;  // channel tiles whose operands are in flight ahead of the one being multiplied
+    constexpr int AHEAD = 1;  // channel tiles whose operands are in flight ahead of the one being multiplied
     Operand vf[AHEAD + 1][NKB];
     auto read_values = [&](int c, Operand (&into)[NKB]) {
 #pragma unroll
@@ -1272,15 +1258,16 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
   const bool direct_ok = HAS_DIRECT && page_shift >= 3 && portion_kernel_choice != 1;
   auto launch_direct = [&](bool two_sets = false) -> int {
     if constexpr (HAS_DIRECT) {
-      dim3 grid((max_q_len * group + 127) / 128, nkv, num_seqs * splits);
+      dim3 grid(num_seqs * splits, nkv, (max_q_len * group + 127) / 128);
+      if (grid.z > 65535u) return (int)hipErrorInvalidValue;  // (more than 8 million rows in one portion)
       if (two_sets)
         direct_attention_kernel<2, 4, 2><<<grid, 512, 0, stream>>>(
             (const bf16_t*)qkv, qkv_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width, cu_q, kv_lens, (bf16_t*)out,
-            part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+            part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
       else
         direct_attention_kernel<2, 4><<<grid, 256, 0, stream>>>(
             (const bf16_t*)qkv, qkv_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width, cu_q, kv_lens, (bf16_t*)out,
-            part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+            part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
     }
     int status = (int)hipGetLastError();
     if (status != 0 || splits == 1) return status;
@@ -1291,25 +1278,30 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
   if (direct_ok && portion_kernel_choice >= 2 && max_q_len * group > 64) return launch_direct(portion_kernel_choice == 3);
   if (direct_ok && max_q_len * group > 64) {
     // Measured on MI355X over prompts and portions of 128 to 8,192 tokens behind up to 30,000 keys, with 28 heads over 4,
-    // 12 over 2 and 40 over 8 (us, the kernels below / direct loads / direct loads with two sets of waves).  From 1.5
-    // workgroups of 128 rows per compute unit on, the kernel with direct loads: 2 x 2,048 tokens 110 / 103 / 115, 4 x 512
-    // behind 512 keys 51.8 / 46.9 / 53.4, 8,192 tokens 631 / 608 / 618.  With fewer, down to 0.6 per compute unit and when the
-    // keys are not split over workgroups, two sets of waves share a workgroup's keys, which fills the compute units
-    // that one set would leave half empty: with 12 heads over 2, 4 x 512 tokens behind 1,536 keys 80.0 / 65.3 / 49.6, 16 x 128
-    // behind 1,920 keys 86.2 / 65.7 / 50.8, 4,096 tokens 123 / 123 / 89.9; with 28 over 4, 1,024 tokens 36.1 / 37.7 / 30.3 and
-    // 2,048 tokens 75.6 / 69.6 / 67.4.  Fewer workgroups still stay with the kernels below (512 tokens: 16.4 / 23.0 / 19.5).
+    // 12 over 2 and 40 over 8 (us: the kernels below / direct loads / direct loads with two sets of waves).  Direct loads
+    // from 0.6 workgroups of 128 rows per compute unit on, and wherever the keys are split over workgroups (few tokens
+    // behind thousands of keys): 2 x 2,048 tokens 105 / 84 / 100, 8,192 tokens 641 / 535 / 575, 512 tokens behind 29,488
+    // keys 397 / 355 / 375; fewer workgroups stay with the kernels below (512 tokens: 16 / 22 / 19).
+    // Two sets of waves share a workgroup's keys, which fills the compute units that one set leaves half empty:
+    //  * up to 1.5 workgroups per compute unit (12 heads over 2: 4 x 512 tokens behind 1,536 keys 79 / 63 / 45, 4,096 tokens
+    //    158 / 122 / 81; 28 over 4: 1,024 tokens 34 / 36 / 28), up to 1.75 for one prompt from an empty cache, the step whose
+    //    last rows decide its time (2,048 tokens: 72 / 67 / 53);
+    //  * with split keys, when even the splits leave compute units empty (12 over 2, 512 tokens behind 3,584 keys: 57 / 48 / 41);
+    //  * above that, where the workgroups are about equally long (at least as many keys in the cache as in the portions,
+    //    2,048 keys or more) and the count says so: one set keeps two workgroups on a compute unit, two sets one that is
+    //    done in 0.55 of the time, and whole rounds of workgroups decide (40 heads over 8, 640 workgroups on 256 compute
+    //    units: 4 x 512 tokens behind 3,584 keys 299 / 238 / 226, behind 7,680 keys 598 / 477 / 438; with 448 one round of one set
+    //    is quicker, 28 over 4, 4 x 512 behind 3,584: 162 / 142 / 152).
+    const long long units = compute_units();
     const long long workgroups = (long long)((max_q_len * group + 127) / 128) * nkv * num_seqs * splits;
-    // (one prompt alone from an empty cache is the step whose last rows decide its time: two sets up to 1.75 workgroups
-    // per compute unit, 2,048 tokens with 28 heads over 4: 68.7 us with one set, 64.2 with two; behind as many keys in the
-    // cache one set is quicker again, 129 against 136)
-    const long long two_sets_up_to = (num_seqs == 1 && max_kv_len <= max_q_len) ? 7LL * compute_units() / 4 : 3LL * compute_units() / 2;
-    if (splits == 1 && workgroups <= two_sets_up_to && workgroups * 5 >= 3LL * compute_units()) return launch_direct(true);
-    if (workgroups * 2 > 3LL * compute_units()) return launch_direct(false);
-    // Keys split over workgroups (few tokens behind thousands of keys): direct loads throughout, 512 tokens behind 3,584
-    // keys 79.8 / 73.8 / 80.5 and behind 29,488 keys 397 / 357 / 378 with 28 heads over 4; with 12 over 2, 2,048 tokens behind
-    // 2,048 keys 110 / 95.8 / 95.0.  Two sets when even the splits leave compute units empty (12 over 2, 512 tokens behind
-    // 3,584 keys: 57.3 / 47.7 / 40.4).
-    if (splits > 1) return launch_direct(workgroups <= compute_units());
+    if (splits > 1) return launch_direct(workgroups <= units);
+    if (workgroups * 5 >= 3 * units) {
+      const long long two_sets_up_to = (num_seqs == 1 && max_kv_len <= max_q_len) ? 7 * units / 4 : 3 * units / 2;
+      bool two_sets = workgroups <= two_sets_up_to;
+      if (!two_sets && max_kv_len >= 2048 && max_kv_len >= 2 * max_q_len)
+        two_sets = 55 * ((workgroups + units - 1) / units) < 100 * ((workgroups + 2 * units - 1) / (2 * units));
+      return launch_direct(two_sets);
+    }
   }
   // Eight waves per workgroup when bfloat16 portions are long enough to fill their rows and the step brings enough rows
   // that the larger workgroups still fill the GPU.  Behind few keys (a causal step's longest workgroup decides how
