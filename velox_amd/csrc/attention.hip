@@ -702,9 +702,41 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     v_chan[m] = s / 8;
   }
   v_key = 8 * ((lane & 7) ^ ((lane >> 3) & 7));  // (the channel's low bits are the lane's: 64 q is a multiple of 8 channels)
-  auto issue = [&](int n0, int buffer) {
+  // A tile that lies wholly inside the sequence, which is every tile but a sequence's last, takes the short way.  The
+  // keys of one load instruction (64 / CPR consecutive ones, at a multiple of as many) lie in one page, since a page
+  // holds at least 8: their page's address is the same for the whole wave and is worked out in scalar registers, and a
+  // lane's offset from it never changes.  A lane's eight values of a channel lie in one page too; its page differs
+  // from other lanes', but is the same for all of the wave's loads of a tile, which are 8 WAVES channels apart.
+  constexpr int KEYS_PER_LOAD = 64 / CPR;
+  const uint32_t k_lane_bytes = (uint32_t)(((lane / CPR) * D + k_col[0]) * 2);
+  const size_t v_page_elems = ((size_t)nkv * D) << page_shift;
+  const uint32_t v_lane_elems = ((uint32_t)(kvh * D + 8 * wave + (lane >> 3))) << page_shift;
+  auto issue = [&](int tile_n0, int tile_buffer) {
+    // (both are the same for the whole wave; said so, or the compiler keeps them and all that follows from them in
+    // vector registers)
+    const int n0 = __builtin_amdgcn_readfirstlane(tile_n0), buffer = __builtin_amdgcn_readfirstlane(tile_buffer);
     char* const k_dst = smem[buffer];
     char* const v_dst = smem[buffer] + TILE_BYTES;
+    if (n0 + BN <= kv_len) {  // (the same for every thread)
+      // (all page ids first: the loads below are barriers to the compiler's reordering, and each id is a trip to LDS)
+      const int window_first = __builtin_amdgcn_readfirstlane(first_page);
+      const int nv = n0 + v_key;
+      const size_t v_page = page_of(nv);
+      size_t k_page[LPW];
+#pragma unroll
+      for (int m = 0; m < LPW; ++m)
+        k_page[m] = (size_t)__builtin_amdgcn_readfirstlane(page_ids[((n0 + KEYS_PER_LOAD * (wave + WAVES * m)) >> page_shift) - window_first]);
+#pragma unroll
+      for (int m = 0; m < LPW; ++m) {
+        const int key0 = n0 + KEYS_PER_LOAD * (wave + WAVES * m);
+        const T* base = k_cache + (((k_page[m] * nkv + kvh) << page_shift) + (key0 & (page_size - 1))) * D;
+        load_to_lds_16(base, k_lane_bytes, k_dst + 1024 * (wave + WAVES * m));
+      }
+      const T* v_src = v_cache + v_page * v_page_elems + (v_lane_elems + (uint32_t)(nv & (page_size - 1)));
+#pragma unroll
+      for (int m = 0; m < LPW; ++m) load_to_lds_16(v_src + ((size_t)(8 * WAVES * m) << page_shift), v_dst + 1024 * (wave + WAVES * m));
+      return;
+    }
 #pragma unroll
     for (int m = 0; m < LPW; ++m) {
       int nk = n0 + k_key[m];

@@ -61,6 +61,12 @@ __device__ __forceinline__ void load_to_lds_16(const void* src, void* dst) {
   const uint32_t at = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)dst;
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(at), "v"(src) : "memory", "m0");
 }
+// The same with the address as a base that is the same for the whole wave (it travels in scalar registers) plus 32 bits of
+// byte offset per lane: no 64-bit vector arithmetic per load.
+__device__ __forceinline__ void load_to_lds_16(const void* wave_base, uint32_t lane_bytes, void* dst) {
+  const uint32_t at = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)dst;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(at), "v"(lane_bytes), "s"(wave_base) : "memory", "m0");
+}
 template <int N> __device__ __forceinline__ void wait_for_loads() {
   static_assert(N >= 0 && N < 64, "the counter of loads in flight has six bits");
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
