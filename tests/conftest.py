@@ -1,7 +1,10 @@
 """Test set-up: the repository root and this folder on the import path; tests marked ``gpu`` are skipped where
-no GPU is visible (the marker itself is registered in pytest.ini)."""
+no GPU is visible (the marker itself is registered in pytest.ini); every test starts from random number generators
+seeded with its own name, so what a test draws does not depend on which tests ran before it."""
 import pathlib
+import random
 import sys
+import zlib
 
 import pytest
 
@@ -23,3 +26,12 @@ def pytest_runtest_setup(item):
         _gpu_visible = torch.cuda.is_available()
     if not _gpu_visible:
         pytest.skip("needs a GPU")
+
+
+@pytest.fixture(autouse=True)
+def seeded_by_test_name(request):
+    import torch
+
+    seed = zlib.crc32(request.node.nodeid.encode())
+    random.seed(seed)
+    torch.manual_seed(seed)  # (the generators of every device)

@@ -144,7 +144,7 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
     T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
-    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens, int slots) {
+    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens) {
   typedef Block<T> B;
   typedef typename B::Operand Operand;
   constexpr int KB = B::KB;
@@ -175,7 +175,14 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
   const int lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 4, i = lane & 15;
   const int group = nh / nkv;
-  const int b = blockIdx.z / splits, split = blockIdx.z % splits;
+  // The grid is (sequence and split, KV head, row block), and blockIdx.z counts a sequence's row blocks from its LAST
+  // rows, which read the most keys.  Workgroups are handed out in launch order, x fastest, each to the first compute
+  // unit with room: the longest of every sequence go first and the short ones fill in as compute units come free.
+  // (Measured on MI355X against an order that paired long with short per compute unit, head size 96, 28 heads over 4:
+  // 4,096 tokens 179 -> 152 us, 8,192 tokens 594 -> 557, 1,024 tokens 28.9 -> 25.4; 2,048 tokens, whose 448 workgroups are
+  // all resident at once, 59.5 -> 62.3.)
+  const int b = blockIdx.x / splits, split = blockIdx.x % splits;
+  const int kvh = blockIdx.y;
   const int page_size = 1 << page_shift;
 
   const int q_start = cu_q[b];
@@ -183,17 +190,9 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
   const int kv_len = kv_lens[b];
   const int ctx = kv_len - q_len;
   const int rows_total = q_len * group;
-  // Which (row block, KV head) this workgroup takes.  Late rows read the most keys.  Workgroups are handed to the
-  // compute units in launch order, `slots` at a time: the first round takes the longest units, the second the
-  // shortest (so that a compute unit's second workgroup makes up for its first), the third the next longest, ...
   const int blocks_here = (rows_total + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
-  const int units = blocks_here * nkv;
-  const int launch_index = blockIdx.x + gridDim.x * blockIdx.y;
-  if (launch_index >= units) return;
-  const int round = launch_index / slots, within = launch_index % slots;
-  const int rank = (round & 1) ? units - 1 - ((round >> 1) * slots + within) : (round >> 1) * slots + within;  // 0 = longest
-  const int kvh = rank % nkv;
-  const int r0 = (blocks_here - 1 - rank / nkv) * ROWS_PER_BLOCK;
+  if ((int)blockIdx.z >= blocks_here) return;
+  const int r0 = (blocks_here - 1 - (int)blockIdx.z) * ROWS_PER_BLOCK;
 
   bool row_ok[CT];
   int tok[CT], head[CT], pos[CT];
@@ -1343,9 +1342,10 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
   // keys 315 us against 426 the other way round; the two meet where an average row reads about 1,300 keys.
   constexpr int WIDE = (sizeof(T) == 2 && D <= 128) ? 2 : 1;
   const int rows = max_q_len * group;
+  if ((rows + 63) / 64 > 65535) return (int)hipErrorInvalidValue;  // (row blocks are the grid's third dimension)
   if (WIDE == 2 && rows > 64 && (long long)total_tokens * group / 128 * nkv * splits >= compute_units()) {
     if (max_kv_len - max_q_len / 2 <= 1280 || rows < 192) {  // (keys an average row reads)
-      dim3 grid((rows + 127) / 128, nkv, num_seqs * splits);
+      dim3 grid(num_seqs * splits, nkv, (rows + 127) / 128);
       // With enough workgroups to keep two on every compute unit, the 128 rows go to four waves of two row tiles: half
       // the reads of K and V^T from LDS per row, which bound this kernel.  Measured on MI355X (us, eight waves of one
       // tile against four of two): 4 x 512 tokens behind 1,024 keys 62.7 / 54.7, 2,048 tokens from an empty cache
@@ -1356,29 +1356,29 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
       if (rows >= 256 && workgroups * 4 >= 7LL * compute_units()) {
         paged_attention_kernel<T, BN, 2, 1, 4><<<grid, 256, 0, stream>>>(
             (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-            part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+            part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
       } else {
         paged_attention_kernel<T, BN, 1, 1, 8><<<grid, 512, 0, stream>>>(
             (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-            part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+            part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
       }
     } else {
-      dim3 grid((rows + 255) / 256, nkv, num_seqs * splits);
+      dim3 grid(num_seqs * splits, nkv, (rows + 255) / 256);
       paged_attention_kernel<T, BN, WIDE, 1, 8><<<grid, 512, 0, stream>>>(
           (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
     }
   } else if (WIDE == 2 && (long long)((rows + 63) / 64) * nkv * num_seqs * splits < 2 * compute_units() && max_kv_len >= 8 * BN) {
     // too few workgroups to fill the GPU and many keys each: two sets of waves share a workgroup's keys
-    dim3 grid((rows + 63) / 64, nkv, num_seqs * splits);
+    dim3 grid(num_seqs * splits, nkv, (rows + 63) / 64);
     paged_attention_kernel<T, BN, 1, WIDE><<<grid, 256 * WIDE, 0, stream>>>(
         (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
   } else {
-    dim3 grid((rows + 63) / 64, nkv, num_seqs * splits);
+    dim3 grid(num_seqs * splits, nkv, (rows + 63) / 64);
     paged_attention_kernel<T, BN, 1, 1><<<grid, 256, 0, stream>>>(
         (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, compute_units());
+        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
   }
   int status = (int)hipGetLastError();
   if (status != 0 || splits == 1) return status;
