@@ -1052,6 +1052,22 @@ def test_grid_barrier_probe_ends_and_counts_every_round(ops):
     assert fenced > relaxed, (relaxed, fenced)
 
 
+def test_kernel_timer_times_a_launch_inside_a_graph(ops):
+    """`velox_amd.kernels.measure` (the timings that the launch rules quote): a case of scattered pages has the shapes
+    the attention entry point checks, and the timer replays a graph of launches and returns a plausible time per call."""
+    import math
+
+    from velox_amd.engine.batch import Workspace
+    from velox_amd.kernels.measure import attention_case, time_in_graph
+
+    qkv, k, v, tables, cu_q, kv_lens = attention_case(2, 96, 160, 4, 2, 64, 16)
+    assert tables.shape == (2, 10) and int(tables.min()) >= 1 and len(set(tables.flatten().tolist())) == 20
+    workspace = Workspace(torch.device("cuda"))
+    each = time_in_graph(lambda: ops.paged_attention(qkv, 4, 2, 64, k, v, 16, tables, cu_q, kv_lens, 96, 160, 1 / math.sqrt(64), None, False, workspace),
+                         launches=2, rounds=2)
+    assert 1.0 < each < 5000.0, each
+
+
 def test_place_tokens_puts_sampled_ids_into_a_steps_rows(ops, ref):
     from velox_amd.kernels.hip_ops import KernelError
 
