@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from velox_amd.cache import NULL_PAGE, CacheManager, PoolExhausted, PageAllocator
-from velox_amd.parts import PagedNeed, StateNeed, kv_pages
+from velox_amd.parts import StateNeed, kv_pages
 
 
 def test_allocator_order_and_errors():

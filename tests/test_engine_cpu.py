@@ -3,7 +3,7 @@ plain PyTorch references standing in for the kernels, against the plain whole-se
 import pytest
 import torch
 
-from helpers import CONFIGS, PAGE_SIZE, Harness, make_folder, random_tokens
+from helpers import PAGE_SIZE, Harness, make_folder, random_tokens
 from plain_qwen2 import qwen2_logits, read_model_folder
 from torch_ops import TorchOps
 

@@ -3,7 +3,7 @@ function, sampler and request bookkeeping together."""
 import pytest
 import torch
 
-from helpers import CONFIGS, PAGE_SIZE, make_folder, random_tokens
+from helpers import PAGE_SIZE, make_folder, random_tokens
 from plain_qwen2 import qwen2_logits, read_model_folder
 from torch_ops import TorchOps
 from velox_amd import Engine, EngineConfig, Request, SamplingParams

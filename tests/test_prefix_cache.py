@@ -15,7 +15,7 @@ from velox_amd.cache.allocator import PageAllocator
 from velox_amd.cache.prefix import PrefixCache
 from velox_amd.engine.request import RequestStatus
 from velox_amd.engine.scheduler import Scheduler, SchedulerConfig
-from velox_amd.parts import PagedNeed, StateNeed, kv_pages
+from velox_amd.parts import StateNeed, kv_pages
 
 
 # -- the trie alone ------------------------------------------------------------------------------------------------------

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 import replay_cases as rc
-from helpers import CONFIGS, PAGE_SIZE, make_folder
+from helpers import PAGE_SIZE, make_folder
 from plain_qwen2 import read_model_folder
 from torch_ops import TorchOps
 from velox_amd.engine.replay import Replayer, TraceError

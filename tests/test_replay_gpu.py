@@ -5,7 +5,6 @@ itself as a user starts it."""
 import json
 import os
 import subprocess
-import sys
 
 import numpy as np
 import pytest

@@ -9,9 +9,6 @@ product never loads this file.
 """
 from __future__ import annotations
 
-import math
-from typing import Optional
-
 import numpy as np
 import torch
 

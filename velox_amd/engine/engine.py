@@ -24,7 +24,6 @@ from ..config.engine_config import EngineConfig
 from ..config.model_config import read_generation_eos
 from ..config.registry import config_from_dict, get_architecture, load_config
 from ..parts.model import DecoderModel
-from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from ..weights import bind_from_checkpoint, bind_random
 from .batch import StepEntry
