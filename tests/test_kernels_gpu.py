@@ -541,6 +541,31 @@ def test_paged_attention_long_portions(ops, ref, dtype, nh, nkv, d, page, window
     torch.testing.assert_close(_run_attention(ops, alone, nh, nkv, d, page, window=window), got[first:first + 300], **same)
 
 
+@pytest.mark.parametrize("dtype,nh,nkv,d,page,long_context,choices", [
+    (torch.bfloat16, 14, 2, 128, 8, 17000, (1, 2, 3)), (torch.bfloat16, 6, 3, 64, 8, 16500, (2, 3)), (torch.float32, 4, 2, 32, 4, 9000, (0,))])
+@pytest.mark.parametrize("window", [None, 5000])
+def test_paged_attention_behind_more_pages_than_the_kernels_keep_ids_of(ops, ref, dtype, nh, nkv, d, page, long_context, choices, window):
+    """A workgroup keeps the page ids of the keys it visits in LDS, 2,048 at a time, and fetches the next lot when its
+    tiles leave the window: portions behind contexts of more than 2,048 pages in one pass over the keys (no split), in
+    every kernel for portions, with a short sequence and a single token behind the long context beside them."""
+    from velox_amd.engine.batch import Workspace
+
+    assert long_context // page > 2048
+    seqs = [(200, long_context), (64, 64), (1, long_context - 300)]
+    case = _attention_case(dtype, nh, nkv, d, page, seqs, seed=d + nh + 5)
+    want = _run_attention(ref, case, nh, nkv, d, page, window=window)
+    tolerance = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    lib = ops.attention_library(d)
+    workspace = Workspace(torch.device("cuda"))
+    try:
+        for choice in choices:
+            lib.velox_attention_portion_kernel(choice)
+            got = _run_attention(ops, case, nh, nkv, d, page, window=window, splits=1, workspace=workspace)
+            torch.testing.assert_close(got, want, **tolerance)
+    finally:
+        lib.velox_attention_portion_kernel(0)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,d,page", [(28, 4, 128, 16), (4, 2, 16, 4), (6, 2, 96, 8), (8, 8, 64, 1)])
 @pytest.mark.parametrize("window", [None, 200])
