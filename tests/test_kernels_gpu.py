@@ -689,6 +689,24 @@ def test_decode_split_keys_equals_one_pass(ops, ref, dtype, nh, nkv, d, page):
         torch.testing.assert_close(got, want, **t)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decode_behind_more_pages_than_the_streaming_kernel_keeps_ids_of(ops, ref, dtype):
+    """The streaming kernel keeps the page ids of a split's keys in LDS; a split of more pages than it has room for
+    (2,048) goes through the kernel for portions instead, with the same result; with more splits the streaming kernel
+    takes it again."""
+    from velox_amd.engine.batch import Workspace
+
+    nh, nkv, d, page = 6, 2, 64, 4
+    seqs = [(1, 9000), (1, 77), (1, 8300)]
+    case = _attention_case(dtype, nh, nkv, d, page, seqs, seed=31)
+    workspace = Workspace(torch.device("cuda"))
+    want = _run_attention(ref, case, nh, nkv, d, page)
+    t = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    for splits in (1, 2, 8):  # 1 and 2: 2,250 and 1,125 + 2 pages per split, beyond and within the room for ids
+        got = _run_attention(ops, case, nh, nkv, d, page, splits=splits, all_decode=True, workspace=workspace)
+        torch.testing.assert_close(got, want, **t)
+
+
 def test_far_key_among_hundreds_is_found(ops):
     # one key far back matches the query strongly: the output must be (nearly) that key's value
     nh, nkv, d, page = 4, 2, 64, 16
