@@ -453,7 +453,8 @@ def _run_attention(impl, case, nh, nkv, d, page, window=None, splits=None, all_d
     ).float()
 
 
-ATTN_SHAPES = [(4, 2, 16, 4), (3, 1, 32, 8), (6, 2, 48, 16), (28, 4, 128, 16), (8, 8, 64, 64), (7, 1, 96, 32), (2, 1, 256, 16), (40, 8, 128, 2)]
+ATTN_SHAPES = [(4, 2, 16, 4), (3, 1, 32, 8), (6, 2, 48, 16), (28, 4, 128, 16), (8, 8, 64, 64), (7, 1, 96, 32), (2, 1, 256, 16), (40, 8, 128, 2), (5, 1, 80, 8),
+               (6, 2, 192, 16)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

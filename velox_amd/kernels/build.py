@@ -27,7 +27,7 @@ CORE_SOURCES = ["elementwise.hip", "gemm.hip", "skinny_gemm.hip", "sampling.hip"
 ATTENTION_SOURCES = ["attention.hip"]
 HEADERS = ["common.h", "no_alloc.h"]
 # head sizes built ahead of time by build_all(); any other multiple of 16 up to 256 is built at first use
-DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 96, 128, 256)
+DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 192, 256)
 
 
 class BuildError(RuntimeError):
