@@ -673,6 +673,43 @@ def test_paged_attention_with_tiles_loaded_straight_into_lds(ops, ref, nh, nkv, 
         lib.velox_attention_portion_kernel(0)
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_paged_attention_random_steps_agree_with_the_reference(ops, ref, seed):
+    """Steps drawn at random: head size, heads and groups, page size, data type, window, splits of the keys, which kernel
+    takes the portions, and one to six sequences that are single tokens, short portions or long ones, from an empty
+    cache or behind up to 5,000 keys."""
+    import random
+
+    from velox_amd.engine.batch import Workspace
+
+    rng = random.Random(seed)
+    workspace = Workspace(torch.device("cuda"))
+    for case_no in range(12):
+        d = rng.choice([16, 48, 64, 80, 96, 128, 192, 256])
+        page = rng.choice([1, 2, 4, 8, 16, 32, 64, 128])
+        dtype = rng.choice(DTYPES)
+        nkv = rng.choice([1, 2, 4, 8])
+        nh = nkv * rng.choice([1, 2, 3, 5, 7])
+        seqs = []
+        for _ in range(rng.randint(1, 6)):
+            kind = rng.random()
+            q = 1 if kind < 0.25 else rng.randint(2, 70) if kind < 0.5 else rng.randint(71, 900)
+            seqs.append((q, q + rng.choice([0, 0, rng.randint(1, 300), rng.randint(300, 5000)])))
+        window = rng.choice([None, None, rng.randint(1, 3000)])
+        choice = rng.choice([0, 0, 1, 2, 3])
+        splits = rng.choice([None, None, 1, 2, 3])
+        case = _attention_case(dtype, nh, nkv, d, page, seqs, seed=100 * seed + case_no)
+        lib = ops.attention_library(d)
+        lib.velox_attention_portion_kernel(choice)
+        try:
+            got = _run_attention(ops, case, nh, nkv, d, page, window=window, splits=splits, workspace=workspace)
+        finally:
+            lib.velox_attention_portion_kernel(0)
+        want = _run_attention(ref, case, nh, nkv, d, page, window=window)
+        said = f"seed {seed} case {case_no}: {dtype} d={d} page={page} heads {nh}/{nkv} {seqs} window={window} kernel {choice} splits={splits}"
+        torch.testing.assert_close(got, want, msg=lambda m: f"{said}: {m}", **(dict(rtol=2e-2, atol=2e-2) if dtype == torch.bfloat16 else dict(rtol=1e-4, atol=2e-5)))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 4), (28, 4, 128, 16), (3, 1, 32, 8), (2, 1, 256, 16)])
 def test_decode_split_keys_equals_one_pass(ops, ref, dtype, nh, nkv, d, page):
