@@ -134,7 +134,13 @@ def test_pre_norm_block_alone(ops):
     after_mixer = start + 2 * rms_norm(start, w1, 1e-5)
     torch.testing.assert_close(residual.cpu(), after_mixer, rtol=1e-5, atol=1e-5)  # the mixer's output is in, the feed-forward's is pending
     want = gated_mlp(rms_norm(after_mixer, w2, 1e-5), wf["gate_up_weight"][:inter], wf["gate_up_weight"][inter:], wf["down_weight"])
-    torch.testing.assert_close(pending.float().cpu(), want, rtol=1e-4, atol=1e-5)
+    # Outputs of size 30 that are sums of terms of both signs: float32 sums of them differ by some 1e-5 from one order of
+    # adding to another (over 400 draws of h the plain float32 result misses rtol 1e-4, atol 1e-5 against the kernels'
+    # in 26).  The yardstick is the same formula in float64: the kernels are as close to it as the plain float32 result is
+    # (measured: 0.45 of its error in the median, 1.02 at most), within a factor of two.
+    exact = gated_mlp(rms_norm(after_mixer.double(), w2.double(), 1e-5), wf["gate_up_weight"][:inter].double(), wf["gate_up_weight"][inter:].double(),
+                      wf["down_weight"].double())
+    assert float((pending.double().cpu() - exact).abs().max()) <= 2 * float((want.double() - exact).abs().max()) + 1e-7
 
 
 @pytest.mark.parametrize("nh,nkv,d,hidden,bias,window", [(4, 2, 16, 64, True, None), (6, 2, 48, 80, False, None), (3, 1, 32, 96, True, 5)])
